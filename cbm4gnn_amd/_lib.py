@@ -1,0 +1,93 @@
+"""ctypes bindings of the two C-ABI libraries declared in ``include/cbm_hip.h``.
+
+The libraries are loaded from ``cbm4gnn_amd/lib`` (built in-tree by ``cbm4gnn_amd.build``).
+There is no fallback of any kind: a missing library raises ``CbmLibraryError`` and a non-zero
+status from a call raises ``RuntimeError``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from .build import HIP_LIB, HOST_LIB
+
+CBM_OK = 0
+CBM_PROP_SCALE_ROOTS = 1
+CBM_PROP_PERSISTENT = 2
+
+
+class CbmLibraryError(RuntimeError):
+    pass
+
+
+class CbmFormat(C.Structure):
+    """Mirror of ``struct cbm_format``."""
+    _fields_ = [
+        ("n", C.c_int32), ("n_levels", C.c_int32), ("nnz", C.c_int64), ("nnz_a", C.c_int64),
+        ("n_candidates", C.c_int64), ("msa_weight", C.c_int64),
+        ("rowptr", C.POINTER(C.c_int32)), ("idx", C.POINTER(C.c_uint32)), ("parent", C.POINTER(C.c_int32)),
+        ("order", C.POINTER(C.c_int32)), ("level_off", C.POINTER(C.c_int32)),
+        ("mst_row", C.POINTER(C.c_int32)), ("mst_col", C.POINTER(C.c_int32)),
+    ]
+
+
+_P = C.c_void_p
+_I32, _I64 = C.c_int32, C.c_int64
+
+# name -> (restype, argtypes); the single list every symbol check iterates over
+HOST_SYMBOLS = {
+    "cbm_host_version": (C.c_char_p, []),
+    "cbm_build_host": (C.c_int, [_P, _P, _I64, _I32, _I32, _I32, C.POINTER(CbmFormat)]),
+    "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
+}
+HIP_SYMBOLS = {
+    "cbm_version": (C.c_char_p, []),
+    "cbm_status_string": (C.c_char_p, [C.c_int]),
+    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
+    "cbm_spmm_update_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+}
+
+_host = None
+_hip = None
+
+
+def _load(path: str, symbols: dict, what: str):
+    if not os.path.exists(path):
+        raise CbmLibraryError(
+            f"{what} library not found at {path}; build it with `python -m cbm4gnn_amd.build` "
+            "(there is no CPU fallback)")
+    try:
+        lib = C.CDLL(path)
+    except OSError as e:                                   # e.g. libamdhip64 missing
+        raise CbmLibraryError(f"cannot load {path}: {e}") from e
+    for name, (res, args) in symbols.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as e:
+            raise CbmLibraryError(f"{path} does not export {name}") from e
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def host_lib():
+    global _host
+    if _host is None:
+        _host = _load(HOST_LIB, HOST_SYMBOLS, "host builder")
+    return _host
+
+
+def hip_lib():
+    global _hip
+    if _hip is None:
+        _hip = _load(HIP_LIB, HIP_SYMBOLS, "HIP kernel")
+    return _hip
+
+
+def check(status: int, where: str):
+    if status != CBM_OK:
+        msg = hip_lib().cbm_status_string(status).decode() if _hip is not None else f"status {status}"
+        exc = ValueError if status in (1, 3) else RuntimeError
+        raise exc(f"{where}: {msg} (status {status})")

@@ -1,0 +1,441 @@
+"""``cbm_matrix`` -- the reference's Python surface (``/root/reference/cbm/cbm.py:9-275``) over
+the MI355X kernels.
+
+Same constructor, same attributes (``deltas``, ``mst_row``, ``mst_col``, ``col_multiplier``) and
+the same method names with the same in-place semantics, so the reference's message-passing
+layers (``gnns/message_passing/cbm_message_passing.py:16-107``) and tests run against it
+unchanged.  What differs is what happens behind the methods:
+
+* construction calls the host builder ``cbm_build_host`` (packed-sign delta CSR + level
+  ordering of the arborescence) instead of ``cbm_.from_coo_int32_t_v1_/_v2_``;
+* every multiply runs the two HIP kernels through the C ABI on torch's current stream.
+  The reference re-slices and re-casts the CSR arrays on every call (``cbm.py:145-148``); here
+  the device copies of the format are made once per device and cached;
+* ``seq_*`` and ``omp_*`` twins are the same GPU path (the distinction is CPU threading);
+* CPU tensors are staged through the GPU (copy in, multiply, copy out).  There is no CPU
+  implementation: without a GPU or without the built library every multiply raises.
+
+Additions that the reference lacks: ``matmul`` / ``CBMMatmul`` with a correct autograd backward
+(the reference's ``*_torch_csr_matmul`` differentiates only ``deltas @ x``, ``cbm.py:255-265``),
+``compression_ratio`` (``benchmark/utility.py:45-64``) and the packed arrays themselves.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import warnings
+from collections import deque
+
+import numpy as np
+import torch
+
+from . import _lib
+
+warnings.filterwarnings("ignore", message="Sparse CSR tensor support is in beta state", category=UserWarning)
+
+__all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels"]
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("cbm_matrix multiplies run on the GPU only and no HIP device is available "
+                           "(there is no CPU fallback)")
+
+
+def _check_f32_matrix(t, name, n=None):
+    # dtype errors mirror the TORCH_CHECKs of cbm_extensions.cpp:659-666; shape / layout checks
+    # are new (the reference has none and reads out of bounds instead)
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"{name} tensor (NOT torch::kFloat32)")
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be 2-D [N, d], got shape {tuple(t.shape)}")
+    if n is not None and t.size(0) != n:
+        raise ValueError(f"{name} has {t.size(0)} rows, the matrix has {n}")
+    if t.size(1) > 1 and t.stride(1) != 1:
+        raise ValueError(f"{name} must be row-major with unit column stride")
+    if t.size(0) > 1 and t.stride(0) < t.size(1):
+        raise ValueError(f"{name} has overlapping rows (stride {t.stride(0)} < width {t.size(1)})")
+
+
+def _ld(t):
+    return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
+
+
+def tree_levels(mst_row: np.ndarray, mst_col: np.ndarray):
+    """(parent, order, level_off) from the reference's tree CSR (``mst_row`` [N+2], ``mst_col``
+    [N], row N = virtual root).  parent is -1 for children of the root; order is sorted by
+    (level, id)."""
+    mst_row = np.asarray(mst_row, np.int64)
+    mst_col = np.asarray(mst_col, np.int64)
+    n = mst_col.shape[0]
+    if mst_row.shape[0] != n + 2:
+        raise ValueError("mst_row must have N + 2 entries")
+    counts = np.diff(mst_row)
+    parent = np.full(n, -2, np.int64)
+    parent[mst_col] = np.repeat(np.arange(n + 1), counts)
+    if (parent == -2).any():
+        raise ValueError("tree does not cover every row")
+    parent[parent == n] = -1
+    level = np.full(n, -1, np.int64)
+    frontier = mst_col[mst_row[n]:mst_row[n + 1]]
+    depth = 0
+    seen = 0
+    while frontier.size:
+        level[frontier] = depth
+        seen += frontier.size
+        cnt = counts[frontier]
+        tot = int(cnt.sum())
+        if tot == 0:
+            break
+        starts = np.repeat(mst_row[frontier], cnt)
+        offs = np.arange(tot) - np.repeat(np.cumsum(cnt) - cnt, cnt)
+        frontier = mst_col[starts + offs]
+        depth += 1
+    if seen != n:
+        raise ValueError("tree is not connected to the root")
+    order = np.lexsort((np.arange(n), level))
+    n_levels = int(level.max()) + 1 if n else 0
+    level_off = np.searchsorted(level[order], np.arange(n_levels + 1))
+    return parent.astype(np.int32), order.astype(np.int32), level_off.astype(np.int32)
+
+
+class cbm_matrix:
+
+    def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
+                 deltas_format="csr", threads=0):
+        ei = torch.as_tensor(edge_index)
+        if ei.dim() != 2 or ei.size(0) != 2:
+            raise ValueError("Edge index should have shape (2, num_edges)")
+        ei_cpu = ei.detach().to("cpu", torch.int32).contiguous()
+        if ei_cpu.size(1) == 0:
+            raise ValueError("empty edge index")
+        if int(ei_cpu.min()) < 0:
+            raise ValueError("Edge index should start from 0")
+        n = int(max(ei_cpu[0].max(), ei_cpu[1].max())) + 1          # cbm.py:15 (square matrix)
+        for given in (rows, cols):
+            if given is not None and int(given) != n:
+                raise ValueError(f"rows/cols ({given}) do not match edge_index.max() + 1 ({n})")
+        self.num_rows = n
+        self.alpha = int(alpha)
+        self.normalized = bool(normalized)
+        self.deltas_format = deltas_format if deltas_format in ("csr", "coo") else "csr"
+
+        fmt = _lib.CbmFormat()
+        rc = _lib.host_lib().cbm_build_host(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()),
+                                            ei_cpu.size(1), n, self.alpha, int(threads), C.byref(fmt))
+        try:
+            _lib.check(rc, "cbm_build_host")
+
+            def take(ptr, count, dtype):
+                return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))
+
+            self.nnz = int(fmt.nnz)
+            self.nnz_a = int(fmt.nnz_a)
+            self.n_candidates = int(fmt.n_candidates)
+            self.n_levels = int(fmt.n_levels)
+            self.rowptr = take(fmt.rowptr, n + 1, np.int32)
+            # packed column | sign << 31; kept as the int32 bit pattern (torch has no uint32 math)
+            self.idx = take(fmt.idx, self.nnz, np.uint32).view(torch.int32) if self.nnz else torch.empty(0, dtype=torch.int32)
+            self.parent = take(fmt.parent, n, np.int32)
+            self.order = take(fmt.order, n, np.int32)
+            self.level_off = take(fmt.level_off, self.n_levels + 1, np.int32)
+            self.mst_row = take(fmt.mst_row, n + 2, np.int32)
+            self.mst_col = take(fmt.mst_col, n, np.int32)
+        finally:
+            _lib.host_lib().cbm_format_free(C.byref(fmt))
+
+        if self.normalized:
+            # m[i] = (#edges with row == i) ** -0.5, cbm.py:34-41 (there a Python loop per edge)
+            deg = torch.bincount(ei_cpu[0].to(torch.int64), minlength=n).to(torch.float32)
+            self.col_multiplier = deg.pow(-0.5)
+        else:
+            self.col_multiplier = None
+
+        self._deltas = None
+        self._dev = {}
+        self._transposed = None
+        keys = ei_cpu[0].to(torch.int64) * n + ei_cpu[1].to(torch.int64)
+        keys_t = ei_cpu[1].to(torch.int64) * n + ei_cpu[0].to(torch.int64)
+        self.is_symmetric = bool(torch.equal(torch.unique(keys), torch.unique(keys_t)))
+        self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
+
+    # ------------------------------------------------------------------ format views --------
+    def columns(self):
+        """Delta column indices (int64) and signs (+1/-1, fp32), unpacked from ``idx``."""
+        col = (self.idx & 0x7FFFFFFF).to(torch.int64)
+        sign = torch.where(self.idx < 0, -1.0, 1.0).to(torch.float32)
+        return col, sign
+
+    @property
+    def deltas(self):
+        """Delta matrix as a torch sparse tensor with values +-1 (or +-m[col] when normalised),
+        what the reference keeps in ``self.deltas`` (``cbm.py:56-66``).  Built on first use."""
+        if self._deltas is None:
+            col, val = self.columns()
+            if self.col_multiplier is not None:
+                val = val * self.col_multiplier[col]
+            n = self.num_rows
+            csr = torch.sparse_csr_tensor(self.rowptr.to(torch.int64), col, val, size=(n, n))
+            self._deltas = csr if self.deltas_format == "csr" else csr.to_sparse_coo().coalesce()
+        return self._deltas
+
+    def compression_ratio(self):
+        """Element-count ratio CSR(A) / CBM, ``benchmark/utility.py:45-64``."""
+        n = self.num_rows
+        return (n + 1 + 2 * self.nnz_a) / (n + 1 + 2 * self.nnz + (n + 2) + n)
+
+    def check_format(self, edge_index):
+        """Rebuild every row from the tree and the signed deltas and compare with the adjacency
+        lists (``cbm.py:69-115``).  Raises ``ValueError`` on any mismatch."""
+        ei = torch.as_tensor(edge_index).to("cpu", torch.int64)
+        n_rows = int(ei[0].max()) + 1
+        rowptr = self.rowptr.tolist()
+        col, sign = self.columns()
+        col = col.tolist(); sign = sign.tolist()
+        mst_row = self.mst_row.tolist(); mst_col = self.mst_col.tolist()
+        s = [set() for _ in range(n_rows + 1)]
+        queue = deque([n_rows])
+        visited = 0
+        while queue:
+            u = queue.popleft()
+            for v in mst_col[mst_row[u]:mst_row[u + 1]]:
+                queue.append(v)
+                visited += 1
+                sv = set(s[u])
+                for k in range(rowptr[v], rowptr[v + 1]):
+                    if sign[k] > 0:
+                        sv.add(col[k])
+                    else:
+                        sv.remove(col[k])
+                s[v] = sv
+            if u != n_rows:
+                s[u] = frozenset(s[u])
+        if visited != n_rows:
+            raise ValueError("Format is incorrect!")
+        a = [set() for _ in range(n_rows)]
+        for r, c in zip(ei[0].tolist(), ei[1].tolist()):
+            a[r].add(c)
+        for v in range(n_rows):
+            if s[v] != a[v]:
+                raise ValueError("Format is incorrect!")
+        return True
+
+    # ------------------------------------------------------------------ device state --------
+    def _device_arrays(self, device):
+        device = torch.device(device)
+        key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+        st = self._dev.get(key)
+        if st is None:
+            st = {
+                "rowptr": self.rowptr.to(device), "idx": self.idx.to(device), "parent": self.parent.to(device),
+                "order": self.order.to(device), "level_off": self.level_off.to(device),
+                "m": self.col_multiplier.to(device) if self.col_multiplier is not None else None,
+            }
+            self._dev[key] = st
+        return st
+
+    def to(self, device):
+        """Upload the format to ``device`` now (it is otherwise uploaded at the first multiply)."""
+        _require_gpu()
+        self._device_arrays(device)
+        return self
+
+    def _stage(self, t, like=None):
+        """(device tensor, needs_copy_back).  CPU tensors are staged through the current GPU."""
+        if t.is_cuda:
+            return t, False
+        _require_gpu()
+        return t.to("cuda"), True
+
+    # ------------------------------------------------------------------ kernels -------------
+    def _run_spmm(self, x, y, use_m, scale_roots):
+        n = self.num_rows
+        _check_f32_matrix(x, "rhs", n)
+        _check_f32_matrix(y, "dst", n)
+        if x.size(1) != y.size(1):
+            raise ValueError(f"rhs has {x.size(1)} columns, dst has {y.size(1)}")
+        if use_m and self.col_multiplier is None:
+            raise RuntimeError("this cbm_matrix was built with normalized=False")
+        _require_gpu()
+        xd, _ = self._stage(x)
+        yd = y if y.is_cuda else torch.empty(y.shape, dtype=y.dtype, device=xd.device)
+        if yd.device != xd.device:
+            raise ValueError("rhs and dst are on different devices")
+        st = self._device_arrays(xd.device)
+        with torch.cuda.device(xd.device):
+            rc = _lib.hip_lib().cbm_spmm_f32(
+                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
+                _ptr(st["parent"]) if scale_roots else None, None, _ptr(xd), _ptr(yd),
+                n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
+        _lib.check(rc, "cbm_spmm_f32")
+        if yd is not y:
+            y.copy_(yd)
+
+    def _run_propagate(self, y, use_m, flags=0):
+        n = self.num_rows
+        _check_f32_matrix(y, "dst", n)
+        if use_m and self.col_multiplier is None:
+            raise RuntimeError("this cbm_matrix was built with normalized=False")
+        _require_gpu()
+        yd, back = self._stage(y)
+        st = self._device_arrays(yd.device)
+        if use_m:
+            flags |= _lib.CBM_PROP_SCALE_ROOTS
+        with torch.cuda.device(yd.device):
+            rc = _lib.hip_lib().cbm_propagate_f32(
+                _ptr(st["parent"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off),
+                self.n_levels, _ptr(st["m"]) if use_m else None, _ptr(yd), n, y.size(1), _ld(yd),
+                flags, _stream(yd.device))
+        _lib.check(rc, "cbm_propagate_f32")
+        if back:
+            y.copy_(yd)
+
+    def _run_spmm_update(self, x, y, use_m, flags=0):
+        n = self.num_rows
+        _check_f32_matrix(x, "rhs", n)
+        _check_f32_matrix(y, "dst", n)
+        if x.size(1) != y.size(1):
+            raise ValueError(f"rhs has {x.size(1)} columns, dst has {y.size(1)}")
+        if use_m and self.col_multiplier is None:
+            raise RuntimeError("this cbm_matrix was built with normalized=False")
+        _require_gpu()
+        xd, _ = self._stage(x)
+        yd = y if y.is_cuda else torch.empty(y.shape, dtype=y.dtype, device=xd.device)
+        if yd.device != xd.device:
+            raise ValueError("rhs and dst are on different devices")
+        if yd.data_ptr() == xd.data_ptr():
+            raise ValueError("dst must not alias rhs")
+        st = self._device_arrays(xd.device)
+        with torch.cuda.device(xd.device):
+            rc = _lib.hip_lib().cbm_spmm_update_f32(
+                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None, _ptr(st["parent"]),
+                None, _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
+                _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
+        _lib.check(rc, "cbm_spmm_update_f32")
+        if yd is not y:
+            y.copy_(yd)
+
+    # ------------------------------------------------------------------ reference methods ---
+    # "Sequential" methods (cbm.py:144-188)
+    def seq_mkl_csr_spmm_update(self, x, y):
+        self._run_spmm_update(x, y, use_m=False)
+
+    def seq_mkl_csr_spmm(self, x, y):
+        self._run_spmm(x, y, use_m=self.col_multiplier is not None, scale_roots=False)
+
+    def seq_mkl_csr_update(self, y):
+        self._run_propagate(y, use_m=False)
+
+    def seq_mkl_csr_fused_spmm_update(self, x, y):
+        self._run_spmm_update(x, y, use_m=True)
+
+    def seq_mkl_csr_fused_update(self, y):
+        self._run_propagate(y, use_m=True)
+
+    # "Parallel" methods (cbm.py:191-249)
+    def omp_mkl_csr_spmm_update(self, x, y):
+        self._run_spmm_update(x, y, use_m=False)
+
+    def omp_mkl_csr_spmm(self, x, y):
+        self._run_spmm(x, y, use_m=self.col_multiplier is not None, scale_roots=False)
+
+    def omp_mkl_csr_update(self, y):
+        self._run_propagate(y, use_m=False)
+
+    def omp_avx_csr_update(self, y):
+        self._run_propagate(y, use_m=False)
+
+    def omp_mkl_csr_spmm_update_v2(self, x, y):
+        # the reference wrapper (cbm.py:219-228) names a native function that its extension
+        # never exports; here it is the plain spmm + update
+        self._run_spmm_update(x, y, use_m=False)
+
+    def omp_mkl_csr_fused_spmm_update(self, x, y):
+        self._run_spmm_update(x, y, use_m=True)
+
+    def omp_mkl_csr_fused_update(self, y):
+        self._run_propagate(y, use_m=True)
+
+    # "mixed" methods (cbm.py:255-275): deltas @ x, then the update; here both on the GPU and
+    # differentiable with the full operator (not only the delta part)
+    def seq_torch_csr_matmul(self, x):
+        return CBMMatmul.apply(x, self, False)
+
+    def omp_torch_csr_matmul(self, x):
+        return CBMMatmul.apply(x, self, False)
+
+    def seq_torch_csr_fused_matmul(self, x):
+        return CBMMatmul.apply(x, self, True)
+
+    def omp_torch_csr_fused_matmul(self, x):
+        return CBMMatmul.apply(x, self, True)
+
+    # ------------------------------------------------------------------ additions -----------
+    def matmul(self, x):
+        """``A_hat @ x`` (normalised if the matrix was built so), differentiable in ``x``."""
+        return CBMMatmul.apply(x, self, self.col_multiplier is not None)
+
+    def transposed(self):
+        """CBM of the transposed matrix (the operator of the backward pass).  For a symmetric
+        edge list -- every undirected graph -- this is the object itself."""
+        if self.is_symmetric:
+            return self
+        if self._transposed is None:
+            ei = self._edge_index_cpu
+            t = cbm_matrix(torch.stack([ei[1], ei[0]]), None, alpha=self.alpha, normalized=False)
+            t.col_multiplier = self.col_multiplier      # diag(m) A^T diag(m): same vector both sides
+            t.normalized = self.normalized
+            t._transposed = self
+            self._transposed = t
+        return self._transposed
+
+
+class CBMMatmul(torch.autograd.Function):
+    """y = A_hat x with backward g -> A_hat^T g, both through the HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, x, mat, fused):
+        ctx.mat = mat
+        ctx.fused = fused
+        xd = x.detach()
+        if xd.dtype != torch.float32:
+            raise RuntimeError("rhs tensor (NOT torch::kFloat32)")
+        xd = xd.contiguous()
+        y = torch.empty_like(xd)
+        mat._run_spmm_update(xd, y, use_m=fused)
+        return y
+
+    @staticmethod
+    def backward(ctx, g):
+        g = g.contiguous()
+        gx = torch.empty_like(g)
+        ctx.mat.transposed()._run_spmm_update(g, gx, use_m=ctx.fused)
+        return gx, None, None
+
+
+def csr_spmm(rowptr, col, val, x, y):
+    """Plain CSR SpMM ``y = A @ x`` on the GPU: the hand-written baseline the CBM multiply is
+    measured against (role of ``omp_s_spmm_csr_int32``, ``cbm_extensions.cpp:1707-1755``).
+    ``rowptr`` [N+1] / ``col`` int32 device tensors, ``val`` fp32 or None (all ones)."""
+    n = rowptr.numel() - 1
+    _check_f32_matrix(x, "rhs")
+    _check_f32_matrix(y, "dst", n)
+    if rowptr.dtype != torch.int32 or col.dtype != torch.int32:
+        raise RuntimeError("lhs_col (NOT torch::kInt32)")
+    if val is not None and val.dtype != torch.float32:
+        raise RuntimeError("lhs_val (NOT torch::kFloat32)")
+    if not (x.is_cuda and y.is_cuda and rowptr.is_cuda and col.is_cuda):
+        raise ValueError("csr_spmm expects device tensors")
+    with torch.cuda.device(x.device):
+        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), None, _ptr(x), _ptr(y),
+                                         n, x.size(1), _ld(x), _ld(y), _stream(x.device))
+    _lib.check(rc, "csr_spmm_f32")

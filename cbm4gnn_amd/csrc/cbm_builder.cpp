@@ -1,0 +1,377 @@
+// Host-side construction of the CBM (compressed binary matrix) format.
+//
+// Replaces the reference builders cbm_init_v1_/_v2_ (/root/reference/cbm/cbm_extensions.cpp:8-326,
+// :328-644).  Same mathematics -- distance graph with the alpha admission rule (:75-103), a
+// minimum spanning arborescence rooted at a virtual node (the reference calls arbok::TarjanPQ,
+// :109-148), signed row deltas by a sorted merge (:186-261) -- but a different product: instead
+// of a delta COO with fp32 values and a tree CSR only, it emits the device format the HIP kernels
+// consume:
+//   rowptr[N+1]      CSR offsets of the delta matrix
+//   idx[nnz]         column | (negative ? 1u<<31 : 0), columns ascending within a row
+//   parent[N]        parent row, -1 for children of the virtual root
+//   order[N]         rows sorted by (tree level, id); level 0 = children of the root
+//   level_off[L+1]   offsets of the levels inside order[]
+// plus the reference's own tree arrays mst_row[N+2] / mst_col[N] (:274-286) so that code written
+// against the reference's cbm_matrix attributes keeps working.
+//
+// Differences in method (none in result class):
+//   * |row_i ^ row_j| is streamed row by row with a sparse accumulator and only admissible pairs
+//     are kept; the reference materialises all of A*A^T with mkl_sparse_syrk (:46-65).
+//   * the arborescence is found by an own implementation of Tarjan's O(m log n) algorithm
+//     (meldable leftist heaps with lazy keys, union-find with rollback for the expansion).
+//   * the normalisation vector is NOT folded into delta values here; kernels apply it.
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <utility>
+#include <vector>
+#include <omp.h>
+
+#include "../../include/cbm_hip.h"
+
+namespace {
+
+struct CandEdge { int32_t u, v, w; };
+
+// ---------------------------------------------------------------------------------------------
+// Minimum spanning arborescence (Tarjan 1977 / Camerini-Fratta-Maffioli 1979 expansion).
+// ---------------------------------------------------------------------------------------------
+class Arborescence {
+public:
+    Arborescence(int32_t n, const std::vector<CandEdge>& edges)
+        : n_(n), edges_(edges), key_(edges.size()), lazy_(edges.size(), 0), lc_(edges.size(), -1),
+          rc_(edges.size(), -1), rank_(edges.size(), 1), heap_(n, -1), uf_(n, -1) {}
+
+    // Returns total weight; par[v] = tail of the edge entering v (par[root] = -1).
+    int64_t run(int32_t root, std::vector<int32_t>& par) {
+        const int64_t m = (int64_t)edges_.size();
+        for (int64_t e = 0; e < m; e++) key_[e] = edges_[e].w;
+        // bulk-build one heap per head node: gather ids per node, then pairwise meld
+        {
+            std::vector<int64_t> cnt(n_ + 1, 0);
+            for (int64_t e = 0; e < m; e++) cnt[edges_[e].v + 1]++;
+            for (int32_t v = 0; v < n_; v++) cnt[v + 1] += cnt[v];
+            std::vector<int32_t> ids(m);
+            std::vector<int64_t> fill(cnt.begin(), cnt.end() - 1);
+            for (int64_t e = 0; e < m; e++) ids[fill[edges_[e].v]++] = (int32_t)e;
+            std::vector<int32_t> q;
+            for (int32_t v = 0; v < n_; v++) {
+                int64_t b = cnt[v], e = cnt[v + 1];
+                if (b == e) continue;
+                q.assign(ids.begin() + b, ids.begin() + e);
+                size_t len = q.size();
+                while (len > 1) {                      // rounds of pairwise melds: O(len) total
+                    size_t o = 0;
+                    for (size_t i = 0; i + 1 < len; i += 2) q[o++] = meld(q[i], q[i + 1]);
+                    if (len & 1) q[o++] = q[len - 1];
+                    len = o;
+                }
+                heap_[v] = q[0];
+            }
+        }
+        std::vector<int32_t> seen(n_, -1), path(n_), Q(n_), in(n_, -1);
+        seen[root] = root;
+        int64_t res = 0;
+        struct Cycle { int32_t node; int32_t time; int32_t eb, ee; };
+        std::vector<Cycle> cycles;
+        std::vector<int32_t> cyc_edges;
+        for (int32_t s = 0; s < n_; s++) {
+            int32_t u = s, qi = 0;
+            while (seen[u] < 0) {
+                int32_t h = heap_[u];
+                if (h < 0) return -1;                   // node not reachable from the root
+                push_down(h);
+                const int32_t e = h;
+                const int32_t w = key_[e];
+                heap_[u] = meld(lc_[e], rc_[e]);         // pop
+                if (heap_[u] >= 0) lazy_[heap_[u]] -= w;  // remaining keys become reduced costs
+                Q[qi] = e; path[qi++] = u; seen[u] = s;
+                res += w;
+                u = find(edges_[e].u);
+                if (seen[u] == s) {                      // closed a cycle: contract it into u
+                    int32_t cyc = -1;
+                    const int32_t end = qi, time = (int32_t)hist_.size();
+                    int32_t x;
+                    do { x = path[--qi]; cyc = meld(cyc, heap_[x]); } while (join(u, x));
+                    u = find(u);
+                    heap_[u] = cyc; seen[u] = -1;
+                    cycles.push_back({u, time, (int32_t)cyc_edges.size(), (int32_t)cyc_edges.size() + (end - qi)});
+                    for (int32_t i = qi; i < end; i++) cyc_edges.push_back(Q[i]);
+                }
+            }
+            for (int32_t i = 0; i < qi; i++) in[find(edges_[Q[i]].v)] = Q[i];
+        }
+        for (int64_t c = (int64_t)cycles.size() - 1; c >= 0; c--) {   // expand, most recent first
+            const Cycle& cy = cycles[c];
+            rollback(cy.time);
+            const int32_t in_edge = in[cy.node];
+            for (int32_t i = cy.eb; i < cy.ee; i++) in[find(edges_[cyc_edges[i]].v)] = cyc_edges[i];
+            in[find(edges_[in_edge].v)] = in_edge;
+        }
+        par.assign(n_, -1);
+        for (int32_t v = 0; v < n_; v++) if (v != root) par[v] = edges_[in[v]].u;
+        return res;
+    }
+
+private:
+    int32_t n_;
+    const std::vector<CandEdge>& edges_;
+    std::vector<int32_t> key_, lazy_, lc_, rc_;
+    std::vector<uint8_t> rank_;
+    std::vector<int32_t> heap_;
+    std::vector<int32_t> uf_;                                  // <0: -size, else parent
+    std::vector<std::pair<int32_t, int32_t>> hist_;
+
+    void push_down(int32_t a) {
+        const int32_t z = lazy_[a];
+        if (z) {
+            key_[a] += z;
+            if (lc_[a] >= 0) lazy_[lc_[a]] += z;
+            if (rc_[a] >= 0) lazy_[rc_[a]] += z;
+            lazy_[a] = 0;
+        }
+    }
+    // Leftist heap meld; the right spine is O(log size) so the recursion is shallow.  Ties are
+    // broken towards the smaller edge id, which makes the result independent of meld order.
+    int32_t meld(int32_t a, int32_t b) {
+        if (a < 0) return b;
+        if (b < 0) return a;
+        push_down(a); push_down(b);
+        if (key_[a] > key_[b] || (key_[a] == key_[b] && a > b)) std::swap(a, b);
+        rc_[a] = meld(rc_[a], b);
+        const uint8_t rl = lc_[a] >= 0 ? rank_[lc_[a]] : 0, rr = rank_[rc_[a]];
+        if (rl < rr) std::swap(lc_[a], rc_[a]);
+        rank_[a] = (uint8_t)((rc_[a] >= 0 ? rank_[rc_[a]] : 0) + 1);
+        return a;
+    }
+    int32_t find(int32_t x) const { while (uf_[x] >= 0) x = uf_[x]; return x; }
+    bool join(int32_t a, int32_t b) {
+        a = find(a); b = find(b);
+        if (a == b) return false;
+        if (uf_[a] > uf_[b]) std::swap(a, b);
+        hist_.push_back({a, uf_[a]}); hist_.push_back({b, uf_[b]});
+        uf_[a] += uf_[b]; uf_[b] = a;
+        return true;
+    }
+    void rollback(int32_t t) {
+        for (int32_t i = (int32_t)hist_.size(); i-- > t;) uf_[hist_[i].first] = hist_[i].second;
+        hist_.resize(t);
+    }
+};
+
+template <class T> T* dup_array(const std::vector<T>& v) {
+    T* p = (T*)std::malloc(sizeof(T) * (v.size() ? v.size() : 1));
+    if (!p) throw std::bad_alloc();
+    if (!v.empty()) std::memcpy(p, v.data(), sizeof(T) * v.size());
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cbm_host_version(void) { return "cbm4gnn_amd host builder 0.1"; }
+
+void cbm_format_free(cbm_format* f) {
+    if (!f) return;
+    std::free(f->rowptr); std::free(f->idx); std::free(f->parent); std::free(f->order);
+    std::free(f->level_off); std::free(f->mst_row); std::free(f->mst_col);
+    std::memset(f, 0, sizeof(*f));
+}
+
+int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t alpha,
+                   int32_t threads, cbm_format* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if ((!row || !col) && E > 0) return CBM_ERR_NULL;
+    if (N <= 0 || E < 0 || N >= (1 << 30)) return CBM_ERR_SHAPE;
+    if (threads <= 0) threads = omp_get_max_threads();
+    try {
+        // ---- COO -> CSR(A) with sorted unique columns, and its transpose -----------------------
+        std::vector<int64_t> rp(N + 1, 0);
+        for (int64_t k = 0; k < E; k++) {
+            if (row[k] < 0 || row[k] >= N || col[k] < 0 || col[k] >= N) return CBM_ERR_SHAPE;
+            rp[row[k] + 1]++;
+        }
+        for (int32_t r = 0; r < N; r++) rp[r + 1] += rp[r];
+        std::vector<int32_t> ci(E);
+        {
+            std::vector<int64_t> fill(rp.begin(), rp.end() - 1);
+            for (int64_t k = 0; k < E; k++) ci[fill[row[k]]++] = col[k];
+        }
+        std::vector<int32_t> nnz(N);
+#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
+        for (int32_t r = 0; r < N; r++) {
+            auto b = ci.begin() + rp[r], e = ci.begin() + rp[r + 1];
+            std::sort(b, e);
+            nnz[r] = (int32_t)(std::unique(b, e) - b);
+        }
+        {   // compact duplicates away
+            int64_t w = 0;
+            for (int32_t r = 0; r < N; r++) {
+                const int64_t b = rp[r];
+                rp[r] = w;
+                if (w != b) std::memmove(&ci[w], &ci[b], sizeof(int32_t) * (size_t)nnz[r]);
+                w += nnz[r];
+            }
+            rp[N] = w;
+            ci.resize(w);
+        }
+        const int64_t nnzA = rp[N];
+        std::vector<int64_t> tp(N + 1, 0);
+        for (int64_t k = 0; k < nnzA; k++) tp[ci[k] + 1]++;
+        for (int32_t c = 0; c < N; c++) tp[c + 1] += tp[c];
+        std::vector<int32_t> tr(nnzA);
+        {
+            std::vector<int64_t> fill(tp.begin(), tp.end() - 1);
+            for (int32_t r = 0; r < N; r++)
+                for (int64_t k = rp[r]; k < rp[r + 1]; k++) tr[fill[ci[k]]++] = r;   // ascending r per column
+        }
+
+        // ---- candidate edges (reference rule, cpp:75-103), streamed and pruned ------------------
+        // pair (i, j>i) with s shared columns: h = nnz_i + nnz_j - 2s;
+        //   j -> i admitted iff h < nnz_i - alpha  <=>  2s > nnz_j + alpha
+        //   i -> j admitted iff h < nnz_j - alpha  <=>  2s > nnz_i + alpha
+        const int32_t CH = 64;
+        const int32_t n_chunks = (N + CH - 1) / CH;
+        std::vector<std::vector<CandEdge>> chunk_out(n_chunks);
+#pragma omp parallel num_threads(threads)
+        {
+            std::vector<int32_t> cnt(N, 0), touched;
+            std::vector<std::pair<int32_t, int32_t>> adm;
+            touched.reserve(1024);
+#pragma omp for schedule(dynamic, 1)
+            for (int32_t ch = 0; ch < n_chunks; ch++) {
+                std::vector<CandEdge>& o = chunk_out[ch];
+                const int32_t i_end = std::min(N, (ch + 1) * CH);
+                for (int32_t i = ch * CH; i < i_end; i++) {
+                    const int32_t ni = nnz[i];
+                    o.push_back({N, i, ni});
+                    touched.clear();
+                    for (int64_t k = rp[i]; k < rp[i + 1]; k++) {
+                        const int32_t c = ci[k];
+                        const int32_t* lo = tr.data() + tp[c];
+                        const int32_t* hi = tr.data() + tp[c + 1];
+                        for (const int32_t* q = std::upper_bound(lo, hi, i); q < hi; ++q) {
+                            const int32_t j = *q;
+                            if (cnt[j]++ == 0) touched.push_back(j);
+                        }
+                    }
+                    adm.clear();
+                    for (int32_t j : touched) {
+                        const int32_t s = cnt[j];
+                        cnt[j] = 0;
+                        if (2 * s > std::min(ni, nnz[j]) + alpha) adm.push_back({j, s});
+                    }
+                    std::sort(adm.begin(), adm.end());
+                    for (auto& js : adm) {
+                        const int32_t j = js.first, nj = nnz[j];
+                        const int32_t h = ni + nj - 2 * js.second;
+                        if (h < ni - alpha) o.push_back({j, i, h});
+                        if (h < nj - alpha) o.push_back({i, j, h});
+                    }
+                }
+            }
+        }
+        std::vector<CandEdge> cand;
+        {
+            size_t tot = 0;
+            for (auto& o : chunk_out) tot += o.size();
+            cand.reserve(tot);
+            for (auto& o : chunk_out) { cand.insert(cand.end(), o.begin(), o.end()); std::vector<CandEdge>().swap(o); }
+        }
+        if (cand.size() >= (size_t)INT32_MAX) return CBM_ERR_SHAPE;
+
+        // ---- arborescence ----------------------------------------------------------------------
+        std::vector<int32_t> par;
+        int64_t weight;
+        {
+            Arborescence msa(N + 1, cand);
+            weight = msa.run(N, par);
+        }
+        if (weight < 0) return CBM_ERR_INTERNAL;
+        const int64_t n_cand = (int64_t)cand.size();
+        std::vector<CandEdge>().swap(cand);
+
+        // ---- tree arrays: children ascending per parent; levels by BFS --------------------------
+        std::vector<int32_t> mst_row(N + 2, 0), mst_col(N);
+        for (int32_t v = 0; v < N; v++) mst_row[par[v] + 1]++;
+        for (int32_t u = 0; u <= N; u++) mst_row[u + 1] += mst_row[u];
+        {
+            std::vector<int32_t> fill(mst_row.begin(), mst_row.end() - 1);
+            for (int32_t v = 0; v < N; v++) mst_col[fill[par[v]]++] = v;
+        }
+        std::vector<int32_t> level(N, -1), order(N), level_off;
+        {
+            int32_t head = 0, tail = 0;
+            for (int32_t q = mst_row[N]; q < mst_row[N + 1]; q++) { level[mst_col[q]] = 0; order[tail++] = mst_col[q]; }
+            level_off.push_back(0);
+            int32_t cur = 0;
+            while (head < tail) {
+                const int32_t u = order[head];
+                if (level[u] != cur) { level_off.push_back(head); cur = level[u]; }
+                head++;
+                for (int32_t q = mst_row[u]; q < mst_row[u + 1]; q++) { level[mst_col[q]] = level[u] + 1; order[tail++] = mst_col[q]; }
+            }
+            if (tail != N) return CBM_ERR_INTERNAL;
+            level_off.push_back(N);
+            // BFS yields (level, parent-visit) order; the format wants (level, id)
+            for (size_t l = 0; l + 1 < level_off.size(); l++)
+                std::sort(order.begin() + level_off[l], order.begin() + level_off[l + 1]);
+        }
+
+        // ---- signed deltas, packed --------------------------------------------------------------
+        std::vector<int32_t> drp(N + 1, 0);
+#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
+        for (int32_t v = 0; v < N; v++) {
+            const int32_t u = par[v];
+            int32_t c = 0;
+            if (u == N) c = nnz[v];
+            else {
+                int64_t a = rp[u], ae = rp[u + 1], b = rp[v], be = rp[v + 1];
+                while (a < ae && b < be) {
+                    if (ci[a] == ci[b]) { a++; b++; }
+                    else if (ci[a] > ci[b]) { c++; b++; }
+                    else { c++; a++; }
+                }
+                c += (int32_t)((ae - a) + (be - b));
+            }
+            drp[v + 1] = c;
+        }
+        int64_t run = 0;
+        for (int32_t v = 0; v < N; v++) { run += drp[v + 1]; if (run > INT32_MAX) return CBM_ERR_SHAPE; drp[v + 1] = (int32_t)run; }
+        if (run != weight) return CBM_ERR_INTERNAL;      // nnz(delta) must equal the arborescence weight
+        std::vector<uint32_t> idx(run);
+#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
+        for (int32_t v = 0; v < N; v++) {
+            const int32_t u = par[v];
+            uint32_t* o = idx.data() + drp[v];
+            int64_t b = rp[v], be = rp[v + 1];
+            if (u == N) { for (; b < be; b++) *o++ = (uint32_t)ci[b]; continue; }
+            int64_t a = rp[u], ae = rp[u + 1];
+            while (a < ae && b < be) {
+                if (ci[a] == ci[b]) { a++; b++; }
+                else if (ci[a] > ci[b]) *o++ = (uint32_t)ci[b++];
+                else *o++ = (uint32_t)ci[a++] | 0x80000000u;
+            }
+            for (; a < ae; a++) *o++ = (uint32_t)ci[a] | 0x80000000u;
+            for (; b < be; b++) *o++ = (uint32_t)ci[b];
+        }
+        std::vector<int32_t> parent(N);
+        for (int32_t v = 0; v < N; v++) parent[v] = par[v] == N ? -1 : par[v];
+
+        out->n = N; out->nnz = run; out->n_levels = (int32_t)level_off.size() - 1;
+        out->n_candidates = n_cand; out->msa_weight = weight; out->nnz_a = nnzA;
+        out->rowptr = dup_array(drp); out->idx = dup_array(idx); out->parent = dup_array(parent);
+        out->order = dup_array(order); out->level_off = dup_array(level_off);
+        out->mst_row = dup_array(mst_row); out->mst_col = dup_array(mst_col);
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        cbm_format_free(out);
+        return CBM_ERR_ALLOC;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,434 @@
+// HIP kernels (gfx950 / CDNA4) and C-ABI launchers of the CBM multiply.
+//
+// Two bandwidth-bound kernels, no MFMA:
+//   (1) delta SpMM      Z = D * diag(m) * X      one 64-lane wavefront per row, lanes span the
+//                       feature columns (float4 / float2 / float per lane so that one load
+//                       instruction fetches a whole contiguous row of X); the row's packed
+//                       indices are fetched 64 at a time with one coalesced load and broadcast
+//                       lane by lane through v_readlane into scalar registers, so every X-row
+//                       load has a scalar base address.
+//   (2) tree propagate  Y[v] (+)= Y[parent(v)]   level-synchronous over a host-computed
+//                       (level, id) ordering: one launch per wide level, one single-workgroup
+//                       launch per run of narrow levels.
+// The same SpMM template without the sign bit is the plain CSR baseline.
+//
+// What each launcher replaces in the reference is stated in include/cbm_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cbm_hip.h"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;          // SpMM / wide-level propagate: 256 threads
+constexpr int kNarrowWaves = 16;           // narrow-level propagate: one 1024-thread workgroup
+constexpr int kNarrowWidth = 64;           // a level with at most this many rows is "narrow"
+constexpr int kXcds = 8;                   // MI355X: 8 XCDs, workgroups are dealt round-robin
+
+// Workgroup ids are dealt to the 8 XCDs round-robin; give every XCD a contiguous range of
+// logical blocks so that neighbouring rows (which share columns in clustered graphs) meet in
+// the same L2.
+__device__ __forceinline__ int xcd_contiguous_block(int bid, int nb) {
+    const int q = nb / kXcds, r = nb % kXcds;
+    const int x = bid % kXcds;
+    return x * q + (x < r ? x : r) + bid / kXcds;
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_vec(const float* __restrict__ p, float (&v)[VEC]) {
+    if constexpr (VEC == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (VEC == 2) {
+        const float2 t = *reinterpret_cast<const float2*>(p);
+        v[0] = t.x; v[1] = t.y;
+    } else {
+        v[0] = *p;
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_vec(float* __restrict__ p, const float (&v)[VEC]) {
+    if constexpr (VEC == 4) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else if constexpr (VEC == 2) {
+        *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
+    } else {
+        *p = v[0];
+    }
+}
+
+__device__ __forceinline__ int bcast_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ float bcast_f(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// ---------------------------------------------------------------------------------------------
+// (1) SpMM, one wavefront per row.
+//   PACKED: idx = col | sign<<31, coefficient = +-1 or +-m[col]
+//   !PACKED: idx = col (int32), coefficient = val[k] or 1
+//   VEC floats per lane per chunk, CH chunks of 64*VEC columns per wave; grid.y tiles wider d.
+//   FULL: d is an exact multiple of the tile, no column guards.
+// ---------------------------------------------------------------------------------------------
+template <int VEC, int CH, bool PACKED, bool FULL>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
+    const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
+    const float* __restrict__ m, const int32_t* __restrict__ parent, const int32_t* __restrict__ perm,
+    const float* __restrict__ X, float* __restrict__ Z, int n, int d, int64_t ldx, int64_t ldz) {
+    constexpr int U = (CH == 1) ? 8 : (CH == 2 ? 4 : 2);      // X-row loads in flight per wave
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    int row = xcd_contiguous_block(blockIdx.x, gridDim.x) * kWavesPerBlock + wave;
+    if (row >= n) return;
+    if (perm) row = perm[row];
+    row = __builtin_amdgcn_readfirstlane(row);
+    const int start = __builtin_amdgcn_readfirstlane(rowptr[row]);
+    const int end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
+    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
+
+    float acc[CH][VEC];
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[c][v] = 0.0f;
+
+    for (int base = start; base < end; base += kWave) {
+        const int cnt = min(kWave, end - base);
+        int my_col = 0;
+        float my_cf = 0.0f;
+        if (lane < cnt) {
+            if constexpr (PACKED) {
+                const uint32_t p = idx[base + lane];
+                my_col = (int)(p & 0x7fffffffu);
+                const float mag = m ? m[my_col] : 1.0f;
+                my_cf = (p >> 31) ? -mag : mag;
+            } else {
+                my_col = (int)idx[base + lane];
+                my_cf = val ? val[base + lane] : 1.0f;
+            }
+        }
+        int k = 0;
+        for (; k + U <= cnt; k += U) {
+            float x[U][CH][VEC];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float* __restrict__ xr = X + (int64_t)bcast_i(my_col, k + u) * ldx + col0;
+#pragma unroll
+                for (int c = 0; c < CH; c++) {
+                    if (FULL || col0 + c * kWave * VEC < d) load_vec<VEC>(xr + c * kWave * VEC, x[u][c]);
+                    else
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) x[u][c][v] = 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float f = bcast_f(my_cf, k + u);
+#pragma unroll
+                for (int c = 0; c < CH; c++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[c][v] = fmaf(f, x[u][c][v], acc[c][v]);
+            }
+        }
+        for (; k < cnt; k++) {
+            const float* __restrict__ xr = X + (int64_t)bcast_i(my_col, k) * ldx + col0;
+            const float f = bcast_f(my_cf, k);
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                if (FULL || col0 + c * kWave * VEC < d) {
+                    float x[VEC];
+                    load_vec<VEC>(xr + c * kWave * VEC, x);
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[c][v] = fmaf(f, x[v], acc[c][v]);
+                }
+            }
+        }
+    }
+    if constexpr (PACKED) {
+        if (m && parent && parent[row] < 0) {      // child of the root: left scaling, final value
+            const float s = m[row];
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[c][v] *= s;
+        }
+    }
+    float* __restrict__ zr = Z + (int64_t)row * ldz + col0;
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+        if (FULL || col0 + c * kWave * VEC < d) store_vec<VEC>(zr + c * kWave * VEC, acc[c]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// (2) propagate: one row v = order[i], parent u.  dv = d - d % 8 separates the reference's
+// FMA vector body from its scalar tail (cbm_extensions.cpp:966-990).
+// ---------------------------------------------------------------------------------------------
+template <int VEC, int CH, bool NORM, bool FULL>
+__device__ __forceinline__ void propagate_row(int v, int u, const float* __restrict__ m, float* __restrict__ Y,
+                                              int d, int dv, int64_t ldy, int col0) {
+    float mu = 1.0f, mv = 1.0f, inv_mu = 1.0f;
+    if constexpr (NORM) { mu = m[u]; mv = m[v]; inv_mu = 1.0f / mu; }
+    const float* __restrict__ yu = Y + (int64_t)u * ldy + col0;
+    float* __restrict__ yv = Y + (int64_t)v * ldy + col0;
+    float a[CH][VEC], b[CH][VEC];
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+        if (FULL || col0 + c * kWave * VEC < d) {
+            load_vec<VEC>(yu + c * kWave * VEC, a[c]);
+            load_vec<VEC>(yv + c * kWave * VEC, b[c]);
+        }
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+        if (FULL || col0 + c * kWave * VEC < d) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                if constexpr (NORM) {
+                    const int j = col0 + c * kWave * VEC + e;
+                    b[c][e] = (j < dv) ? fmaf(a[c][e], inv_mu, b[c][e]) * mv : (b[c][e] + a[c][e] / mu) * mv;
+                } else {
+                    b[c][e] += a[c][e];
+                }
+            }
+            store_vec<VEC>(yv + c * kWave * VEC, b[c]);
+        }
+}
+
+template <int VEC, int CH, bool NORM, bool FULL>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void propagate_level(
+    const int32_t* __restrict__ parent, const int32_t* __restrict__ order, int beg, int end,
+    const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int i = beg + blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (i >= end) return;
+    const int v = __builtin_amdgcn_readfirstlane(order[i]);
+    const int u = __builtin_amdgcn_readfirstlane(parent[v]);
+    propagate_row<VEC, CH, NORM, FULL>(v, u, m, Y, d, dv, ldy, blockIdx.y * (kWave * VEC * CH) + lane * VEC);
+}
+
+// A run of narrow levels [l_beg, l_end) handled by ONE workgroup: its 16 waves share each level's
+// rows and meet at a barrier between levels.  Column tiles (grid.y) are independent of each
+// other, so every tile is its own single workgroup.
+template <int VEC, int CH, bool NORM, bool FULL>
+__global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_narrow_levels(
+    const int32_t* __restrict__ parent, const int32_t* __restrict__ order,
+    const int32_t* __restrict__ level_off, int l_beg, int l_end, const float* __restrict__ m,
+    float* __restrict__ Y, int d, int dv, int64_t ldy) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
+    for (int l = l_beg; l < l_end; l++) {
+        const int beg = level_off[l], end = level_off[l + 1];
+        for (int i = beg + wave; i < end; i += kNarrowWaves) {
+            const int v = __builtin_amdgcn_readfirstlane(order[i]);
+            const int u = __builtin_amdgcn_readfirstlane(parent[v]);
+            propagate_row<VEC, CH, NORM, FULL>(v, u, m, Y, d, dv, ldy, col0);
+        }
+        __threadfence();
+        __syncthreads();
+    }
+}
+
+// Y[r,:] *= m[r] for the rows of level 0 (children of the root), cbm_extensions.cpp:910-940.
+template <int VEC, int CH, bool FULL>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void scale_level0(
+    const int32_t* __restrict__ order, int end, const float* __restrict__ m, float* __restrict__ Y, int d,
+    int64_t ldy) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int i = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (i >= end) return;
+    const int r = __builtin_amdgcn_readfirstlane(order[i]);
+    const float s = m[r];
+    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
+    float* __restrict__ y = Y + (int64_t)r * ldy + col0;
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+        if (FULL || col0 + c * kWave * VEC < d) {
+            float t[VEC];
+            load_vec<VEC>(y + c * kWave * VEC, t);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) t[e] *= s;
+            store_vec<VEC>(y + c * kWave * VEC, t);
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side: shape selection and dispatch
+// ---------------------------------------------------------------------------------------------
+struct Tiling { int vec, ch, grid_y; bool full; };
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Largest vector width the alignment allows that still keeps 64 lanes busy; then as many
+// 64-lane chunks per wave (1, 2 or 4) as d needs; anything wider is tiled over grid.y.
+inline Tiling pick_tiling(int d, int64_t ld_a, int64_t ld_b, const void* pa, const void* pb) {
+    int vmax = 1;
+    if (d % 4 == 0 && ld_a % 4 == 0 && ld_b % 4 == 0 && aligned(pa, 16) && aligned(pb, 16)) vmax = 4;
+    else if (d % 2 == 0 && ld_a % 2 == 0 && ld_b % 2 == 0 && aligned(pa, 8) && aligned(pb, 8)) vmax = 2;
+    int vec = vmax;
+    while (vec > 1 && d / vec < kWave) vec /= 2;
+    const int units = (d + vec - 1) / vec;
+    const int ch = units <= kWave ? 1 : (units <= 2 * kWave ? 2 : 4);
+    const int tile = kWave * vec * ch;
+    Tiling t;
+    t.vec = vec; t.ch = ch; t.grid_y = (d + tile - 1) / tile; t.full = (d == t.grid_y * tile);
+    return t;
+}
+
+#define CBM_DISPATCH_TILING(T, LAUNCH)                                              \
+    do {                                                                            \
+        if ((T).full) { CBM_DISPATCH_VC(T, true, LAUNCH); }                         \
+        else { CBM_DISPATCH_VC(T, false, LAUNCH); }                                 \
+    } while (0)
+#define CBM_DISPATCH_VC(T, FULLV, LAUNCH)                                           \
+    do {                                                                            \
+        switch ((T).vec * 10 + (T).ch) {                                            \
+            case 11: LAUNCH(1, 1, FULLV); break;                                    \
+            case 12: LAUNCH(1, 2, FULLV); break;                                    \
+            case 14: LAUNCH(1, 4, FULLV); break;                                    \
+            case 21: LAUNCH(2, 1, FULLV); break;                                    \
+            case 22: LAUNCH(2, 2, FULLV); break;                                    \
+            case 24: LAUNCH(2, 4, FULLV); break;                                    \
+            case 41: LAUNCH(4, 1, FULLV); break;                                    \
+            case 42: LAUNCH(4, 2, FULLV); break;                                    \
+            default: LAUNCH(4, 4, FULLV); break;                                    \
+        }                                                                           \
+    } while (0)
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? CBM_OK : CBM_ERR_LAUNCH; }
+
+inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
+    if (n < 0 || d < 0 || ld < d) return CBM_ERR_SHAPE;
+    return CBM_OK;
+}
+
+template <bool PACKED>
+int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, const float* m,
+                const int32_t* parent, const int32_t* perm, const float* X, float* Z, int32_t n, int32_t d,
+                int64_t ldx, int64_t ldz, hipStream_t s) {
+    if (!rowptr || !X || !Z) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (int rc = check_matrix(n, d, ldz)) return rc;
+    if (n == 0 || d == 0) return CBM_OK;
+    const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
+    const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
+#define LAUNCH(V, C, F)                                                                              \
+    hipLaunchKernelGGL((spmm_wave_per_row<V, C, PACKED, F>), grid, block, 0, s, rowptr, idx, val, m, \
+                       parent, perm, X, Z, n, d, ldx, ldz)
+    CBM_DISPATCH_TILING(t, LAUNCH);
+#undef LAUNCH
+    return check_launch();
+}
+
+template <bool NORM>
+int launch_propagate(const int32_t* parent, const int32_t* order, const int32_t* level_off_dev,
+                     const int32_t* lo, int32_t n_levels, const float* m, float* Y, int32_t n, int32_t d,
+                     int64_t ldy, int32_t flags, hipStream_t s) {
+    const Tiling t = pick_tiling(d, ldy, ldy, Y, Y);
+    const int dv = d - d % 8;
+    const dim3 block(kWave * kWavesPerBlock);
+    if (NORM && (flags & CBM_PROP_SCALE_ROOTS) && lo[1] > lo[0]) {
+        const dim3 grid((lo[1] + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y);
+#define LAUNCH(V, C, F) \
+    hipLaunchKernelGGL((scale_level0<V, C, F>), grid, block, 0, s, order, lo[1], m, Y, d, ldy)
+        CBM_DISPATCH_TILING(t, LAUNCH);
+#undef LAUNCH
+    }
+    int l = 1;
+    while (l < n_levels) {
+        const int width = lo[l + 1] - lo[l];
+        if (width <= kNarrowWidth) {
+            int l_end = l + 1;
+            while (l_end < n_levels && lo[l_end + 1] - lo[l_end] <= kNarrowWidth) l_end++;
+            if (l_end - l >= 2) {
+                const dim3 grid(1, t.grid_y), nblock(kWave * kNarrowWaves);
+#define LAUNCH(V, C, F)                                                                                 \
+    hipLaunchKernelGGL((propagate_narrow_levels<V, C, NORM, F>), grid, nblock, 0, s, parent, order,     \
+                       level_off_dev, l, l_end, m, Y, d, dv, ldy)
+                CBM_DISPATCH_TILING(t, LAUNCH);
+#undef LAUNCH
+                l = l_end;
+                continue;
+            }
+        }
+        const dim3 grid((width + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y);
+#define LAUNCH(V, C, F)                                                                                 \
+    hipLaunchKernelGGL((propagate_level<V, C, NORM, F>), grid, block, 0, s, parent, order, lo[l],       \
+                       lo[l + 1], m, Y, d, dv, ldy)
+        CBM_DISPATCH_TILING(t, LAUNCH);
+#undef LAUNCH
+        l++;
+    }
+    return check_launch();
+}
+
+int validate_levels(const int32_t* lo, int32_t n_levels, int32_t n) {
+    if (n_levels < 0) return CBM_ERR_SHAPE;
+    if (n_levels == 0) return n == 0 ? CBM_OK : CBM_ERR_SHAPE;
+    if (lo[0] != 0 || lo[n_levels] != n) return CBM_ERR_SHAPE;
+    for (int l = 0; l < n_levels; l++)
+        if (lo[l + 1] < lo[l]) return CBM_ERR_SHAPE;
+    return CBM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cbm_version(void) { return "cbm4gnn_amd hip 0.1 (gfx950)"; }
+
+const char* cbm_status_string(int status) {
+    switch (status) {
+        case CBM_OK: return "ok";
+        case CBM_ERR_NULL: return "a required pointer is NULL";
+        case CBM_ERR_ALLOC: return "allocation failed";
+        case CBM_ERR_SHAPE: return "size, stride or index out of range";
+        case CBM_ERR_LAUNCH: return "HIP launch failed";
+        case CBM_ERR_INTERNAL: return "internal invariant failed";
+        case CBM_ERR_UNSUPPORTED: return "not implemented in this build";
+        default: return "unknown status";
+    }
+}
+
+int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const int32_t* parent,
+                 const int32_t* row_perm, const float* X, float* Z, int32_t n, int32_t d, int64_t ldx,
+                 int64_t ldz, void* stream) {
+    if (!idx && n > 0) return CBM_ERR_NULL;
+    return launch_spmm<true>(rowptr, idx, nullptr, m, parent, row_perm, X, Z, n, d, ldx, ldz,
+                             static_cast<hipStream_t>(stream));
+}
+
+int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_perm,
+                 const float* X, float* Y, int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream) {
+    if (!col && n > 0) return CBM_ERR_NULL;
+    return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_perm,
+                              X, Y, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
+}
+
+int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t* level_off_dev,
+                      const int32_t* level_off_host, int32_t n_levels, const float* m, float* Y, int32_t n,
+                      int32_t d, int64_t ldy, int32_t flags, void* stream) {
+    if (!parent || !order || !level_off_dev || !level_off_host || !Y) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldy)) return rc;
+    if (int rc = validate_levels(level_off_host, n_levels, n)) return rc;
+    if (flags & CBM_PROP_PERSISTENT) return CBM_ERR_UNSUPPORTED;
+    if (n == 0 || d == 0) return CBM_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return m ? launch_propagate<true>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s)
+             : launch_propagate<false>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s);
+}
+
+int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const int32_t* parent,
+                        const int32_t* row_perm, const int32_t* order, const int32_t* level_off_dev,
+                        const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, int32_t n,
+                        int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
+    if (!parent) return CBM_ERR_NULL;
+    if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
+    int rc = cbm_spmm_f32(rowptr, idx, m, parent, row_perm, X, Y, n, d, ldx, ldy, stream);
+    if (rc) return rc;
+    // children of the root were scaled by the SpMM epilogue already
+    return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,
+                             flags & ~CBM_PROP_SCALE_ROOTS, stream);
+}
+
+}  // extern "C"

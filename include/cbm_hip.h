@@ -1,0 +1,134 @@
+/*
+ * C ABI of the MI355X (gfx950) compressed-binary-matrix (CBM) multiply.
+ *
+ * Two shared libraries implement it:
+ *   libcbm_host.so  -- host-only (g++/OpenMP): format construction.           [cbm_build_host ...]
+ *   libcbm_hip.so   -- HIP kernels for gfx950 and their launchers.            [cbm_spmm_f32 ...]
+ *
+ * Conventions
+ *   * plain pointers and sizes only; every `const T* dev` / `T* dev` argument of the device
+ *     library is a DEVICE pointer owned by the caller; the library never allocates, frees or
+ *     retains caller memory and never synchronises: work is enqueued on `stream`
+ *     (a hipStream_t passed as void*, NULL = the default stream) and the call returns.
+ *   * every function returns CBM_OK (0) or a CBM_ERR_* code; nothing calls exit() (the
+ *     reference's helpers.hpp:58-84 does on MKL failure).
+ *   * matrices X, Y, Z are row-major fp32 with a row stride `ld*` given in ELEMENTS (>= d).
+ *   * index arrays are int32, as in the reference (it is built LP64: cbm/setup.py:14-16).
+ *
+ * Each entry point names the function of /root/reference/cbm/cbm_extensions.cpp it replaces.
+ */
+#ifndef CBM_HIP_H
+#define CBM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    CBM_OK = 0,
+    CBM_ERR_NULL = 1,        /* a required pointer is NULL                         */
+    CBM_ERR_ALLOC = 2,       /* host allocation failed (builder only)              */
+    CBM_ERR_SHAPE = 3,       /* size / stride / index out of the supported range   */
+    CBM_ERR_LAUNCH = 4,      /* the HIP runtime rejected a launch                  */
+    CBM_ERR_INTERNAL = 5,    /* an internal invariant failed                       */
+    CBM_ERR_UNSUPPORTED = 6  /* valid request this build does not implement        */
+};
+
+/* flags of cbm_propagate_f32 / cbm_spmm_update_f32 */
+enum {
+    CBM_PROP_SCALE_ROOTS = 1, /* normalised only: first do Y[r,:] *= m[r] for children of the root */
+    CBM_PROP_PERSISTENT = 2   /* one persistent kernel walking the levels instead of per-level launches */
+};
+
+/* The CBM format as built on the host.  All arrays are malloc'd by cbm_build_host and are
+ * released together by cbm_format_free.
+ *   rowptr/idx   delta matrix in CSR form; idx = column | (negative entry ? 1u<<31 : 0),
+ *                columns ascending within a row (what the reference stores as a torch sparse
+ *                CSR with values +-1, cbm/cbm.py:56-58)
+ *   parent       parent row in the arborescence, -1 for children of the virtual root
+ *   order        rows sorted by (level, id); level 0 = children of the virtual root
+ *   level_off    n_levels + 1 offsets into order[]
+ *   mst_row/col  the reference's tree CSR (cbm_extensions.cpp:274-286): N+2 offsets, row N is
+ *                the virtual root; N children, ascending id within a parent */
+typedef struct cbm_format {
+    int32_t n;
+    int32_t n_levels;
+    int64_t nnz;            /* delta non-zeros = weight of the arborescence */
+    int64_t nnz_a;          /* non-zeros of the input matrix after de-duplication */
+    int64_t n_candidates;   /* edges of the distance graph, root edges included */
+    int64_t msa_weight;
+    int32_t* rowptr;        /* [n + 1]        */
+    uint32_t* idx;          /* [nnz]          */
+    int32_t* parent;        /* [n]            */
+    int32_t* order;         /* [n]            */
+    int32_t* level_off;     /* [n_levels + 1] */
+    int32_t* mst_row;       /* [n + 2]        */
+    int32_t* mst_col;       /* [n]            */
+} cbm_format;
+
+/* ------------------------------------------------------------------ libcbm_host.so ---------- */
+
+const char* cbm_host_version(void);
+
+/* Build the format from a COO list (row[k], col[k]) of a 0/1 N x N matrix; duplicates are merged,
+ * any order.  alpha is the reference's pruning parameter: row u may serve as parent of row v only
+ * if hamming(u, v) < nnz(v) - alpha.  threads <= 0 means all OpenMP threads.  HOST pointers.
+ * Replaces cbm_init_v1_ (cbm_extensions.cpp:8-326) and cbm_init_v2_ (:328-644); the
+ * normalisation vector of v2 is not an input: the kernels apply it. */
+int cbm_build_host(const int32_t* row, const int32_t* col, int64_t n_edges, int32_t n, int32_t alpha,
+                   int32_t threads, cbm_format* out);
+
+void cbm_format_free(cbm_format* f);
+
+/* ------------------------------------------------------------------ libcbm_hip.so ----------- */
+
+const char* cbm_version(void);
+const char* cbm_status_string(int status);
+
+/* Z = D * diag(m) * X for the packed delta matrix D (m == NULL: Z = D * X).  If `parent` and `m`
+ * are both given, rows with parent[r] < 0 are additionally scaled by m[r] (the first step of
+ * the normalised tree walk, cbm_extensions.cpp:910-940, folded into the producer).  row_perm, if
+ * not NULL, is a permutation of 0..N-1 giving the order in which rows are scheduled.
+ * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
+ * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
+int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
+                 const int32_t* parent_dev, const int32_t* row_perm_dev, const float* X_dev, float* Z_dev,
+                 int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
+
+/* In-place tree propagation over Y (which holds Z on entry), level by level.
+ *   m == NULL : Y[v,:] += Y[parent[v],:]
+ *               replaces seq_/omp_s_update_csr_int32_ and omp_s_update_avx_int32_
+ *               (cbm_extensions.cpp:742-786, :1485-1610, :1612-1705) and the walk inside
+ *               seq_/omp_s_spmm_update_csr_int32_ (:713-738, :1166-1218)
+ *   m != NULL : Y[v,:] = fma(Y[u,:], 1/m[u], Y[v,:]) * m[v], u = parent[v]; the last d mod 8
+ *               columns use (Y[v] + Y[u]/m[u]) * m[v] exactly as the reference's scalar tail;
+ *               with CBM_PROP_SCALE_ROOTS, children of the root are first scaled by m[r].
+ *               replaces seq_/omp_s_fused_update_csr_int32_ (:998-1105, :1376-1483) and the walk
+ *               inside seq_/omp_s_fused_spmm_update_csr_int32_ (:908-995, :1285-1373)
+ * level_off_host is a HOST array (launch shapes are derived from it); level_off_dev is the same
+ * array in device memory (read by kernels that walk several levels in one launch). */
+int cbm_propagate_f32(const int32_t* parent_dev, const int32_t* order_dev, const int32_t* level_off_dev,
+                      const int32_t* level_off_host, int32_t n_levels, const float* m_dev, float* Y_dev,
+                      int32_t n, int32_t d, int64_t ldy, int32_t flags, void* stream);
+
+/* Y = A_hat * X in one call: cbm_spmm_f32 followed by cbm_propagate_f32 on the same stream.
+ * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);
+ * m != NULL replaces seq_/omp_s_fused_spmm_update_csr_int32_ (:845-996, :1224-1374). */
+int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
+                        const int32_t* parent_dev, const int32_t* row_perm_dev, const int32_t* order_dev,
+                        const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
+                        const float* X_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
+                        int32_t flags, void* stream);
+
+/* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
+ * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
+int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, const float* val_dev,
+                 const int32_t* row_perm_dev, const float* X_dev, float* Y_dev, int32_t n, int32_t d,
+                 int64_t ldx, int64_t ldy, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CBM_HIP_H */

@@ -1,0 +1,67 @@
+"""The C-ABI libraries load without a GPU and export every function include/cbm_hip.h declares;
+the Python struct mirror matches; the reference-extension shim exports the reference's names."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from cbm4gnn_amd import _lib, build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "cbm_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(\w+)\s*\([^;{]*\)\s*;", text)))
+
+
+def test_header_declares_what_python_binds():
+    declared = _declared_functions()
+    assert set(declared) == set(_lib.HOST_SYMBOLS) | set(_lib.HIP_SYMBOLS)
+
+
+def test_libraries_export_every_declared_symbol():
+    host = C.CDLL(build.HOST_LIB)
+    hip = C.CDLL(build.HIP_LIB)
+    for name in _declared_functions():
+        lib = host if name in _lib.HOST_SYMBOLS else hip
+        assert hasattr(lib, name), name
+    assert b"gfx950" in _lib.hip_lib().cbm_version()
+    assert _lib.hip_lib().cbm_status_string(3) != _lib.hip_lib().cbm_status_string(0)
+
+
+def test_struct_mirror_layout():
+    # struct cbm_format: 2 x int32, 4 x int64, 7 pointers
+    assert C.sizeof(_lib.CbmFormat) == 8 + 32 + 56
+    assert _lib.CbmFormat.rowptr.offset == 40
+
+
+def test_shim_exports_the_reference_extension_names():
+    from cbm import cbm_mkl_cpp
+    ref = ["from_coo_int32_t_v1_", "from_coo_int32_t_v2_", "seq_s_spmm_update_csr_int32", "seq_s_update_csr_int32",
+           "seq_s_spmm_csr_int32", "omp_s_spmm_update_csr_int32", "omp_s_update_avx_int32", "omp_s_update_csr_int32",
+           "omp_s_spmm_csr_int32", "omp_s_fused_spmm_update_csr_int32", "omp_s_fused_update_csr_int32",
+           "seq_s_fused_spmm_update_csr_int32", "seq_s_fused_update_csr_int32"]       # cbm_extensions.cpp:1757-1771
+    for name in ref:
+        assert callable(getattr(cbm_mkl_cpp, name)), name
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "cbm4gnn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("cbm_oracle", "oracle") or "import" not in "".join(
+                    l for l in text.splitlines() if "oracle" in l), f
+    for f in ("cbm.py", "cbm_mkl_cpp.py", "utility.py", "__init__.py"):
+        assert "oracle" not in open(os.path.join(ROOT, "cbm", f)).read()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_hip", None)
+    monkeypatch.setattr(_lib, "HIP_LIB", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.CbmLibraryError):
+        _lib.hip_lib()

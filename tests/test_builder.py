@@ -1,0 +1,175 @@
+"""The product's host builder (libcbm_host.so) against the oracle and against invariants.
+"Bit-exact format arrays": every integer array the builder emits equals the independent
+derivation from its own parent[] (oracle.format_from_parent, set differences)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from cbm4gnn_amd import _lib, graphs
+from cbm4gnn_amd.cbm import cbm_matrix, tree_levels
+
+
+def _u32(t):
+    return t.numpy().view(np.uint32)
+
+
+def _assert_format_equals_derivation(orc, ei, n, mat):
+    f = orc.format_from_parent(ei, n, mat.parent.numpy())
+    assert np.array_equal(f["rowptr"], mat.rowptr.numpy())
+    assert np.array_equal(f["idx"], _u32(mat.idx))
+    assert np.array_equal(f["order"], mat.order.numpy())
+    assert np.array_equal(f["level_off"], mat.level_off.numpy())
+    assert np.array_equal(f["mst_row"], mat.mst_row.numpy())
+    assert np.array_equal(f["mst_col"], mat.mst_col.numpy())
+
+
+@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("alpha", [0, 1, 3, 8])
+def test_builder_matches_oracle_small(orc, seed, alpha):
+    n = 25 + 6 * seed
+    ei = graphs.erdos_renyi(n, [0.15, 0.5, 0.75][seed % 3], seed)
+    if seed % 2:
+        ei = graphs.add_self_loops(ei, n)
+    mat = cbm_matrix(torch.from_numpy(ei), torch.ones(ei.shape[1]), alpha=alpha)
+    o = orc.build_format(ei, n, alpha)
+    assert mat.n_candidates == o["n_candidates"]
+    assert mat.nnz == o["msa_weight"] == o["nnz"]          # two different MSA algorithms, same optimum
+    assert mat.nnz_a == ei.shape[1]
+    _assert_format_equals_derivation(orc, ei, n, mat)
+    assert orc.check_format(ei, n, mat.rowptr.numpy(), _u32(mat.idx), mat.mst_row.numpy(), mat.mst_col.numpy())
+    assert mat.check_format(torch.from_numpy(ei))
+
+
+def _small_chain_workload():
+    # the alpha-sweep workload's construction (clique blocks + staircase chain) at a size the
+    # oracle's O(V E) arborescence finishes in seconds
+    ei = graphs.sbm_with_chain(n=1500, blocks=24, p_in=1.0, mean_deg=80.0, chain=64, base=48, seed=0)
+    return graphs.Workload("c5-small", ei, 1500, 32, False, (0, 4), "normal")
+
+
+@pytest.mark.parametrize("name,scale", [("c1", 1.0), ("c2", 0.25), ("c3", 0.02), ("c5-small", 1.0)])
+def test_builder_matches_oracle_workloads(orc, name, scale):
+    w = _small_chain_workload() if name == "c5-small" else graphs.workload(name, scale=scale)
+    for alpha in w.alphas[:2]:
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized)
+        o = orc.build_format(w.edge_index, w.n, alpha)
+        assert mat.n_candidates == o["n_candidates"]
+        assert mat.nnz == o["msa_weight"]
+        assert orc.check_format(w.edge_index, w.n, mat.rowptr.numpy(), _u32(mat.idx), mat.mst_row.numpy(), mat.mst_col.numpy())
+        assert mat.compression_ratio() == pytest.approx(orc.compression_ratio(w.n, w.edge_index.shape[1], o["nnz"]))
+
+
+def test_level_ordering_invariants():
+    w = graphs.workload("c2", scale=0.25)
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=0)
+    n = w.n
+    parent, order, lo = mat.parent.numpy(), mat.order.numpy(), mat.level_off.numpy()
+    assert sorted(order.tolist()) == list(range(n))
+    assert lo[0] == 0 and lo[-1] == n and (np.diff(lo) > 0).all()
+    level = np.empty(n, np.int64)
+    for l in range(len(lo) - 1):
+        seg = order[lo[l]:lo[l + 1]]
+        assert (np.diff(seg) > 0).all()                     # ids ascending inside a level
+        level[seg] = l
+    roots = parent < 0
+    assert (level[roots] == 0).all()
+    assert (level[~roots] == level[parent[~roots]] + 1).all()
+    assert mat.n_levels > 3                                 # the workload really has a deep-ish tree
+    # the tree CSR and the level arrays describe the same tree
+    p2, o2, lo2 = tree_levels(mat.mst_row.numpy(), mat.mst_col.numpy())
+    assert np.array_equal(p2, parent) and np.array_equal(o2, order) and np.array_equal(lo2, lo)
+
+
+def test_packed_sign_round_trip_and_deltas_tensor(orc):
+    n = 60
+    ei = graphs.add_self_loops(graphs.erdos_renyi(n, 0.4, 4), n)
+    for normalized in (False, True):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=normalized)
+        d = mat.deltas
+        assert d.layout == torch.sparse_csr
+        assert d.crow_indices().dtype == torch.int64 and d.values().dtype == torch.float32
+        idx = _u32(mat.idx)
+        assert np.array_equal(d.col_indices().numpy(), (idx & 0x7FFFFFFF).astype(np.int64))
+        assert np.array_equal(d.values().numpy() < 0, (idx >> 31).astype(bool))
+        assert (idx >> 31).any()                            # the case has negative entries at all
+        # values are +-1, or +-m[col] exactly as the reference's v2 builder stores them
+        o = orc.build_format(ei, n, 1)
+        m = orc.col_multiplier(ei, n) if normalized else None
+        if np.array_equal(o["parent"] % n, mat.parent.numpy() % n):
+            crow, col, val = orc.deltas_csr(o, n, m)
+            assert np.array_equal(d.crow_indices().numpy(), crow)
+            assert np.array_equal(d.col_indices().numpy(), col)
+            assert np.array_equal(d.values().numpy(), val)
+        if normalized:
+            assert np.array_equal(mat.col_multiplier.numpy(), m)
+        # columns ascending within each row
+        crow = d.crow_indices().numpy()
+        for r in range(n):
+            assert (np.diff(d.col_indices().numpy()[crow[r]:crow[r + 1]]) > 0).all()
+
+
+def test_special_cases():
+    n = 40
+    ei = graphs.erdos_renyi(n, 0.5, 3)
+    flat = cbm_matrix(torch.from_numpy(ei), None, alpha=10_000)
+    assert flat.n_levels == 1 and (flat.parent == -1).all() and flat.nnz == ei.shape[1]
+    assert np.array_equal((_u32(flat.idx)).astype(np.int64), ei[1][np.lexsort((ei[1], ei[0]))])
+    clique = np.array([(i, j) for i in range(9) for j in range(9)], np.int32).T
+    star = cbm_matrix(torch.from_numpy(clique), None, alpha=0)
+    assert star.nnz == 9 and int((star.parent == -1).sum()) == 1 and star.n_levels == 2
+    assert star.compression_ratio() > 1.5
+
+
+def test_deep_chain_is_found():
+    # the staircase of the alpha-sweep workload forces a path of chain+1 rows
+    w = _small_chain_workload()
+    for alpha in (0, 8, 32):
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha)
+        assert mat.n_levels >= 65                            # root -> c_0 -> ... -> c_64
+
+
+def test_builder_is_thread_count_invariant_and_merges_duplicates():
+    w = graphs.workload("c1")
+    ei = torch.from_numpy(w.edge_index)
+    a = cbm_matrix(ei, None, alpha=0, threads=1)
+    b = cbm_matrix(ei, None, alpha=0, threads=4)
+    perm = torch.randperm(ei.size(1), generator=torch.Generator().manual_seed(0))
+    c = cbm_matrix(torch.cat([ei[:, perm], ei[:, :100]], dim=1), None, alpha=0)     # shuffled + duplicates
+    for x in (b, c):
+        for name in ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col"):
+            assert torch.equal(getattr(a, name), getattr(x, name)), name
+        assert x.nnz_a == a.nnz_a
+
+
+def test_builder_error_codes():
+    fmt = _lib.CbmFormat()
+    lib = _lib.host_lib()
+    row = np.array([0, 1, 5], np.int32); col = np.array([1, 0, 0], np.int32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    assert lib.cbm_build_host(p(row), p(col), 3, 3, 0, 0, C.byref(fmt)) == 3         # index out of range
+    assert lib.cbm_build_host(p(row), p(col), 3, 0, 0, 0, C.byref(fmt)) == 3         # n <= 0
+    assert lib.cbm_build_host(None, None, 3, 3, 0, 0, C.byref(fmt)) == 1             # NULL
+    assert lib.cbm_build_host(p(row), p(col), 3, 6, 0, 0, None) == 1
+    assert lib.cbm_build_host(p(row), p(col), 3, 6, 0, 0, C.byref(fmt)) == 0         # rows 2,3,4 empty: fine
+    assert fmt.n == 6 and fmt.nnz == 2                                         # rows 1 and 5 are identical
+    lib.cbm_format_free(C.byref(fmt))
+    assert not fmt.rowptr
+    with pytest.raises(ValueError):
+        cbm_matrix(torch.zeros((3, 4), dtype=torch.int32), None)
+    with pytest.raises(ValueError):
+        cbm_matrix(torch.tensor([[0, 1], [1, 0]], dtype=torch.int32), None, rows=7)
+
+
+def test_graph_generators_are_pinned():
+    import json, os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "graph_hashes.json")) as f:
+        want = json.load(f)
+    for name in ("c1", "c2", "c3"):
+        w = graphs.workload(name)
+        assert w.edge_index.shape[1] == want[name]["edges"]
+        assert graphs.edge_hash(w.edge_index) == want[name]["sha256"], name
+        if name == "c1":
+            from cbm4gnn_amd.utility import check_edge_index
+            check_edge_index(torch.from_numpy(w.edge_index).long())
