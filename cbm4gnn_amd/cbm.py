@@ -188,6 +188,16 @@ class cbm_matrix:
             self._deltas = csr if self.deltas_format == "csr" else csr.to_sparse_coo().coalesce()
         return self._deltas
 
+    def to_sparse_coo_tensor(self, row, col, val, data_type=torch.float32):
+        """COO triplets -> coalesced torch COO tensor (``cbm.py:120-129``)."""
+        size = int(max(row.max(), col.max())) + 1
+        index = torch.stack((row.to(torch.int64), col.to(torch.int64)))
+        return torch.sparse_coo_tensor(index, val, size=(size, size)).to(data_type).coalesce()
+
+    def to_sparse_csr_tensor(self, row, col, val, data_type=torch.float32):
+        """COO triplets -> torch CSR tensor (``cbm.py:132-141``)."""
+        return self.to_sparse_coo_tensor(row, col, val, data_type).to_sparse_csr()
+
     def compression_ratio(self):
         """Element-count ratio CSR(A) / CBM, ``benchmark/utility.py:45-64``."""
         n = self.num_rows
@@ -217,8 +227,6 @@ class cbm_matrix:
                     else:
                         sv.remove(col[k])
                 s[v] = sv
-            if u != n_rows:
-                s[u] = frozenset(s[u])
         if visited != n_rows:
             raise ValueError("Format is incorrect!")
         a = [set() for _ in range(n_rows)]

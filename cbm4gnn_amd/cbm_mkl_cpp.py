@@ -101,9 +101,12 @@ def _csr_spmm(row_b, row_e, col, val, rhs, dst_dev, dev):
     rowptr = torch.cat([row_b.detach().cpu().reshape(-1), row_e.detach().cpu().reshape(-1)[-1:]]).contiguous()
     if n > 1 and not torch.equal(rowptr[1:-1], row_e.detach().cpu().reshape(-1)[:-1]):
         raise ValueError("row_b / row_e must be the two slices of one row-pointer array")
+    # device copies stay referenced until the launch is enqueued: a temporary freed earlier could
+    # be handed out again by the caching allocator and overwritten by the next upload
     x = rhs.to(dev)
-    rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr.to(dev)), _ptr(col.to(dev).contiguous()), _ptr(val.to(dev).contiguous()),
-                                     None, _ptr(x), _ptr(dst_dev), n, x.size(1), _ld(x), _ld(dst_dev), _stream(dev))
+    rowptr_d, col_d, val_d = rowptr.to(dev), col.to(dev).contiguous(), val.to(dev).contiguous()
+    rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr_d), _ptr(col_d), _ptr(val_d), None, _ptr(x), _ptr(dst_dev),
+                                     n, x.size(1), _ld(x), _ld(dst_dev), _stream(dev))
     _lib.check(rc, "csr_spmm_f32")
 
 

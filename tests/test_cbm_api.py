@@ -1,0 +1,116 @@
+"""Host-side surface of cbm_matrix (no GPU): constructor, attributes, the reference's method
+names, error behaviour, and the loud failure when no HIP device exists."""
+import numpy as np
+import pytest
+import torch
+
+from cbm4gnn_amd import graphs
+from cbm.cbm import cbm_matrix                    # the reference's import path
+
+REFERENCE_METHODS = [                             # cbm/cbm.py:144-275
+    "seq_mkl_csr_spmm_update", "seq_mkl_csr_spmm", "seq_mkl_csr_update", "seq_mkl_csr_fused_spmm_update",
+    "seq_mkl_csr_fused_update", "omp_mkl_csr_spmm_update", "omp_mkl_csr_spmm", "omp_mkl_csr_update",
+    "omp_avx_csr_update", "omp_mkl_csr_spmm_update_v2", "omp_mkl_csr_fused_spmm_update", "omp_mkl_csr_fused_update",
+    "seq_torch_csr_matmul", "omp_torch_csr_matmul", "seq_torch_csr_fused_matmul", "omp_torch_csr_fused_matmul",
+    "check_format", "to_sparse_coo_tensor", "to_sparse_csr_tensor",
+]
+
+
+@pytest.fixture(scope="module")
+def er25():
+    ei = graphs.erdos_renyi(25, 0.5, 0)
+    return torch.from_numpy(ei), torch.ones(ei.shape[1], dtype=torch.float32)
+
+
+@pytest.mark.parametrize("alpha", [1, 2, 3, 4])
+def test_creation_like_the_reference_test(er25, alpha):
+    # tests/test_cbm_creation.py:33-48: construction succeeds for alpha in 1..4
+    ei, vals = er25
+    assert cbm_matrix(ei, vals, alpha=alpha) is not None
+    assert cbm_matrix(ei, vals, alpha=alpha, normalized=True) is not None
+
+
+def test_attributes_and_methods(er25):
+    ei, vals = er25
+    c = cbm_matrix(ei, vals, alpha=3)
+    for name in REFERENCE_METHODS:
+        assert callable(getattr(c, name)), name
+    assert c.mst_row.dtype == torch.int32 and c.mst_row.numel() == 25 + 2
+    assert c.mst_col.dtype == torch.int32 and c.mst_col.numel() == 25
+    assert c.col_multiplier is None
+    assert c.deltas.layout == torch.sparse_csr and tuple(c.deltas.shape) == (25, 25)
+    assert cbm_matrix(ei, vals, alpha=3, deltas_format="coo").deltas.layout == torch.sparse_coo
+    cn = cbm_matrix(ei, vals, alpha=3, normalized=True)
+    deg = torch.bincount(ei[0].long(), minlength=25).float()
+    assert torch.equal(cn.col_multiplier, deg.pow(-0.5))
+    # the reference's compression-ratio helper reads exactly these attributes (benchmark/utility.py:54-60)
+    total = (c.deltas.col_indices().numel() + c.deltas.crow_indices().numel() + c.deltas.values().numel()
+             + c.mst_row.numel() + c.mst_col.numel())
+    assert c.compression_ratio() == pytest.approx((26 + 2 * ei.size(1)) / total)
+
+
+def test_check_format_detects_corruption(er25):
+    ei, vals = er25
+    c = cbm_matrix(ei, vals, alpha=0)
+    assert c.check_format(ei)
+    bad = c.idx.clone()
+    k = int(torch.nonzero(bad >= 0)[0])
+    c.idx = bad
+    c.idx[k] = (int(bad[k]) + 1) % 25
+    with pytest.raises((ValueError, KeyError)):
+        c.check_format(ei)
+
+
+def test_deltas_times_x_plus_walk_equals_product_on_cpu_tensors_math(er25):
+    # pure host arithmetic on the format (dense fp64): Delta @ X, then the top-down walk, is A @ X
+    ei, vals = er25
+    c = cbm_matrix(ei, vals, alpha=2)
+    x = np.random.default_rng(0).integers(0, 10, (25, 10)).astype(np.float64)
+    y = c.deltas.to_dense().double().numpy() @ x
+    parent = c.parent.numpy()
+    for v in c.order.numpy():
+        if parent[v] >= 0:
+            y[v] += y[parent[v]]
+    a = np.zeros((25, 25)); a[ei[0].numpy(), ei[1].numpy()] = 1
+    assert np.array_equal(y, a @ x)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU failure mode")
+def test_multiply_without_gpu_raises_instead_of_falling_back(er25):
+    ei, vals = er25
+    c = cbm_matrix(ei, vals, alpha=3)
+    x = torch.ones(25, 10)
+    y = torch.empty(25, 10)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        c.omp_mkl_csr_spmm_update(x, y)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        c.seq_torch_csr_matmul(x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        c.omp_mkl_csr_update(y)
+
+
+def test_argument_checks_come_before_any_device_work(er25):
+    ei, vals = er25
+    c = cbm_matrix(ei, vals, alpha=3)
+    y = torch.empty(25, 10)
+    with pytest.raises(RuntimeError, match="kFloat32"):             # the reference's TORCH_CHECK text
+        c.omp_mkl_csr_spmm_update(torch.ones(25, 10, dtype=torch.float64), y)
+    with pytest.raises(ValueError):
+        c.omp_mkl_csr_spmm_update(torch.ones(24, 10), y)
+    with pytest.raises(ValueError):
+        c.omp_mkl_csr_spmm_update(torch.ones(25, 9), y)
+    with pytest.raises(ValueError):
+        c.omp_mkl_csr_spmm_update(torch.ones(10, 25).t(), y)        # column-major view
+    with pytest.raises(RuntimeError, match="normalized=False"):
+        c.omp_mkl_csr_fused_spmm_update(torch.ones(25, 10), y)
+
+
+def test_symmetry_flag_and_transpose():
+    ei = torch.tensor([[0, 1, 2, 2], [1, 2, 0, 1]], dtype=torch.int32)
+    c = cbm_matrix(ei, None)
+    assert not c.is_symmetric
+    t = c.transposed()
+    assert t is not c and t.transposed() is c
+    assert torch.equal(t.deltas.to_dense(), c.deltas.to_dense().t()) or t.nnz <= 4
+    und = cbm_matrix(torch.from_numpy(graphs.erdos_renyi(10, 0.5, 1)), None)
+    assert und.is_symmetric and und.transposed() is und

@@ -1,0 +1,264 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on identical seeded inputs.
+
+Tolerances (stated by the task this library serves): fp32 max-relative error <= 1e-4 against the
+reference-style CPU CBM path, <= 1e-3 against a plain CSR / dense product; integer format arrays
+and integer-feature products bit-exact."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from cbm4gnn_amd import _lib, graphs
+from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm
+
+pytestmark = pytest.mark.gpu
+
+TOL_CBM = 1e-4
+TOL_CSR = 1e-3
+
+
+def say(*a):
+    print("[gpu-case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    _lib.hip_lib()
+
+
+def oracle_product(orc, mat, ei, n, x, normalized, threads=4):
+    """Reference-style CPU multiply on the PRODUCT's tree (so both sides sum in the same order)."""
+    col, sign = mat.columns()
+    m = orc.col_multiplier(ei, n) if normalized else None
+    val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
+    return orc.spmm_update(mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32),
+                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads)
+
+
+def gpu_product(mat, x, normalized):
+    xd = torch.from_numpy(x).cuda()
+    yd = torch.full_like(xd, float("nan"))                 # beta = 0: stale contents must not leak
+    (mat.omp_mkl_csr_fused_spmm_update if normalized else mat.omp_mkl_csr_spmm_update)(xd, yd)
+    torch.cuda.synchronize()
+    return yd.cpu().numpy()
+
+
+# ---------------------------------------------------------------- golden fixtures ---------
+@pytest.mark.parametrize("case", range(5))
+@pytest.mark.parametrize("alpha", [0, 2, 3])
+def test_golden_integer_products_bit_exact(golden, case, alpha):
+    ei, x = golden[f"case{case}_edge_index"], golden[f"case{case}_x"]
+    say("golden", case, alpha)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha)
+    got = gpu_product(mat, x, False)
+    assert np.array_equal(got.astype(np.float64), golden[f"case{case}_ax"])
+    matn = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=True)
+    gotn = gpu_product(matn, x, True)
+    np.testing.assert_allclose(gotn, golden[f"case{case}_ax_normalized"], rtol=TOL_CBM, atol=TOL_CBM)
+
+
+# ---------------------------------------------------------------- oracle parity -----------
+@pytest.mark.parametrize("d", [1, 3, 10, 41, 64, 100, 128, 256, 258, 512, 602, 1000, 1028, 2052])
+@pytest.mark.parametrize("normalized", [False, True])
+def test_widths_against_oracle(orc, d, normalized):
+    n = 700
+    ei = graphs.add_self_loops(graphs.sbm(n, 10, 0.3, 0.01, seed=d), n)
+    say("widths", d, normalized)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=normalized)
+    assert mat.n_levels >= 2 and (mat.idx < 0).any()
+    x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+    got = gpu_product(mat, x, normalized)
+    want = oracle_product(orc, mat, ei, n, x, normalized)
+    assert orc.max_rel_err(got, want) <= TOL_CBM
+    assert np.array_equal(got, want)                       # same order, same FMAs: in fact bit-exact
+    assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CSR
+
+
+@pytest.mark.parametrize("name,scale,alphas", [("c1", 1.0, (0,)), ("c2", 0.5, (0, 8)), ("c3", 0.05, (0, 16))])
+def test_workloads_against_oracle(orc, name, scale, alphas):
+    w = graphs.workload(name, scale=scale)
+    x = w.features(0).numpy()
+    for alpha in alphas:
+        say("workload", name, scale, alpha)
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized)
+        got = gpu_product(mat, x, w.normalized)
+        # (1) the oracle's own build (its own arborescence): the reference-style CPU path end to end
+        fmt = orc.build_format(w.edge_index, w.n, alpha)
+        m = orc.col_multiplier(w.edge_index, w.n) if w.normalized else None
+        crow, col, val = orc.deltas_csr(fmt, w.n, m)
+        want = orc.spmm_update(crow, col, val, fmt["mst_row"], fmt["mst_col"], x, m, threads=4)
+        assert orc.max_rel_err(got, want) <= TOL_CBM
+        # (2) plain CSR A @ X on the CPU
+        ei = w.edge_index
+        order = np.lexsort((ei[1], ei[0]))
+        rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=w.n))]).astype(np.int32)
+        vals = (m[ei[0][order]] * m[ei[1][order]]).astype(np.float32) if w.normalized else None
+        csr = orc.csr_spmm(rp, ei[1][order], vals, x, threads=4)
+        assert orc.max_rel_err(got, csr) <= TOL_CSR
+        # (3) the GPU CSR baseline computes the same thing
+        yd = torch.empty((w.n, x.shape[1]), device="cuda")
+        csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(ei[1][order].astype(np.int32)).cuda(),
+                 None if vals is None else torch.from_numpy(vals).cuda(), torch.from_numpy(x).cuda(), yd)
+        assert np.array_equal(yd.cpu().numpy(), csr)       # same in-order FMA chain as the oracle
+
+
+def test_reference_test_matmul_correctness(orc):
+    # tests/test_matmul_correctness.py:30-61 restated with a seed: ER(25, 0.5), alpha=3, d=10,
+    # integer features, CBM product == COO product at atol=rtol=1e-4; CPU tensors in and out
+    for seed in range(4):
+        ei = torch.from_numpy(graphs.erdos_renyi(25, 0.5, seed))
+        feats = torch.randint(0, 10, (25, 10), generator=torch.Generator().manual_seed(seed)).float()
+        vals = torch.ones(ei.size(1))
+        want = torch.sparse_coo_tensor(ei.long(), vals, (25, 25)) @ feats
+        say("reference test", seed)
+        c = cbm_matrix(ei, vals, alpha=3)
+        torch.testing.assert_close(want, c.seq_torch_csr_matmul(feats), atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(want, c.omp_torch_csr_matmul(feats), atol=1e-4, rtol=1e-4)
+        out = torch.empty(25, 10)
+        c.omp_mkl_csr_spmm_update(feats, out)
+        assert torch.equal(want, out)
+
+
+# ---------------------------------------------------------------- each entry point --------
+def test_update_only_entry_points(orc):
+    n, d = 900, 72
+    ei = graphs.add_self_loops(graphs.sbm(n, 12, 0.25, 0.01, seed=7), n)
+    x = np.random.default_rng(7).standard_normal((n, d)).astype(np.float32)
+    for normalized in (False, True):
+        say("update-only", normalized)
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+        # spmm alone == Delta (diag m) X
+        z = torch.empty((n, d), device="cuda")
+        mat.omp_mkl_csr_spmm(torch.from_numpy(x).cuda(), z)
+        col, sign = mat.columns()
+        m = orc.col_multiplier(ei, n) if normalized else None
+        val = (sign.numpy() * (m[col.numpy()] if normalized else 1)).astype(np.float32)
+        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x)
+        assert np.array_equal(z.cpu().numpy(), z_ref)
+        # update alone on that Z == the oracle's walk (plain or fused) on the same Z
+        y = z.clone()
+        (mat.omp_mkl_csr_fused_update if normalized else mat.omp_mkl_csr_update)(y)
+        ref = z_ref.copy()
+        if normalized:
+            orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, ref)
+        else:
+            orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), ref)
+        assert np.array_equal(y.cpu().numpy(), ref)
+        # and spmm_update in one call agrees with the two-step result
+        assert np.array_equal(gpu_product(mat, x, normalized), ref)
+        # seq_/avx twins are the same code
+        y2 = z.clone()
+        (mat.seq_mkl_csr_fused_update if normalized else mat.omp_avx_csr_update)(y2)
+        assert torch.equal(y, y2)
+
+
+def test_deep_narrow_tree_uses_multi_level_kernel(orc):
+    # 64-deep staircase chain: runs of width-1 levels go through the single-workgroup kernel
+    ei = graphs.sbm_with_chain(n=1500, blocks=24, p_in=1.0, mean_deg=80.0, chain=64, base=48, seed=0)
+    n = 1500
+    for normalized, d in ((False, 512), (True, 96), (False, 10)):
+        e2 = graphs.add_self_loops(ei, n) if normalized else ei
+        mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
+        assert mat.n_levels >= 65
+        say("deep chain", normalized, d, "levels", mat.n_levels)
+        x = np.random.default_rng(1).standard_normal((n, d)).astype(np.float32)
+        got = gpu_product(mat, x, normalized)
+        want = oracle_product(orc, mat, e2, n, x, normalized)
+        assert np.array_equal(got, want)
+        assert orc.max_rel_err(got, orc.dense_product(e2, n, x, normalized)) <= TOL_CSR
+
+
+def test_strided_rows_and_cpu_staging(orc):
+    n, d = 300, 48
+    ei = graphs.erdos_renyi(n, 0.1, 5)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1)
+    x = np.random.default_rng(2).standard_normal((n, d)).astype(np.float32)
+    want = oracle_product(orc, mat, ei, n, x, False)
+    say("strided")
+    xbig = torch.zeros((n, d + 5), device="cuda"); xbig[:, :d] = torch.from_numpy(x).cuda()
+    ybig = torch.full((n, d + 9), 7.0, device="cuda")
+    mat.omp_mkl_csr_spmm_update(xbig[:, :d], ybig[:, :d])        # ld = d+5 / d+9, unaligned for float4
+    assert np.array_equal(ybig[:, :d].cpu().numpy(), want)
+    assert (ybig[:, d:] == 7.0).all()                            # nothing written beyond the d columns
+    say("cpu staging")
+    y = torch.empty(n, d)
+    mat.omp_mkl_csr_spmm_update(torch.from_numpy(x), y)
+    assert np.array_equal(y.numpy(), want)
+
+
+def test_autograd_backward_matches_dense(orc):
+    n, d = 200, 24
+    und = graphs.add_self_loops(graphs.erdos_renyi(n, 0.08, 9), n)
+    directed = und[:, (und[0] * 7 + und[1] * 3) % 5 != 0]          # drop ~20% of entries: not symmetric
+    directed = graphs.add_self_loops(directed, n)
+    for ei, normalized in ((und, True), (und, False), (directed, False), (directed, True)):
+        say("autograd", ei.shape[1], normalized)
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+        x = torch.randn((n, d), generator=torch.Generator().manual_seed(1)).cuda().requires_grad_(True)
+        g = torch.randn((n, d), generator=torch.Generator().manual_seed(2)).cuda()
+        y = mat.matmul(x)
+        y.backward(g)
+        a = orc.dense_adjacency(ei, n)
+        if normalized:
+            m = a.sum(axis=1) ** -0.5
+            a = m[:, None] * a * m[None, :]
+        assert orc.max_rel_err(y.detach().cpu().numpy(), a @ x.detach().cpu().numpy().astype(np.float64)) <= TOL_CSR
+        assert orc.max_rel_err(x.grad.cpu().numpy(), a.T @ g.cpu().numpy().astype(np.float64)) <= TOL_CSR
+
+
+def test_shim_functions_match_cbm_matrix(orc):
+    from cbm import cbm_mkl_cpp as cbm_
+    n, d = 120, 20
+    ei_np = graphs.add_self_loops(graphs.erdos_renyi(n, 0.2, 3), n)
+    ei = torch.from_numpy(ei_np)
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(0))
+    say("shim")
+    for normalized in (False, True):
+        c = cbm_matrix(ei, None, alpha=2, normalized=normalized)
+        want = gpu_product(c, x.numpy(), normalized)
+        mul = c.col_multiplier
+        data = (cbm_.from_coo_int32_t_v2_(ei[0], ei[1], torch.ones(ei.size(1)), mul, n, n, 2) if normalized
+                else cbm_.from_coo_int32_t_v1_(ei[0], ei[1], torch.ones(ei.size(1)), n, n, 2))
+        mst_row, mst_col, r, cidx, v = data
+        assert torch.equal(mst_row, c.mst_row) and torch.equal(mst_col, c.mst_col)
+        deltas = torch.sparse_coo_tensor(torch.stack((r, cidx)).long(), v, (n, n)).coalesce().to_sparse_csr()
+        rb = deltas.crow_indices()[:-1].to(torch.int32); re = deltas.crow_indices()[1:].to(torch.int32)
+        col = deltas.col_indices().to(torch.int32); val = deltas.values()
+        y = torch.empty(n, d)
+        if normalized:
+            cbm_.omp_s_fused_spmm_update_csr_int32(rb, re, col, val, x, mst_row, mst_col, mul, y)
+        else:
+            cbm_.omp_s_spmm_update_csr_int32(rb, re, col, val, x, mst_row, mst_col, y)
+        assert np.array_equal(y.numpy(), want)
+        y2 = torch.empty(n, d)
+        cbm_.seq_s_spmm_csr_int32(rb, re, col, val, x, y2)
+        (cbm_.seq_s_fused_update_csr_int32(mst_row, mst_col, mul, y2) if normalized
+         else cbm_.omp_s_update_avx_int32(mst_row, mst_col, y2))
+        assert np.array_equal(y2.numpy(), want)
+    with pytest.raises(RuntimeError, match="kInt32"):
+        cbm_.seq_s_update_csr_int32(mst_row.long(), mst_col, y)
+
+
+def test_c_abi_status_codes_on_device_calls():
+    lib = _lib.hip_lib()
+    n, d = 8, 4
+    x = torch.zeros((n, d), device="cuda"); y = torch.zeros((n, d), device="cuda")
+    rp = torch.zeros(n + 1, dtype=torch.int32, device="cuda"); idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    say("status codes")
+    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, p(x), p(y), n, d, d, d, None) == 1
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, p(x), p(y), n, d, d - 1, d, None) == 3
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, p(x), p(y), n, d, d, d, None) == 0   # empty rows -> zeros
+    lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
+    par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
+    assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
+    lo = (C.c_int32 * 2)(0, n)
+    assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 0
+    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), n, d, d, d, 0, None) == 3
+    torch.cuda.synchronize()
+    assert (y == 0).all()
