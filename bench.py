@@ -124,6 +124,9 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter run: 3 multiplies and 3 plain device copies of X (known size, for scaling "
+                         "FETCH_SIZE / WRITE_SIZE), no timing, no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); "
@@ -154,6 +157,15 @@ def main():
     mat.to(xd.device)
 
     step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
+    if args.probe:
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            yd.copy_(xd)                                   # reads and writes n*d*4 bytes each
+        torch.cuda.synchronize()
+        print(f"probe: 3 multiplies, then 3 device copies of {xd.numel() * 4} bytes (read) + the same written")
+        return
     wall_ms, span_ms, med_ms = time_gpu(step, args.steps, args.warmup, torch)
 
     # the dominant kernel alone (delta SpMM), same launch as inside the step

@@ -162,6 +162,7 @@ class cbm_matrix:
 
         self._deltas = None
         self._dev = {}
+        self.stream_coefficients = True     # False: gather m[col] in the kernel, 4 B/entry less device memory
         self._transposed = None
         keys = ei_cpu[0].to(torch.int64) * n + ei_cpu[1].to(torch.int64)
         keys_t = ei_cpu[1].to(torch.int64) * n + ei_cpu[0].to(torch.int64)
@@ -247,7 +248,16 @@ class cbm_matrix:
                 "rowptr": self.rowptr.to(device), "idx": self.idx.to(device), "parent": self.parent.to(device),
                 "order": self.order.to(device), "level_off": self.level_off.to(device),
                 "m": self.col_multiplier.to(device) if self.col_multiplier is not None else None,
+                "coef": None,
             }
+            if st["m"] is not None and self.nnz and self.stream_coefficients:
+                # +-m[col] per delta entry, expanded once on the device (what the reference keeps
+                # as the fp32 values of its delta matrix); streamed by the SpMM instead of a gather
+                st["coef"] = torch.empty(self.nnz, dtype=torch.float32, device=device)
+                with torch.cuda.device(device):
+                    rc = _lib.hip_lib().cbm_expand_coef_f32(_ptr(st["idx"]), _ptr(st["m"]), _ptr(st["coef"]),
+                                                            self.nnz, _stream(device))
+                _lib.check(rc, "cbm_expand_coef_f32")
             self._dev[key] = st
         return st
 
@@ -282,6 +292,7 @@ class cbm_matrix:
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
+                _ptr(st["coef"]) if use_m else None,
                 _ptr(st["parent"]) if scale_roots else None, None, _ptr(xd), _ptr(yd),
                 n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
         _lib.check(rc, "cbm_spmm_f32")
@@ -325,7 +336,8 @@ class cbm_matrix:
         st = self._device_arrays(xd.device)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
-                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None, _ptr(st["parent"]),
+                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
+                _ptr(st["coef"]) if use_m else None, _ptr(st["parent"]),
                 None, _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
                 _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
         _lib.check(rc, "cbm_spmm_update_f32")

@@ -15,13 +15,28 @@
 // What each launcher replaces in the reference is stated in include/cbm_hip.h.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/cbm_hip.h"
 
 namespace {
 
+// Tunables (overridable with -D for sweeps; the defaults are what measurements on MI355X chose).
+#ifndef CBM_WAVES_PER_BLOCK
+#define CBM_WAVES_PER_BLOCK 4
+#endif
+#ifndef CBM_UNROLL_CH1
+#define CBM_UNROLL_CH1 8
+#endif
+#ifndef CBM_XCD_REMAP
+#define CBM_XCD_REMAP 1
+#endif
+#ifndef CBM_NT_STORE
+#define CBM_NT_STORE 0
+#endif
+
 constexpr int kWave = 64;
-constexpr int kWavesPerBlock = 4;          // SpMM / wide-level propagate: 256 threads
+constexpr int kWavesPerBlock = CBM_WAVES_PER_BLOCK;   // SpMM / wide-level propagate
 constexpr int kNarrowWaves = 16;           // narrow-level propagate: one 1024-thread workgroup
 constexpr int kNarrowWidth = 64;           // a level with at most this many rows is "narrow"
 constexpr int kXcds = 8;                   // MI355X: 8 XCDs, workgroups are dealt round-robin
@@ -30,6 +45,7 @@ constexpr int kXcds = 8;                   // MI355X: 8 XCDs, workgroups are dea
 // logical blocks so that neighbouring rows (which share columns in clustered graphs) meet in
 // the same L2.
 __device__ __forceinline__ int xcd_contiguous_block(int bid, int nb) {
+    if (!CBM_XCD_REMAP) return bid;
     const int q = nb / kXcds, r = nb % kXcds;
     const int x = bid % kXcds;
     return x * q + (x < r ? x : r) + bid / kXcds;
@@ -50,7 +66,13 @@ __device__ __forceinline__ void load_vec(const float* __restrict__ p, float (&v)
 
 template <int VEC>
 __device__ __forceinline__ void store_vec(float* __restrict__ p, const float (&v)[VEC]) {
-    if constexpr (VEC == 4) {
+    if constexpr (CBM_NT_STORE) {
+        typedef float vf __attribute__((ext_vector_type(VEC)));
+        vf t;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) t[e] = v[e];
+        __builtin_nontemporal_store(t, reinterpret_cast<vf*>(p));
+    } else if constexpr (VEC == 4) {
         *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
     } else if constexpr (VEC == 2) {
         *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
@@ -76,7 +98,7 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
     const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
     const float* __restrict__ m, const int32_t* __restrict__ parent, const int32_t* __restrict__ perm,
     const float* __restrict__ X, float* __restrict__ Z, int n, int d, int64_t ldx, int64_t ldz) {
-    constexpr int U = (CH == 1) ? 8 : (CH == 2 ? 4 : 2);      // X-row loads in flight per wave
+    constexpr int U = (CH == 1) ? CBM_UNROLL_CH1 : (CH == 2 ? CBM_UNROLL_CH1 / 2 : CBM_UNROLL_CH1 / 4);   // X-row loads in flight per wave
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     int row = xcd_contiguous_block(blockIdx.x, gridDim.x) * kWavesPerBlock + wave;
@@ -86,6 +108,15 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
     const int start = __builtin_amdgcn_readfirstlane(rowptr[row]);
     const int end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
     const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
+    // left scaling of root children: fetched up front so the loads overlap the gather
+    float root_scale = 1.0f;
+    if constexpr (PACKED) {
+        if (m && parent) {
+            const int par = parent[row];
+            const float mr = m[row];
+            root_scale = par < 0 ? mr : 1.0f;
+        }
+    }
 
     float acc[CH][VEC];
 #pragma unroll
@@ -93,6 +124,11 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
 #pragma unroll
         for (int v = 0; v < VEC; v++) acc[c][v] = 0.0f;
 
+    // One coalesced load brings 64 packed indices into the wave and, in the same step, each lane
+    // resolves the coefficient of its entry (sign bit, m[col] gather, or the streamed CSR value);
+    // entry k is then broadcast with v_readlane into scalar registers, so the row address of X
+    // is wave-uniform and the only per-entry vector memory traffic is the X row itself.
+    // (Looking m[col] up per entry through the scalar cache instead measured 3% slower.)
     for (int base = start; base < end; base += kWave) {
         const int cnt = min(kWave, end - base);
         int my_col = 0;
@@ -101,8 +137,11 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
             if constexpr (PACKED) {
                 const uint32_t p = idx[base + lane];
                 my_col = (int)(p & 0x7fffffffu);
-                const float mag = m ? m[my_col] : 1.0f;
-                my_cf = (p >> 31) ? -mag : mag;
+                if (val) my_cf = val[base + lane];                     // streamed +-m[col]
+                else {
+                    const uint32_t mag = m ? __float_as_uint(m[my_col]) : 0x3f800000u;
+                    my_cf = __uint_as_float(mag ^ (p & 0x80000000u));  // +-1 or +-m[col], exact
+                }
             } else {
                 my_col = (int)idx[base + lane];
                 my_cf = val ? val[base + lane] : 1.0f;
@@ -146,18 +185,129 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
         }
     }
     if constexpr (PACKED) {
-        if (m && parent && parent[row] < 0) {      // child of the root: left scaling, final value
-            const float s = m[row];
+        if (m && parent)                           // child of the root: left scaling, final value
 #pragma unroll
             for (int c = 0; c < CH; c++)
 #pragma unroll
-                for (int v = 0; v < VEC; v++) acc[c][v] *= s;
-        }
+                for (int v = 0; v < VEC; v++) acc[c][v] *= root_scale;
     }
     float* __restrict__ zr = Z + (int64_t)row * ldz + col0;
 #pragma unroll
     for (int c = 0; c < CH; c++)
         if (FULL || col0 + c * kWave * VEC < d) store_vec<VEC>(zr + c * kWave * VEC, acc[c]);
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// (1b) SpMM with the feature dimension split into slabs, one slab per XCD.
+//
+// X is N x d fp32.  A workgroup on XCD x only ever touches the columns of its slab s (LPE float4
+// per row: 128 B for LPE = 8, 256 B for LPE = 16) of X and Z, so the working set each XCD's 4 MB
+// L2 sees is N x slab bytes instead of all of X: rows of X that many delta rows share stay
+// resident.  Inside a wave, LPE lanes serve one delta entry and the 64 / LPE lane groups serve
+// that many consecutive entries of the same row at once; each group keeps its own partial sum
+// (entries k = g mod (64 / LPE), in order) and the partial sums are added by a xor-shuffle tree
+// at the end of the row.  The price: index (and coefficient) arrays are streamed once per slab.
+// Coefficients: `coef` (streamed, +-m[col] precomputed) if given, else m[col] gathered, else +-1.
+// ---------------------------------------------------------------------------------------------
+template <int LPE, bool PACKED, int U>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
+    const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
+    const float* __restrict__ m, const int32_t* __restrict__ parent, const int32_t* __restrict__ perm,
+    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int row_blocks, int64_t ldx,
+    int64_t ldz) {
+    constexpr int kSlab = LPE * 4;                         // floats per slab
+    constexpr int kStep = kWave / LPE;                     // entries per wave instruction
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int sub = lane / LPE;                            // which entry of a step
+    const int li = lane % LPE;                             // float4 position inside the slab
+    // workgroup b runs on XCD b % 8.  n_slabs >= 8 (a multiple of 8): XCD x owns slabs x, x + 8, ...
+    // and finishes all row blocks of one slab before it starts the next, so one slab at a time
+    // competes for its L2;  n_slabs < 8 (a divisor of 8): 8 / n_slabs XCDs share a slab and split
+    // its row blocks.
+    int slab, rb;
+    {
+        const int b = blockIdx.x;
+        const int x = b % kXcds, j = b / kXcds;
+        if (n_slabs >= kXcds) {
+            slab = x + kXcds * (j / row_blocks);
+            rb = j % row_blocks;
+        } else {
+            const int share = kXcds / n_slabs;
+            slab = x % n_slabs;
+            rb = j * share + x / n_slabs;
+        }
+    }
+    if (rb >= row_blocks) return;
+    int row = rb * kWavesPerBlock + wave;
+    if (row >= n) return;
+    if (perm) row = perm[row];
+    row = __builtin_amdgcn_readfirstlane(row);
+    const int start = __builtin_amdgcn_readfirstlane(rowptr[row]);
+    const int end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
+    const float* __restrict__ Xs = X + slab * kSlab + li * 4;
+    // left scaling of root children: fetched up front so the loads overlap the gather
+    float root_scale = 1.0f;
+    if constexpr (PACKED) {
+        if (m && parent) {
+            const int par = parent[row];
+            const float mr = m[row];
+            root_scale = par < 0 ? mr : 1.0f;
+        }
+    }
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int pos = start; pos < end; pos += kStep * U) {
+        float x[U][4];
+        float f[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = pos + u * kStep + sub;
+            f[u] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) x[u][e] = 0.0f;
+            if (k < end) {
+                const uint32_t p = idx[k];
+                const uint32_t c = PACKED ? (p & 0x7fffffffu) : p;
+                if constexpr (PACKED) {
+                    if (val) f[u] = val[k];                // streamed +-m[col]
+                    else {
+                        const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
+                        f[u] = __uint_as_float(mag ^ (p & 0x80000000u));
+                    }
+                } else {
+                    f[u] = val ? val[k] : 1.0f;
+                }
+                load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] = fmaf(f[u], x[u][e], acc[e]);
+    }
+#pragma unroll
+    for (int off = LPE; off < kWave; off <<= 1)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
+    if (sub == 0) {
+        if constexpr (PACKED) {
+            if (m && parent)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e] *= root_scale;
+        }
+        store_vec<4>(Z + (int64_t)row * ldz + slab * kSlab + li * 4, acc);
+    }
+}
+
+// coef[k] = +-m[col(k)]: the packed entries expanded once so the SpMM can stream coefficients.
+__global__ __launch_bounds__(256) void expand_coef(const uint32_t* __restrict__ idx, const float* __restrict__ m,
+                                                   float* __restrict__ coef, int64_t nnz) {
+    const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= nnz) return;
+    const uint32_t p = idx[k];
+    coef[k] = __uint_as_float(__float_as_uint(m[p & 0x7fffffffu]) ^ (p & 0x80000000u));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -275,6 +425,22 @@ inline Tiling pick_tiling(int d, int64_t ld_a, int64_t ld_b, const void* pa, con
     return t;
 }
 
+// SpMM kernel choice: 0 = automatic, 1 = always one wave per row, 2 = slabs whenever the shape allows
+int g_spmm_kernel = 0;
+
+// Lanes per delta entry of the slab kernel (8 -> 128-byte slabs, 16 -> 256-byte slabs), or 0 when
+// the wave-per-row kernel should run: d must split into whole slabs whose count divides, or is a
+// multiple of, the 8 XCDs, and rows must be float4-addressable.  A wider slab is taken only when
+// it still leaves one slab per XCD.
+inline int pick_slab_lanes(int d, int64_t ld_a, int64_t ld_b, const void* pa, const void* pb) {
+    if (g_spmm_kernel == 1) return 0;
+    if (d % 32 != 0 || ld_a % 4 != 0 || ld_b % 4 != 0 || !aligned(pa, 16) || !aligned(pb, 16)) return 0;
+    int lpe = 8;
+    if (d % 64 == 0 && d / 64 >= kXcds) lpe = 16;
+    const int n_slabs = d / (lpe * 4);
+    return (n_slabs % kXcds == 0 || kXcds % n_slabs == 0) ? lpe : 0;
+}
+
 #define CBM_DISPATCH_TILING(T, LAUNCH)                                              \
     do {                                                                            \
         if ((T).full) { CBM_DISPATCH_VC(T, true, LAUNCH); }                         \
@@ -311,6 +477,23 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
     if (int rc = check_matrix(n, d, ldz)) return rc;
     if (n == 0 || d == 0) return CBM_OK;
     const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
+    if (const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z)) {
+        const int n_slabs = d / (lpe * 4);
+        const int row_blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
+        int64_t gx;
+        if (n_slabs >= kXcds) gx = (int64_t)row_blocks * n_slabs;
+        else { const int share = kXcds / n_slabs; gx = (int64_t)((row_blocks + share - 1) / share) * kXcds; }
+        if (gx <= INT32_MAX) {
+            const dim3 grid((unsigned)gx), block(kWave * kWavesPerBlock);
+#define LAUNCH_SLAB(L)                                                                                        \
+    hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, 8>), grid, block, 0, s, rowptr, idx, val, m, parent, perm, \
+                       X, Z, n, n_slabs, row_blocks, ldx, ldz)
+            if (lpe == 8) LAUNCH_SLAB(8);
+            else LAUNCH_SLAB(16);
+#undef LAUNCH_SLAB
+            return check_launch();
+        }
+    }
     const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
 #define LAUNCH(V, C, F)                                                                              \
     hipLaunchKernelGGL((spmm_wave_per_row<V, C, PACKED, F>), grid, block, 0, s, rowptr, idx, val, m, \
@@ -390,12 +573,35 @@ const char* cbm_status_string(int status) {
     }
 }
 
-int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const int32_t* parent,
-                 const int32_t* row_perm, const float* X, float* Z, int32_t n, int32_t d, int64_t ldx,
-                 int64_t ldz, void* stream) {
+int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
+                 const int32_t* parent, const int32_t* row_perm, const float* X, float* Z, int32_t n, int32_t d,
+                 int64_t ldx, int64_t ldz, void* stream) {
     if (!idx && n > 0) return CBM_ERR_NULL;
-    return launch_spmm<true>(rowptr, idx, nullptr, m, parent, row_perm, X, Z, n, d, ldx, ldz,
+    if (coef && !m) return CBM_ERR_NULL;                 // coef is the expansion of m, not a substitute
+    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_perm, X, Z, n, d, ldx, ldz,
                              static_cast<hipStream_t>(stream));
+}
+
+int cbm_set_spmm_kernel(int kind) {
+    if (kind < 0 || kind > 2) return CBM_ERR_SHAPE;
+    g_spmm_kernel = kind;
+    return CBM_OK;
+}
+
+int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
+    const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z);
+    return lpe ? kWave / lpe : 1;
+}
+
+int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_t nnz, void* stream) {
+    if (nnz < 0) return CBM_ERR_SHAPE;
+    if (nnz == 0) return CBM_OK;
+    if (!idx || !m || !coef) return CBM_ERR_NULL;
+    const int64_t blocks = (nnz + 255) / 256;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    hipLaunchKernelGGL(expand_coef, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), idx, m,
+                       coef, nnz);
+    return check_launch();
 }
 
 int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_perm,
@@ -418,13 +624,13 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
              : launch_propagate<false>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s);
 }
 
-int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const int32_t* parent,
-                        const int32_t* row_perm, const int32_t* order, const int32_t* level_off_dev,
+int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
+                        const int32_t* parent, const int32_t* row_perm, const int32_t* order, const int32_t* level_off_dev,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, int32_t n,
                         int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, m, parent, row_perm, X, Y, n, d, ldx, ldy, stream);
+    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_perm, X, Y, n, d, ldx, ldy, stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,

@@ -87,13 +87,31 @@ void cbm_format_free(cbm_format* f);
 const char* cbm_version(void);
 const char* cbm_status_string(int status);
 
-/* Z = D * diag(m) * X for the packed delta matrix D (m == NULL: Z = D * X).  If `parent` and `m`
- * are both given, rows with parent[r] < 0 are additionally scaled by m[r] (the first step of
- * the normalised tree walk, cbm_extensions.cpp:910-940, folded into the producer).  row_perm, if
- * not NULL, is a permutation of 0..N-1 giving the order in which rows are scheduled.
+/* Choice of the SpMM kernel for later calls of this process: 0 = automatic (default), 1 = always
+ * one wavefront per row, 2 = reserved (same as 0).  A tuning and test hook; no reference
+ * counterpart. */
+int cbm_set_spmm_kernel(int kind);
+
+/* How many interleaved partial sums the SpMM keeps per output element for this shape (1 = the
+ * entries of a row are accumulated strictly in order; g > 1 = entry k goes to partial sum
+ * k mod g and the g sums are added as a balanced tree).  Lets a checker reproduce the fp32
+ * summation order bit for bit.  No reference counterpart (MKL does not document its order). */
+int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
+
+/* coef[k] = +-m[column of entry k] for the packed entries idx[0 .. nnz): the delta VALUES of the
+ * reference's normalised builder (cbm_extensions.cpp:504-585), expanded on the device once so
+ * that cbm_spmm_f32 can stream them instead of gathering m[col] per entry.  Optional. */
+int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef_dev, int64_t nnz, void* stream);
+
+/* Z = D * diag(m) * X for the packed delta matrix D (m == NULL: Z = D * X).  coef, if not NULL,
+ * must be the output of cbm_expand_coef_f32 for (idx, m); the result is the same, the kernel
+ * streams coef instead of gathering m.  If `parent` and `m` are both given, rows with
+ * parent[r] < 0 are additionally scaled by m[r] (the first step of the normalised tree walk,
+ * cbm_extensions.cpp:910-940, folded into the producer).  row_perm, if not NULL, is a
+ * permutation of 0..N-1 giving the order in which rows are scheduled.
  * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
-int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
+int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
                  const int32_t* parent_dev, const int32_t* row_perm_dev, const float* X_dev, float* Z_dev,
                  int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
 
@@ -117,7 +135,8 @@ int cbm_propagate_f32(const int32_t* parent_dev, const int32_t* order_dev, const
  * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);
  * m != NULL replaces seq_/omp_s_fused_spmm_update_csr_int32_ (:845-996, :1224-1374). */
 int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
-                        const int32_t* parent_dev, const int32_t* row_perm_dev, const int32_t* order_dev,
+                        const float* coef_dev, const int32_t* parent_dev, const int32_t* row_perm_dev,
+                        const int32_t* order_dev,
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
                         const float* X_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
                         int32_t flags, void* stream);

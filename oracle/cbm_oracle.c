@@ -318,6 +318,36 @@ void oracle_csr_spmm(const int32_t* row_b, const int32_t* row_e, const int32_t* 
     }
 }
 
+/* Same product with the summation order of a SIMD kernel that deals the entries of a row to
+ * `groups` lanes round-robin: partial sum g takes entries k = g (mod groups) in order (FMA), and
+ * the partial sums are combined by a butterfly (xor 1, 2, 4, ...), i.e. a balanced binary tree.
+ * groups must be a power of two <= 64; groups == 1 is oracle_csr_spmm.  MKL's own order inside
+ * mkl_sparse_s_mm is not documented, so this is as valid a restatement of cpp:1149-1159 as the
+ * in-order one; it exists so that GPU results can be compared bit for bit. */
+void oracle_csr_spmm_grouped(const int32_t* row_b, const int32_t* row_e, const int32_t* col, const float* val,
+                             const float* X, float* Y, int32_t N, int32_t d, int32_t groups, int32_t threads) {
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 64) num_threads(threads > 0 ? threads : 1)
+#endif
+    for (int32_t r = 0; r < N; r++) {
+        float* y = Y + (size_t)r * d;
+        for (int32_t j = 0; j < d; j++) {
+            float part[64];
+            for (int32_t g = 0; g < groups; g++) part[g] = 0.0f;
+            for (int32_t k = row_b[r]; k < row_e[r]; k++) {
+                const int32_t g = (k - row_b[r]) % groups;
+                part[g] = fmaf(val ? val[k] : 1.0f, X[(size_t)col[k] * d + j], part[g]);
+            }
+            for (int32_t off = 1; off < groups; off <<= 1) {
+                float next[64];
+                for (int32_t g = 0; g < groups; g++) next[g] = part[g] + part[g ^ off];
+                for (int32_t g = 0; g < groups; g++) part[g] = next[g];
+            }
+            y[j] = part[0];
+        }
+    }
+}
+
 /* Tree walk, plain: Y[v,:] += Y[parent(v),:] top-down (cpp:713-738; omp :1166-1218).
  * mst_row has N+2 entries; the root's children are mst_col[mst_row[N] .. mst_row[N+1]). */
 void oracle_update_plain(const int32_t* mst_row, const int32_t* mst_col, float* Y, int32_t N, int32_t d,

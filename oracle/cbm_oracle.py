@@ -56,6 +56,8 @@ def lib():
         L.oracle_candidates.argtypes = [I32, P, P, I32, C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(I64)]
         L.oracle_csr_spmm.restype = None
         L.oracle_csr_spmm.argtypes = [P, P, P, P, P, P, I32, I32, I32]
+        L.oracle_csr_spmm_grouped.restype = None
+        L.oracle_csr_spmm_grouped.argtypes = [P, P, P, P, P, P, I32, I32, I32, I32]
         L.oracle_update_plain.restype = None
         L.oracle_update_plain.argtypes = [P, P, P, I32, I32, I32]
         L.oracle_update_fused.restype = None
@@ -145,15 +147,20 @@ def deltas_csr(fmt: dict, n: int, m=None):
     return np.cumsum(crow).astype(np.int32), col, val.astype(np.float32)
 
 
-def csr_spmm(crow, col, val, x, threads: int = 1):
-    """Y = A @ X, the role of ``mkl_sparse_s_mm`` (``cbm_extensions.cpp:1149-1159``)."""
+def csr_spmm(crow, col, val, x, threads: int = 1, groups: int = 1):
+    """Y = A @ X, the role of ``mkl_sparse_s_mm`` (``cbm_extensions.cpp:1149-1159``).
+    ``groups`` > 1 selects the round-robin partial-sum order of a SIMD kernel (see the C file)."""
     crow = np.ascontiguousarray(crow, np.int32); col = np.ascontiguousarray(col, np.int32)
     val = None if val is None else np.ascontiguousarray(val, np.float32)
     x = np.ascontiguousarray(x, np.float32)
     n = crow.shape[0] - 1
     y = np.empty((n, x.shape[1]), np.float32)
     rb = np.ascontiguousarray(crow[:-1]); re = np.ascontiguousarray(crow[1:])
-    lib().oracle_csr_spmm(_p(rb), _p(re), _p(col), _p(val), _p(x), _p(y), n, x.shape[1], threads)
+    if groups == 1:
+        lib().oracle_csr_spmm(_p(rb), _p(re), _p(col), _p(val), _p(x), _p(y), n, x.shape[1], threads)
+    else:
+        assert groups in (2, 4, 8, 16, 32, 64)
+        lib().oracle_csr_spmm_grouped(_p(rb), _p(re), _p(col), _p(val), _p(x), _p(y), n, x.shape[1], groups, threads)
     return y
 
 
@@ -174,10 +181,10 @@ def update_fused(mst_row, mst_col, m, y, threads: int = 1):
     return y
 
 
-def spmm_update(crow, col, val, mst_row, mst_col, x, m=None, threads: int = 1):
+def spmm_update(crow, col, val, mst_row, mst_col, x, m=None, threads: int = 1, groups: int = 1):
     """The whole reference multiply: ``*_s_spmm_update_csr_int32`` (m None) or
     ``*_s_fused_spmm_update_csr_int32`` (m given; val must already hold +-m[col])."""
-    y = csr_spmm(crow, col, val, x, threads)
+    y = csr_spmm(crow, col, val, x, threads, groups)
     return update_plain(mst_row, mst_col, y, threads) if m is None else update_fused(mst_row, mst_col, m, y, threads)
 
 

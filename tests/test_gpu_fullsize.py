@@ -46,7 +46,7 @@ def test_full_size_against_cpu_csr_and_gpu_csr(c3, orc):
     yd = torch.empty_like(xd)
     csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(ei[1][order].astype(np.int32)).cuda(),
              torch.from_numpy(vals).cuda(), xd, yd)
-    assert np.array_equal(yd.cpu().numpy(), cpu)
+    assert orc.max_rel_err(yd.cpu().numpy(), cpu) <= 1e-5
     # alpha = 16 prunes every candidate on this graph: flat tree, Delta == A
     assert mats[16].n_levels == 1 and mats[16].nnz == ei.shape[1]
     assert mats[0].n_levels > 1 and mats[0].nnz < ei.shape[1]

@@ -31,13 +31,31 @@ def _need_gpu():
     _lib.hip_lib()
 
 
-def oracle_product(orc, mat, ei, n, x, normalized, threads=4):
+def groups_for(d, ld=None):
+    """Partial sums per output element the SpMM keeps for contiguous, 16-byte aligned [*, d]
+    matrices (1 = strictly in order); the oracle reproduces that order bit for bit."""
+    ld = d if ld is None else ld
+    return int(_lib.hip_lib().cbm_spmm_summation_groups(d, ld, ld, C.c_void_p(256), C.c_void_p(256)))
+
+
+def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None):
     """Reference-style CPU multiply on the PRODUCT's tree (so both sides sum in the same order)."""
     col, sign = mat.columns()
     m = orc.col_multiplier(ei, n) if normalized else None
     val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
     return orc.spmm_update(mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32),
-                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads)
+                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads,
+                           groups=groups_for(x.shape[1]) if groups is None else groups)
+
+
+@pytest.fixture(params=["auto", "wave-per-row"])
+def spmm_kernel(request):
+    """Run a test once per SpMM kernel: automatic choice (slabs where the shape allows) and the
+    wave-per-row kernel forced."""
+    lib = _lib.hip_lib()
+    assert lib.cbm_set_spmm_kernel(1 if request.param == "wave-per-row" else 0) == 0
+    yield request.param
+    assert lib.cbm_set_spmm_kernel(0) == 0
 
 
 def gpu_product(mat, x, normalized):
@@ -65,22 +83,29 @@ def test_golden_integer_products_bit_exact(golden, case, alpha):
 # ---------------------------------------------------------------- oracle parity -----------
 @pytest.mark.parametrize("d", [1, 3, 10, 41, 64, 100, 128, 256, 258, 512, 602, 1000, 1028, 2052])
 @pytest.mark.parametrize("normalized", [False, True])
-def test_widths_against_oracle(orc, d, normalized):
+def test_widths_against_oracle(orc, d, normalized, spmm_kernel):
     n = 700
     ei = graphs.add_self_loops(graphs.sbm(n, 10, 0.3, 0.01, seed=d), n)
-    say("widths", d, normalized)
+    say("widths", d, normalized, spmm_kernel, "groups", groups_for(d))
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=normalized)
     assert mat.n_levels >= 2 and (mat.idx < 0).any()
+    if spmm_kernel == "auto" and d in (64, 128, 256, 512):
+        assert groups_for(d) > 1                           # these widths really take the slab kernel
     x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
     got = gpu_product(mat, x, normalized)
     want = oracle_product(orc, mat, ei, n, x, normalized)
     assert orc.max_rel_err(got, want) <= TOL_CBM
     assert np.array_equal(got, want)                       # same order, same FMAs: in fact bit-exact
+    assert orc.max_rel_err(got, oracle_product(orc, mat, ei, n, x, normalized, groups=1)) <= TOL_CBM
     assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CSR
+    if normalized:                                         # gathering m[col] instead of streaming +-m[col]
+        mat2 = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+        mat2.stream_coefficients = False
+        assert np.array_equal(gpu_product(mat2, x, True), got)
 
 
 @pytest.mark.parametrize("name,scale,alphas", [("c1", 1.0, (0,)), ("c2", 0.5, (0, 8)), ("c3", 0.05, (0, 16))])
-def test_workloads_against_oracle(orc, name, scale, alphas):
+def test_workloads_against_oracle(orc, name, scale, alphas, spmm_kernel):
     w = graphs.workload(name, scale=scale)
     x = w.features(0).numpy()
     for alpha in alphas:
@@ -104,7 +129,9 @@ def test_workloads_against_oracle(orc, name, scale, alphas):
         yd = torch.empty((w.n, x.shape[1]), device="cuda")
         csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(ei[1][order].astype(np.int32)).cuda(),
                  None if vals is None else torch.from_numpy(vals).cuda(), torch.from_numpy(x).cuda(), yd)
-        assert np.array_equal(yd.cpu().numpy(), csr)       # same in-order FMA chain as the oracle
+        assert orc.max_rel_err(yd.cpu().numpy(), csr) <= 1e-5
+        g = groups_for(x.shape[1])
+        assert np.array_equal(yd.cpu().numpy(), csr if g == 1 else orc.csr_spmm(rp, ei[1][order], vals, x, threads=4, groups=g))
 
 
 def test_reference_test_matmul_correctness(orc):
@@ -138,7 +165,7 @@ def test_update_only_entry_points(orc):
         col, sign = mat.columns()
         m = orc.col_multiplier(ei, n) if normalized else None
         val = (sign.numpy() * (m[col.numpy()] if normalized else 1)).astype(np.float32)
-        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x)
+        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=groups_for(d))
         assert np.array_equal(z.cpu().numpy(), z_ref)
         # update alone on that Z == the oracle's walk (plain or fused) on the same Z
         y = z.clone()
@@ -185,6 +212,15 @@ def test_strided_rows_and_cpu_staging(orc):
     mat.omp_mkl_csr_spmm_update(xbig[:, :d], ybig[:, :d])        # ld = d+5 / d+9, unaligned for float4
     assert np.array_equal(ybig[:, :d].cpu().numpy(), want)
     assert (ybig[:, d:] == 7.0).all()                            # nothing written beyond the d columns
+    say("strided, slab kernel")                                 # d = 64 with ld = 68 / 72: float4-addressable
+    d2 = 64
+    x2 = np.random.default_rng(3).standard_normal((n, d2)).astype(np.float32)
+    want2 = oracle_product(orc, mat, ei, n, x2, False, groups=groups_for(d2, 68))
+    xbig = torch.zeros((n, 68), device="cuda"); xbig[:, :d2] = torch.from_numpy(x2).cuda()
+    ybig = torch.full((n, 72), 7.0, device="cuda")
+    mat.omp_mkl_csr_spmm_update(xbig[:, :d2], ybig[:, :d2])
+    assert np.array_equal(ybig[:, :d2].cpu().numpy(), want2)
+    assert (ybig[:, d2:] == 7.0).all()
     say("cpu staging")
     y = torch.empty(n, d)
     mat.omp_mkl_csr_spmm_update(torch.from_numpy(x), y)
@@ -251,14 +287,15 @@ def test_c_abi_status_codes_on_device_calls():
     rp = torch.zeros(n + 1, dtype=torch.int32, device="cuda"); idx = torch.zeros(1, dtype=torch.int32, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
     say("status codes")
-    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, p(x), p(y), n, d, d, d, None) == 1
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, p(x), p(y), n, d, d - 1, d, None) == 3
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, p(x), p(y), n, d, d, d, None) == 0   # empty rows -> zeros
+    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), n, d, d, d, None) == 1
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), n, d, d - 1, d, None) == 3
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), n, d, d, d, None) == 1   # coef without m
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), n, d, d, d, None) == 0   # empty rows -> zeros
     lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
     par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
     lo = (C.c_int32 * 2)(0, n)
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 0
-    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), n, d, d, d, 0, None) == 3
+    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), n, d, d, d, 0, None) == 3
     torch.cuda.synchronize()
     assert (y == 0).all()
