@@ -32,7 +32,7 @@ from . import _lib
 
 warnings.filterwarnings("ignore", message="Sparse CSR tensor support is in beta state", category=UserWarning)
 
-__all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels"]
+__all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels", "schedule_rows"]
 
 
 def _ptr(t):
@@ -68,6 +68,19 @@ def _check_f32_matrix(t, name, n=None):
 
 def _ld(t):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
+
+
+def schedule_rows(rowptr, parent=None, m=None):
+    """Row schedule of the SpMM kernels (``cbm_schedule_rows``): int32 tensor [n, 4] holding
+    {start, end, row, bits(left scale)} per row, longest rows first."""
+    rowptr = rowptr.to("cpu", torch.int32).contiguous()
+    n = rowptr.numel() - 1
+    parent = None if parent is None else parent.to("cpu", torch.int32).contiguous()
+    m = None if m is None else m.to("cpu", torch.float32).contiguous()
+    out = torch.empty((n, 4), dtype=torch.int32)
+    rc = _lib.host_lib().cbm_schedule_rows(_ptr(rowptr), _ptr(parent), _ptr(m), n, _ptr(out))
+    _lib.check(rc, "cbm_schedule_rows")
+    return out
 
 
 def tree_levels(mst_row: np.ndarray, mst_col: np.ndarray):
@@ -249,6 +262,10 @@ class cbm_matrix:
                 "order": self.order.to(device), "level_off": self.level_off.to(device),
                 "m": self.col_multiplier.to(device) if self.col_multiplier is not None else None,
                 "coef": None,
+                # row schedules (longest rows first): without and with the left scale of root children
+                "sched": schedule_rows(self.rowptr, None, None).to(device),
+                "sched_scaled": (schedule_rows(self.rowptr, self.parent, self.col_multiplier).to(device)
+                                 if self.col_multiplier is not None else None),
             }
             if st["m"] is not None and self.nnz and self.stream_coefficients:
                 # +-m[col] per delta entry, expanded once on the device (what the reference keeps
@@ -293,7 +310,8 @@ class cbm_matrix:
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None,
-                _ptr(st["parent"]) if scale_roots else None, None, _ptr(xd), _ptr(yd),
+                _ptr(st["parent"]) if scale_roots else None,
+                _ptr(st["sched_scaled"] if (scale_roots and use_m) else st["sched"]), _ptr(xd), _ptr(yd),
                 n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
         _lib.check(rc, "cbm_spmm_f32")
         if yd is not y:
@@ -338,7 +356,7 @@ class cbm_matrix:
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None, _ptr(st["parent"]),
-                None, _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
+                _ptr(st["sched_scaled"] if use_m else st["sched"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
                 _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
         _lib.check(rc, "cbm_spmm_update_f32")
         if yd is not y:
@@ -442,10 +460,11 @@ class CBMMatmul(torch.autograd.Function):
         return gx, None, None
 
 
-def csr_spmm(rowptr, col, val, x, y):
+def csr_spmm(rowptr, col, val, x, y, sched=None):
     """Plain CSR SpMM ``y = A @ x`` on the GPU: the hand-written baseline the CBM multiply is
     measured against (role of ``omp_s_spmm_csr_int32``, ``cbm_extensions.cpp:1707-1755``).
-    ``rowptr`` [N+1] / ``col`` int32 device tensors, ``val`` fp32 or None (all ones)."""
+    ``rowptr`` [N+1] / ``col`` int32 device tensors, ``val`` fp32 or None (all ones); ``sched``:
+    optional device copy of ``schedule_rows(rowptr)`` (same scheduling as the CBM kernels)."""
     n = rowptr.numel() - 1
     _check_f32_matrix(x, "rhs")
     _check_f32_matrix(y, "dst", n)
@@ -456,6 +475,6 @@ def csr_spmm(rowptr, col, val, x, y):
     if not (x.is_cuda and y.is_cuda and rowptr.is_cuda and col.is_cuda):
         raise ValueError("csr_spmm expects device tensors")
     with torch.cuda.device(x.device):
-        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), None, _ptr(x), _ptr(y),
+        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), _ptr(sched), _ptr(x), _ptr(y),
                                          n, x.size(1), _ld(x), _ld(y), _stream(x.device))
     _lib.check(rc, "csr_spmm_f32")

@@ -181,6 +181,35 @@ void cbm_format_free(cbm_format* f) {
     std::memset(f, 0, sizeof(*f));
 }
 
+int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
+                      int32_t* sched_out) {
+    if (!rowptr || !sched_out) return CBM_ERR_NULL;
+    if (n < 0) return CBM_ERR_SHAPE;
+    try {
+        // counting sort by gather rounds (64 entries each), longest first, stable
+        std::vector<int32_t> rounds(n);
+        int32_t max_rounds = 0;
+        for (int32_t r = 0; r < n; r++) {
+            const int32_t len = rowptr[r + 1] - rowptr[r];
+            if (len < 0) return CBM_ERR_SHAPE;
+            rounds[r] = (len + 63) / 64;
+            max_rounds = std::max(max_rounds, rounds[r]);
+        }
+        std::vector<int64_t> first(max_rounds + 2, 0);
+        for (int32_t r = 0; r < n; r++) first[max_rounds - rounds[r] + 1]++;
+        for (int32_t b = 0; b <= max_rounds; b++) first[b + 1] += first[b];
+        for (int32_t r = 0; r < n; r++) {
+            int32_t* o = sched_out + 4 * first[max_rounds - rounds[r]]++;
+            const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
+            o[0] = rowptr[r]; o[1] = rowptr[r + 1]; o[2] = r;
+            std::memcpy(&o[3], &scale, sizeof(float));
+        }
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        return CBM_ERR_ALLOC;
+    }
+}
+
 int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t alpha,
                    int32_t threads, cbm_format* out) {
     if (!out) return CBM_ERR_NULL;

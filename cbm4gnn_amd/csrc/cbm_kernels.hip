@@ -96,27 +96,34 @@ __device__ __forceinline__ float bcast_f(float v, int lane) {
 template <int VEC, int CH, bool PACKED, bool FULL>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
     const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
-    const float* __restrict__ m, const int32_t* __restrict__ parent, const int32_t* __restrict__ perm,
+    const float* __restrict__ m, const int32_t* __restrict__ parent, const int4* __restrict__ sched,
     const float* __restrict__ X, float* __restrict__ Z, int n, int d, int64_t ldx, int64_t ldz) {
     constexpr int U = (CH == 1) ? CBM_UNROLL_CH1 : (CH == 2 ? CBM_UNROLL_CH1 / 2 : CBM_UNROLL_CH1 / 4);   // X-row loads in flight per wave
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     int row = xcd_contiguous_block(blockIdx.x, gridDim.x) * kWavesPerBlock + wave;
     if (row >= n) return;
-    if (perm) row = perm[row];
-    row = __builtin_amdgcn_readfirstlane(row);
-    const int start = __builtin_amdgcn_readfirstlane(rowptr[row]);
-    const int end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
-    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
-    // left scaling of root children: fetched up front so the loads overlap the gather
-    float root_scale = 1.0f;
-    if constexpr (PACKED) {
-        if (m && parent) {
-            const int par = parent[row];
-            const float mr = m[row];
-            root_scale = par < 0 ? mr : 1.0f;
+    int start, end;
+    float root_scale = 1.0f;                   // left scaling of root children, fetched up front
+    if (sched) {
+        const int4 r = sched[row];
+        start = __builtin_amdgcn_readfirstlane(r.x);
+        end = __builtin_amdgcn_readfirstlane(r.y);
+        row = __builtin_amdgcn_readfirstlane(r.z);
+        root_scale = __int_as_float(__builtin_amdgcn_readfirstlane(r.w));
+    } else {
+        row = __builtin_amdgcn_readfirstlane(row);
+        start = __builtin_amdgcn_readfirstlane(rowptr[row]);
+        end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
+        if constexpr (PACKED) {
+            if (m && parent) {
+                const int par = parent[row];
+                const float mr = m[row];
+                root_scale = par < 0 ? mr : 1.0f;
+            }
         }
     }
+    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
 
     float acc[CH][VEC];
 #pragma unroll
@@ -212,92 +219,100 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
 // ---------------------------------------------------------------------------------------------
 template <int LPE, bool PACKED, int U>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
-    const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
-    const float* __restrict__ m, const int32_t* __restrict__ parent, const int32_t* __restrict__ perm,
-    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int row_blocks, int64_t ldx,
-    int64_t ldz) {
+    const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
+    const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
+    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int64_t ldx, int64_t ldz) {
     constexpr int kSlab = LPE * 4;                         // floats per slab
     constexpr int kStep = kWave / LPE;                     // entries per wave instruction
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
     const int sub = lane / LPE;                            // which entry of a step
     const int li = lane % LPE;                             // float4 position inside the slab
-    // workgroup b runs on XCD b % 8.  n_slabs >= 8 (a multiple of 8): XCD x owns slabs x, x + 8, ...
-    // and finishes all row blocks of one slab before it starts the next, so one slab at a time
-    // competes for its L2;  n_slabs < 8 (a divisor of 8): 8 / n_slabs XCDs share a slab and split
-    // its row blocks.
-    int slab, rb;
+    // Persistent waves.  Workgroup b runs on XCD b % 8; G workgroups per XCD.
+    //   n_slabs >= 8 (a multiple of 8): XCD x walks slabs x, x + 8, ... one after the other, its
+    //     4 G waves sharing the rows of the current slab cyclically;
+    //   n_slabs < 8 (a divisor of 8): the 8 / n_slabs XCDs of a slab share its rows cyclically.
+    // Rows come in schedule order (longest first), so a cyclic deal gives every wave the same mix.
+    const int xcd = blockIdx.x % kXcds;
+    const int G = gridDim.x / kXcds;
+    int first, stride, slab0, slab_step;
     {
-        const int b = blockIdx.x;
-        const int x = b % kXcds, j = b / kXcds;
+        const int j = blockIdx.x / kXcds;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
         if (n_slabs >= kXcds) {
-            slab = x + kXcds * (j / row_blocks);
-            rb = j % row_blocks;
+            first = j * kWavesPerBlock + wave; stride = G * kWavesPerBlock; slab0 = xcd; slab_step = kXcds;
         } else {
             const int share = kXcds / n_slabs;
-            slab = x % n_slabs;
-            rb = j * share + x / n_slabs;
+            first = ((xcd / n_slabs) * G + j) * kWavesPerBlock + wave; stride = share * G * kWavesPerBlock;
+            slab0 = xcd % n_slabs; slab_step = n_slabs;      // a single slab for this XCD
         }
     }
-    if (rb >= row_blocks) return;
-    int row = rb * kWavesPerBlock + wave;
-    if (row >= n) return;
-    if (perm) row = perm[row];
-    row = __builtin_amdgcn_readfirstlane(row);
-    const int start = __builtin_amdgcn_readfirstlane(rowptr[row]);
-    const int end = __builtin_amdgcn_readfirstlane(rowptr[row + 1]);
-    const float* __restrict__ Xs = X + slab * kSlab + li * 4;
-    // left scaling of root children: fetched up front so the loads overlap the gather
-    float root_scale = 1.0f;
-    if constexpr (PACKED) {
-        if (m && parent) {
-            const int par = parent[row];
-            const float mr = m[row];
-            root_scale = par < 0 ? mr : 1.0f;
-        }
-    }
+    for (int slab = slab0; slab < n_slabs; slab += slab_step) {
+        const float* __restrict__ Xs = X + slab * kSlab + li * 4;
+        float* __restrict__ Zs = Z + slab * kSlab + li * 4;
+        // row descriptor {start, end, row, bits(left scale)} fetched one row ahead of its use
+        auto fetch = [&](int i) -> int4 {
+            if (sched) return sched[i];
+            int4 r;
+            r.x = rowptr[i]; r.y = rowptr[i + 1]; r.z = i; r.w = 0x3f800000;
+            if constexpr (PACKED) {
+                if (m && parent) r.w = parent[i] < 0 ? __float_as_int(m[i]) : 0x3f800000;
+            }
+            return r;
+        };
+        int i = first;
+        int4 nxt = make_int4(0, 0, 0, 0);
+        if (i < n) nxt = fetch(i);
+        while (i < n) {
+            const int start = __builtin_amdgcn_readfirstlane(nxt.x);
+            const int end = __builtin_amdgcn_readfirstlane(nxt.y);
+            const int row = __builtin_amdgcn_readfirstlane(nxt.z);
+            const float row_scale = __int_as_float(__builtin_amdgcn_readfirstlane(nxt.w));
+            i += stride;
+            if (i < n) nxt = fetch(i);
 
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int pos = start; pos < end; pos += kStep * U) {
-        float x[U][4];
-        float f[U];
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int pos = start; pos < end; pos += kStep * U) {
+                float x[U][4];
+                float f[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int k = pos + u * kStep + sub;
-            f[u] = 0.0f;
+                for (int u = 0; u < U; u++) {
+                    const int k = pos + u * kStep + sub;
+                    f[u] = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) x[u][e] = 0.0f;
-            if (k < end) {
-                const uint32_t p = idx[k];
-                const uint32_t c = PACKED ? (p & 0x7fffffffu) : p;
-                if constexpr (PACKED) {
-                    if (val) f[u] = val[k];                // streamed +-m[col]
-                    else {
-                        const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
-                        f[u] = __uint_as_float(mag ^ (p & 0x80000000u));
+                    for (int e = 0; e < 4; e++) x[u][e] = 0.0f;
+                    if (k < end) {
+                        const uint32_t p = idx[k];
+                        const uint32_t c = PACKED ? (p & 0x7fffffffu) : p;
+                        if constexpr (PACKED) {
+                            if (val) f[u] = val[k];        // streamed +-m[col]
+                            else {
+                                const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
+                                f[u] = __uint_as_float(mag ^ (p & 0x80000000u));
+                            }
+                        } else {
+                            f[u] = val ? val[k] : 1.0f;
+                        }
+                        load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
                     }
-                } else {
-                    f[u] = val ? val[k] : 1.0f;
                 }
-                load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
+#pragma unroll
+                for (int u = 0; u < U; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[e] = fmaf(f[u], x[u][e], acc[e]);
+            }
+#pragma unroll
+            for (int off = LPE; off < kWave; off <<= 1)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
+            if (sub == 0) {
+                if constexpr (PACKED) {
+                    if (m && parent)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[e] *= row_scale;
+                }
+                store_vec<4>(Zs + (int64_t)row * ldz, acc);
             }
         }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[e] = fmaf(f[u], x[u][e], acc[e]);
-    }
-#pragma unroll
-    for (int off = LPE; off < kWave; off <<= 1)
-#pragma unroll
-        for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
-    if (sub == 0) {
-        if constexpr (PACKED) {
-            if (m && parent)
-#pragma unroll
-                for (int e = 0; e < 4; e++) acc[e] *= root_scale;
-        }
-        store_vec<4>(Z + (int64_t)row * ldz + slab * kSlab + li * 4, acc);
     }
 }
 
@@ -468,36 +483,52 @@ inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
     return CBM_OK;
 }
 
+// Workgroups per XCD of the persistent slab kernel: as many as are resident at once.
+template <class K>
+int resident_groups_per_xcd(K kernel) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kWave * kWavesPerBlock, 0) != hipSuccess) return 0;
+    if (cus < kXcds || per_cu < 1) return 0;
+    return (cus / kXcds) * per_cu;
+}
+
 template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, const float* m,
-                const int32_t* parent, const int32_t* perm, const float* X, float* Z, int32_t n, int32_t d,
+                const int32_t* parent, const int32_t* sched, const float* X, float* Z, int32_t n, int32_t d,
                 int64_t ldx, int64_t ldz, hipStream_t s) {
-    if (!rowptr || !X || !Z) return CBM_ERR_NULL;
+    if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
+    if (sched && !aligned(sched, 16)) return CBM_ERR_SHAPE;
     if (n == 0 || d == 0) return CBM_OK;
-    const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
+    const int4* sc = reinterpret_cast<const int4*>(sched);
     if (const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z)) {
         const int n_slabs = d / (lpe * 4);
-        const int row_blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
-        int64_t gx;
-        if (n_slabs >= kXcds) gx = (int64_t)row_blocks * n_slabs;
-        else { const int share = kXcds / n_slabs; gx = (int64_t)((row_blocks + share - 1) / share) * kXcds; }
-        if (gx <= INT32_MAX) {
-            const dim3 grid((unsigned)gx), block(kWave * kWavesPerBlock);
-#define LAUNCH_SLAB(L)                                                                                        \
-    hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, 8>), grid, block, 0, s, rowptr, idx, val, m, parent, perm, \
-                       X, Z, n, n_slabs, row_blocks, ldx, ldz)
-            if (lpe == 8) LAUNCH_SLAB(8);
-            else LAUNCH_SLAB(16);
-#undef LAUNCH_SLAB
+        static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, 8>);
+        static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, 8>);
+        int G = lpe == 8 ? g8 : g16;
+        if (G > 0) {
+            // no more waves than rows: with fewer rows than resident waves shrink the grid
+            const int share = n_slabs >= kXcds ? 1 : kXcds / n_slabs;
+            const int need = (n + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
+            if (G > need) G = need;
+            const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
+            if (lpe == 8)
+                hipLaunchKernelGGL((spmm_slab_per_xcd<8, PACKED, 8>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
+                                   X, Z, n, n_slabs, ldx, ldz);
+            else
+                hipLaunchKernelGGL((spmm_slab_per_xcd<16, PACKED, 8>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
+                                   X, Z, n, n_slabs, ldx, ldz);
             return check_launch();
         }
     }
+    const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
     const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
 #define LAUNCH(V, C, F)                                                                              \
     hipLaunchKernelGGL((spmm_wave_per_row<V, C, PACKED, F>), grid, block, 0, s, rowptr, idx, val, m, \
-                       parent, perm, X, Z, n, d, ldx, ldz)
+                       parent, sc, X, Z, n, d, ldx, ldz)
     CBM_DISPATCH_TILING(t, LAUNCH);
 #undef LAUNCH
     return check_launch();
@@ -574,11 +605,11 @@ const char* cbm_status_string(int status) {
 }
 
 int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
-                 const int32_t* parent, const int32_t* row_perm, const float* X, float* Z, int32_t n, int32_t d,
+                 const int32_t* parent, const int32_t* row_sched, const float* X, float* Z, int32_t n, int32_t d,
                  int64_t ldx, int64_t ldz, void* stream) {
     if (!idx && n > 0) return CBM_ERR_NULL;
     if (coef && !m) return CBM_ERR_NULL;                 // coef is the expansion of m, not a substitute
-    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_perm, X, Z, n, d, ldx, ldz,
+    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, n, d, ldx, ldz,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -604,10 +635,10 @@ int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_
     return check_launch();
 }
 
-int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_perm,
+int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_sched,
                  const float* X, float* Y, int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream) {
     if (!col && n > 0) return CBM_ERR_NULL;
-    return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_perm,
+    return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_sched,
                               X, Y, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
 }
 
@@ -625,12 +656,12 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
 }
 
 int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
-                        const int32_t* parent, const int32_t* row_perm, const int32_t* order, const int32_t* level_off_dev,
+                        const int32_t* parent, const int32_t* row_sched, const int32_t* order, const int32_t* level_off_dev,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, int32_t n,
                         int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_perm, X, Y, n, d, ldx, ldy, stream);
+    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, n, d, ldx, ldy, stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,

@@ -82,6 +82,16 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t n_edges, int3
 
 void cbm_format_free(cbm_format* f);
 
+/* Row schedule for the SpMM kernels: rows sorted by descending number of 64-entry gather rounds
+ * (stable, so rows of similar length keep their natural order), one descriptor of 4 int32 per
+ * row: { rowptr[r], rowptr[r + 1], r, bit pattern of the left scale }.  The left scale is m[r]
+ * for children of the root (parent[r] < 0) when m is given, 1.0f otherwise.  Long rows start
+ * first and a cyclic deal of the schedule gives every wavefront the same mix of row lengths.
+ * HOST pointers; sched_out holds 4 * n int32.  parent and m may be NULL (scale 1.0f).
+ * No reference counterpart: MKL keeps its own scheduling inside mkl_sparse_s_mm. */
+int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
+                      int32_t* sched_out);
+
 /* ------------------------------------------------------------------ libcbm_hip.so ----------- */
 
 const char* cbm_version(void);
@@ -107,12 +117,13 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * must be the output of cbm_expand_coef_f32 for (idx, m); the result is the same, the kernel
  * streams coef instead of gathering m.  If `parent` and `m` are both given, rows with
  * parent[r] < 0 are additionally scaled by m[r] (the first step of the normalised tree walk,
- * cbm_extensions.cpp:910-940, folded into the producer).  row_perm, if not NULL, is a
- * permutation of 0..N-1 giving the order in which rows are scheduled.
+ * cbm_extensions.cpp:910-940, folded into the producer).  row_sched, if not NULL, is the row
+ * schedule written by cbm_schedule_rows (4 int32 per row, 16-byte aligned): rows are then
+ * processed in that order, rowptr is not read (may be NULL) and the left scale comes from it.
  * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
 int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
-                 const int32_t* parent_dev, const int32_t* row_perm_dev, const float* X_dev, float* Z_dev,
+                 const int32_t* parent_dev, const int32_t* row_sched_dev, const float* X_dev, float* Z_dev,
                  int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
@@ -135,7 +146,7 @@ int cbm_propagate_f32(const int32_t* parent_dev, const int32_t* order_dev, const
  * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);
  * m != NULL replaces seq_/omp_s_fused_spmm_update_csr_int32_ (:845-996, :1224-1374). */
 int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
-                        const float* coef_dev, const int32_t* parent_dev, const int32_t* row_perm_dev,
+                        const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
                         const int32_t* order_dev,
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
                         const float* X_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
@@ -144,7 +155,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, cons
 /* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
 int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, const float* val_dev,
-                 const int32_t* row_perm_dev, const float* X_dev, float* Y_dev, int32_t n, int32_t d,
+                 const int32_t* row_sched_dev, const float* X_dev, float* Y_dev, int32_t n, int32_t d,
                  int64_t ldx, int64_t ldy, void* stream);
 
 #ifdef __cplusplus
