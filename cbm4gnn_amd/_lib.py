@@ -39,6 +39,7 @@ HOST_SYMBOLS = {
     "cbm_host_version": (C.c_char_p, []),
     "cbm_build_host": (C.c_int, [_P, _P, _I64, _I32, _I32, _I32, C.POINTER(CbmFormat)]),
     "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
+    "cbm_build_host_timings": (None, [C.POINTER(C.c_double)]),
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
 }
 HIP_SYMBOLS = {

@@ -147,6 +147,9 @@ class cbm_matrix:
                                             ei_cpu.size(1), n, self.alpha, int(threads), C.byref(fmt))
         try:
             _lib.check(rc, "cbm_build_host")
+            t4 = (C.c_double * 4)()
+            _lib.host_lib().cbm_build_host_timings(t4)
+            self.build_seconds = dict(zip(("csr", "candidates", "arborescence", "deltas"), list(t4)))
 
             def take(ptr, count, dtype):
                 return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))

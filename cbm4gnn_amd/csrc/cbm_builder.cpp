@@ -40,35 +40,37 @@ struct CandEdge { int32_t u, v, w; };
 // ---------------------------------------------------------------------------------------------
 class Arborescence {
 public:
-    Arborescence(int32_t n, const std::vector<CandEdge>& edges)
-        : n_(n), edges_(edges), key_(edges.size()), lazy_(edges.size(), 0), lc_(edges.size(), -1),
-          rc_(edges.size(), -1), rank_(edges.size(), 1), heap_(n, -1), uf_(n, -1) {}
+    Arborescence(int32_t n, const std::vector<CandEdge>& edges, int threads)
+        : n_(n), threads_(threads), edges_(edges), node_(edges.size()), heap_(n, -1), uf_(n, -1) {}
 
     // Returns total weight; par[v] = tail of the edge entering v (par[root] = -1).
     int64_t run(int32_t root, std::vector<int32_t>& par) {
         const int64_t m = (int64_t)edges_.size();
-        for (int64_t e = 0; e < m; e++) key_[e] = edges_[e].w;
-        // bulk-build one heap per head node: gather ids per node, then pairwise meld
+        // One heap per head node, built without a single meld: the node's incoming edges sorted
+        // by (weight, id) and chained through the LEFT child is a valid leftist heap (every right
+        // child is empty), and the sorts run in parallel.
         {
             std::vector<int64_t> cnt(n_ + 1, 0);
             for (int64_t e = 0; e < m; e++) cnt[edges_[e].v + 1]++;
             for (int32_t v = 0; v < n_; v++) cnt[v + 1] += cnt[v];
             std::vector<int32_t> ids(m);
-            std::vector<int64_t> fill(cnt.begin(), cnt.end() - 1);
-            for (int64_t e = 0; e < m; e++) ids[fill[edges_[e].v]++] = (int32_t)e;
-            std::vector<int32_t> q;
+            {
+                std::vector<int64_t> fill(cnt.begin(), cnt.end() - 1);
+                for (int64_t e = 0; e < m; e++) ids[fill[edges_[e].v]++] = (int32_t)e;
+            }
+#pragma omp parallel for schedule(dynamic, 64) num_threads(threads_)
             for (int32_t v = 0; v < n_; v++) {
-                int64_t b = cnt[v], e = cnt[v + 1];
+                const int64_t b = cnt[v], e = cnt[v + 1];
                 if (b == e) continue;
-                q.assign(ids.begin() + b, ids.begin() + e);
-                size_t len = q.size();
-                while (len > 1) {                      // rounds of pairwise melds: O(len) total
-                    size_t o = 0;
-                    for (size_t i = 0; i + 1 < len; i += 2) q[o++] = meld(q[i], q[i + 1]);
-                    if (len & 1) q[o++] = q[len - 1];
-                    len = o;
+                std::sort(ids.begin() + b, ids.begin() + e, [&](int32_t x, int32_t y) {
+                    return edges_[x].w != edges_[y].w ? edges_[x].w < edges_[y].w : x < y;
+                });
+                for (int64_t k = b; k < e; k++) {
+                    Node& nd = node_[ids[k]];
+                    nd.key = edges_[ids[k]].w; nd.lazy = 0;
+                    nd.lc = k + 1 < e ? ids[k + 1] : -1; nd.rc = -1; nd.rank = 1;
                 }
-                heap_[v] = q[0];
+                heap_[v] = ids[b];
             }
         }
         std::vector<int32_t> seen(n_, -1), path(n_), Q(n_), in(n_, -1);
@@ -84,9 +86,9 @@ public:
                 if (h < 0) return -1;                   // node not reachable from the root
                 push_down(h);
                 const int32_t e = h;
-                const int32_t w = key_[e];
-                heap_[u] = meld(lc_[e], rc_[e]);         // pop
-                if (heap_[u] >= 0) lazy_[heap_[u]] -= w;  // remaining keys become reduced costs
+                const int32_t w = node_[e].key;
+                heap_[u] = meld(node_[e].lc, node_[e].rc);            // pop
+                if (heap_[u] >= 0) node_[heap_[u]].lazy -= w;        // remaining keys become reduced costs
                 Q[qi] = e; path[qi++] = u; seen[u] = s;
                 res += w;
                 u = find(edges_[e].u);
@@ -116,21 +118,23 @@ public:
     }
 
 private:
+    struct Node { int32_t key, lazy, lc, rc; int32_t rank; };   // one cache line holds three
     int32_t n_;
+    int threads_;
     const std::vector<CandEdge>& edges_;
-    std::vector<int32_t> key_, lazy_, lc_, rc_;
-    std::vector<uint8_t> rank_;
+    std::vector<Node> node_;                                   // index = edge id
     std::vector<int32_t> heap_;
     std::vector<int32_t> uf_;                                  // <0: -size, else parent
     std::vector<std::pair<int32_t, int32_t>> hist_;
 
     void push_down(int32_t a) {
-        const int32_t z = lazy_[a];
+        Node& nd = node_[a];
+        const int32_t z = nd.lazy;
         if (z) {
-            key_[a] += z;
-            if (lc_[a] >= 0) lazy_[lc_[a]] += z;
-            if (rc_[a] >= 0) lazy_[rc_[a]] += z;
-            lazy_[a] = 0;
+            nd.key += z;
+            if (nd.lc >= 0) node_[nd.lc].lazy += z;
+            if (nd.rc >= 0) node_[nd.rc].lazy += z;
+            nd.lazy = 0;
         }
     }
     // Leftist heap meld; the right spine is O(log size) so the recursion is shallow.  Ties are
@@ -139,11 +143,12 @@ private:
         if (a < 0) return b;
         if (b < 0) return a;
         push_down(a); push_down(b);
-        if (key_[a] > key_[b] || (key_[a] == key_[b] && a > b)) std::swap(a, b);
-        rc_[a] = meld(rc_[a], b);
-        const uint8_t rl = lc_[a] >= 0 ? rank_[lc_[a]] : 0, rr = rank_[rc_[a]];
-        if (rl < rr) std::swap(lc_[a], rc_[a]);
-        rank_[a] = (uint8_t)((rc_[a] >= 0 ? rank_[rc_[a]] : 0) + 1);
+        if (node_[a].key > node_[b].key || (node_[a].key == node_[b].key && a > b)) std::swap(a, b);
+        Node& na = node_[a];
+        na.rc = meld(na.rc, b);
+        const int32_t rl = na.lc >= 0 ? node_[na.lc].rank : 0, rr = node_[na.rc].rank;
+        if (rl < rr) std::swap(na.lc, na.rc);
+        na.rank = (na.rc >= 0 ? node_[na.rc].rank : 0) + 1;
         return a;
     }
     int32_t find(int32_t x) const { while (uf_[x] >= 0) x = uf_[x]; return x; }
@@ -170,7 +175,15 @@ template <class T> T* dup_array(const std::vector<T>& v) {
 
 }  // namespace
 
+// seconds spent by the last cbm_build_host call of this thread in: CSR + transpose, candidate
+// edges, arborescence, tree arrays + deltas
+thread_local double g_last_timings[4] = {0, 0, 0, 0};
+
 extern "C" {
+
+void cbm_build_host_timings(double* out4) {
+    if (out4) for (int i = 0; i < 4; i++) out4[i] = g_last_timings[i];
+}
 
 const char* cbm_host_version(void) { return "cbm4gnn_amd host builder 0.1"; }
 
@@ -217,6 +230,8 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
     if ((!row || !col) && E > 0) return CBM_ERR_NULL;
     if (N <= 0 || E < 0 || N >= (1 << 30)) return CBM_ERR_SHAPE;
     if (threads <= 0) threads = omp_get_max_threads();
+    double t_mark = omp_get_wtime();
+    auto lap = [&](int slot) { const double t = omp_get_wtime(); g_last_timings[slot] = t - t_mark; t_mark = t; };
     try {
         // ---- COO -> CSR(A) with sorted unique columns, and its transpose -----------------------
         std::vector<int64_t> rp(N + 1, 0);
@@ -259,6 +274,7 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
                 for (int64_t k = rp[r]; k < rp[r + 1]; k++) tr[fill[ci[k]]++] = r;   // ascending r per column
         }
 
+        lap(0);
         // ---- candidate edges (reference rule, cpp:75-103), streamed and pruned ------------------
         // pair (i, j>i) with s shared columns: h = nnz_i + nnz_j - 2s;
         //   j -> i admitted iff h < nnz_i - alpha  <=>  2s > nnz_j + alpha
@@ -313,17 +329,19 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
         }
         if (cand.size() >= (size_t)INT32_MAX) return CBM_ERR_SHAPE;
 
+        lap(1);
         // ---- arborescence ----------------------------------------------------------------------
         std::vector<int32_t> par;
         int64_t weight;
         {
-            Arborescence msa(N + 1, cand);
+            Arborescence msa(N + 1, cand, threads);
             weight = msa.run(N, par);
         }
         if (weight < 0) return CBM_ERR_INTERNAL;
         const int64_t n_cand = (int64_t)cand.size();
         std::vector<CandEdge>().swap(cand);
 
+        lap(2);
         // ---- tree arrays: children ascending per parent; levels by BFS --------------------------
         std::vector<int32_t> mst_row(N + 2, 0), mst_col(N);
         for (int32_t v = 0; v < N; v++) mst_row[par[v] + 1]++;
@@ -391,6 +409,7 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
         std::vector<int32_t> parent(N);
         for (int32_t v = 0; v < N; v++) parent[v] = par[v] == N ? -1 : par[v];
 
+        lap(3);
         out->n = N; out->nnz = run; out->n_levels = (int32_t)level_off.size() - 1;
         out->n_candidates = n_cand; out->msa_weight = weight; out->nnz_a = nnzA;
         out->rowptr = dup_array(drp); out->idx = dup_array(idx); out->parent = dup_array(parent);

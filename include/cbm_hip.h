@@ -82,6 +82,11 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t n_edges, int3
 
 void cbm_format_free(cbm_format* f);
 
+/* Seconds the calling thread's last cbm_build_host spent in its four phases: CSR + transpose,
+ * candidate edges, arborescence, tree arrays + deltas.  (The reference times construction as a
+ * whole, benchmark/parallel/cbm_creation.py:42-51.) */
+void cbm_build_host_timings(double* out4);
+
 /* Row schedule for the SpMM kernels: rows sorted by descending number of 64-entry gather rounds
  * (stable, so rows of similar length keep their natural order), one descriptor of 4 int32 per
  * row: { rowptr[r], rowptr[r + 1], r, bit pattern of the left scale }.  The left scale is m[r]
