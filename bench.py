@@ -120,6 +120,138 @@ def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
     }, y_cbm
 
 
+def gcn_epoch_bench(args):
+    """2-layer GCN forward + backward (cross-entropy) with CBM aggregation; prints one JSON line.
+    Model and protocol follow benchmark/parallel/benchmark_gcn_cpu.py:70-103 (3 warm-up + 10 timed
+    passes, one cbm_matrix shared by both layers), plus the backward pass the reference lacks."""
+    import numpy as np
+    import torch
+
+    from cbm4gnn_amd import graphs
+    from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
+
+    t0 = time.perf_counter()
+    w = graphs.workload(args.workload if args.workload != "c3" else "c4", scale=args.scale)
+    t_gen = time.perf_counter() - t0
+    alpha = args.alpha if args.alpha is not None else w.alphas[-1]
+    hidden, classes = 128, 41
+    ei = torch.from_numpy(w.edge_index)
+    t0 = time.perf_counter()
+    op = build_operator(ei, alpha=alpha, normalized=True)
+    t_build = time.perf_counter() - t0
+    dev = torch.device("cuda:0")
+    op.to(dev)
+    n = w.n
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((n, w.d), generator=g).to(dev)
+    labels = torch.randint(0, classes, (n,), generator=g).to(dev)
+    torch.manual_seed(0)
+    model = TwoLayerGCN(CBMGCNLayer(w.d, hidden, op), CBMGCNLayer(hidden, classes, op)).to(dev)
+    m = op.col_multiplier
+    vals = m[ei[0].long()] * m[ei[1].long()]
+    fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, vals, dev)       # rows = targets, as the CBM operator
+    bwd = fwd if op.is_symmetric else csr_operator(ei, n, vals, dev)
+    torch.manual_seed(0)
+    base = TwoLayerGCN(CSRGCNLayer(w.d, hidden, fwd, bwd), CSRGCNLayer(hidden, classes, fwd, bwd)).to(dev)
+
+    def epoch(net):
+        net.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(net(x), labels)
+        loss.backward()
+        return loss
+
+    def run(net):
+        for _ in range(args.warmup):
+            epoch(net)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(args.steps):
+            loss = epoch(net)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / args.steps, float(loss)
+
+    ms_cbm, loss_cbm = run(model)
+    ms_csr, loss_csr = run(base)
+    # aggregation alone: the 4 multiplies of an epoch (d = hidden and d = classes, forward and backward)
+    agg = 0.0
+    for dd in (hidden, classes):
+        h = torch.randn((n, dd), device=dev)
+        o = torch.empty_like(h)
+        _, t, _ = time_gpu(lambda: op._run_spmm_update(h, o, use_m=True), args.steps, args.warmup, torch)
+        agg += 2 * t
+    grad_err = max(float((p.grad - q.grad).abs().max() / q.grad.abs().max())
+                   for p, q in zip(model.parameters(), base.parameters()))
+    print(json.dumps({
+        "metric": "2-layer GCN epoch ms (forward + backward, CBM aggregation)", "value": ms_cbm, "unit": "ms",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_cbm, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.note}", "nodes": n, "nnz_A": op.nnz_a, "nnz_delta": op.nnz,
+                   "alpha": alpha, "in": w.d, "hidden": hidden, "classes": classes, "tree_levels": op.n_levels,
+                   "scale": args.scale},
+        "compression_ratio": op.compression_ratio(), "gcn_epoch_ms_gpu_csr": ms_csr, "speedup_vs_gpu_csr": ms_csr / ms_cbm,
+        "aggregation_ms_per_epoch": agg, "aggregation_share": agg / ms_cbm,
+        "loss": loss_cbm, "loss_gpu_csr": loss_csr, "max_rel_weight_grad_diff_vs_gpu_csr": grad_err,
+        "host_s": {"generate": t_gen, "build_format": t_build, "build_phases": op.build_seconds},
+    }))
+
+
+def alpha_sweep_bench(args):
+    """CBM multiply per alpha on one graph (default: the dense-community workload c5, d = 512):
+    compression ratio, tree depth and runtime per alpha, as alpha_searcher/spmm_cpu_parallel.py:84-124
+    does on the CPU.  Prints one JSON line with a row per alpha."""
+    import numpy as np
+    import torch
+
+    from cbm4gnn_amd import graphs
+    from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm, schedule_rows
+
+    w = graphs.workload(args.workload if args.workload != "c3" else "c5", scale=args.scale)
+    d = args.d or w.d
+    n = w.n
+    ei = torch.from_numpy(w.edge_index)
+    xd = w.features(0, d).cuda()
+    yd = torch.empty_like(xd)
+    order = np.lexsort((w.edge_index[1], w.edge_index[0]))
+    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(w.edge_index[0], minlength=n))]).astype(np.int32)).cuda()
+    col = torch.from_numpy(w.edge_index[1][order].astype(np.int32)).cuda()
+    val = None
+    if w.normalized:
+        m = torch.bincount(ei[0].long(), minlength=n).float().pow(-0.5)
+        val = (m[torch.from_numpy(w.edge_index[0][order].astype(np.int64))] * m[torch.from_numpy(w.edge_index[1][order].astype(np.int64))]).cuda()
+    ycsr = torch.empty_like(xd)
+    sched = schedule_rows(rp).to(xd.device)
+    _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp, col, val, xd, ycsr, sched), args.steps, args.warmup, torch)
+    rows = []
+    alphas = [args.alpha] if args.alpha is not None else list(w.alphas)
+    for alpha in alphas:
+        t0 = time.perf_counter()
+        mat = cbm_matrix(ei, None, alpha=alpha, normalized=w.normalized)
+        t_build = time.perf_counter() - t0
+        mat.to(xd.device)
+        step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
+        _, ms, _ = time_gpu(step, args.steps, args.warmup, torch)
+        zd = torch.empty_like(xd)
+        _, spmm_ms, _ = time_gpu(lambda: mat._run_spmm(xd, zd, use_m=w.normalized, scale_roots=w.normalized), args.steps, args.warmup, torch)
+        tree_edges = n - int(mat.level_off[1])
+        b_spmm, b_prop, b_csr = algorithmic_bytes(n, mat.nnz, d, int(w.normalized), tree_edges, mat.n_levels, mat.nnz_a)
+        step(); torch.cuda.synchronize()
+        rows.append({"alpha": alpha, "compression_ratio": mat.compression_ratio(), "nnz_delta": mat.nnz,
+                     "tree_levels": mat.n_levels, "tree_edges": tree_edges, "cbm_ms": ms, "delta_spmm_ms": spmm_ms,
+                     "propagate_ms": ms - spmm_ms, "cbm_GBps": (b_spmm + b_prop) / ms / 1e6,
+                     "speedup_vs_gpu_csr": csr_ms / ms, "build_s": t_build, "build_phases": mat.build_seconds,
+                     "max_rel_err_vs_gpu_csr": float((yd - ycsr).abs().max() / ycsr.abs().max())})
+        del mat
+    print(json.dumps({
+        "metric": "CBM SpMM alpha sweep", "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.note}", "nodes": n, "nnz_A": int(ei.size(1)), "d": d, "scale": args.scale,
+                   "mean_degree": ei.size(1) / n},
+        "gpu_csr_ms": csr_ms, "gpu_csr_GBps": algorithmic_bytes(n, 0, d, int(w.normalized), 0, 1, int(ei.size(1)))[2] / csr_ms / 1e6,
+        "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,10 +265,19 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter run: 3 multiplies and 3 plain device copies of X (known size, for scaling "
                          "FETCH_SIZE / WRITE_SIZE), no timing, no JSON")
+    ap.add_argument("--sweep", action="store_true",
+                    help="alpha sweep (default workload c5): compression ratio and runtime per alpha")
+    ap.add_argument("--gcn", action="store_true",
+                    help="measure the 2-layer GCN forward+backward epoch (default workload c4) instead of the multiply")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); "
                  "run with --gpus 1")
+    if args.gcn or args.sweep:
+        import torch
+        if not torch.cuda.is_available():
+            sys.exit("bench.py needs a HIP device")
+        return gcn_epoch_bench(args) if args.gcn else alpha_sweep_bench(args)
 
     import numpy as np
     import torch

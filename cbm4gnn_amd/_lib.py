@@ -23,7 +23,7 @@ class CbmLibraryError(RuntimeError):
 class CbmFormat(C.Structure):
     """Mirror of ``struct cbm_format``."""
     _fields_ = [
-        ("n", C.c_int32), ("n_levels", C.c_int32), ("nnz", C.c_int64), ("nnz_a", C.c_int64),
+        ("n", C.c_int32), ("n_levels", C.c_int32), ("is_symmetric", C.c_int32), ("reserved", C.c_int32), ("nnz", C.c_int64), ("nnz_a", C.c_int64),
         ("n_candidates", C.c_int64), ("msa_weight", C.c_int64),
         ("rowptr", C.POINTER(C.c_int32)), ("idx", C.POINTER(C.c_uint32)), ("parent", C.POINTER(C.c_int32)),
         ("order", C.POINTER(C.c_int32)), ("level_off", C.POINTER(C.c_int32)),

@@ -158,6 +158,7 @@ class cbm_matrix:
             self.nnz_a = int(fmt.nnz_a)
             self.n_candidates = int(fmt.n_candidates)
             self.n_levels = int(fmt.n_levels)
+            self.is_symmetric = bool(fmt.is_symmetric)
             self.rowptr = take(fmt.rowptr, n + 1, np.int32)
             # packed column | sign << 31; kept as the int32 bit pattern (torch has no uint32 math)
             self.idx = take(fmt.idx, self.nnz, np.uint32).view(torch.int32) if self.nnz else torch.empty(0, dtype=torch.int32)
@@ -180,9 +181,6 @@ class cbm_matrix:
         self._dev = {}
         self.stream_coefficients = True     # False: gather m[col] in the kernel, 4 B/entry less device memory
         self._transposed = None
-        keys = ei_cpu[0].to(torch.int64) * n + ei_cpu[1].to(torch.int64)
-        keys_t = ei_cpu[1].to(torch.int64) * n + ei_cpu[0].to(torch.int64)
-        self.is_symmetric = bool(torch.equal(torch.unique(keys), torch.unique(keys_t)))
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
 
     # ------------------------------------------------------------------ format views --------

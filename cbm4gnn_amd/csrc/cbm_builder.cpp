@@ -274,6 +274,8 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
                 for (int64_t k = rp[r]; k < rp[r + 1]; k++) tr[fill[ci[k]]++] = r;   // ascending r per column
         }
 
+        // symmetric pattern <=> CSR(A) == CSR(A^T) (both have ascending columns)
+        const bool symmetric = rp == tp && ci == tr;
         lap(0);
         // ---- candidate edges (reference rule, cpp:75-103), streamed and pruned ------------------
         // pair (i, j>i) with s shared columns: h = nnz_i + nnz_j - 2s;
@@ -412,6 +414,7 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
         lap(3);
         out->n = N; out->nnz = run; out->n_levels = (int32_t)level_off.size() - 1;
         out->n_candidates = n_cand; out->msa_weight = weight; out->nnz_a = nnzA;
+        out->is_symmetric = symmetric ? 1 : 0;
         out->rowptr = dup_array(drp); out->idx = dup_array(idx); out->parent = dup_array(parent);
         out->order = dup_array(order); out->level_off = dup_array(level_off);
         out->mst_row = dup_array(mst_row); out->mst_col = dup_array(mst_col);

@@ -58,16 +58,24 @@ def _bernoulli_positions(rng, m: int, p: float) -> np.ndarray:
     return np.concatenate(out)
 
 
-def coalesce_undirected(u: np.ndarray, v: np.ndarray, n: int, drop_loops: bool = True) -> np.ndarray:
-    """Symmetrise, de-duplicate and sort an undirected pair list -> int32 [2, E]."""
+def coalesce_undirected(u: np.ndarray, v: np.ndarray, n: int, drop_loops: bool = True,
+                        assume_unique: bool = False) -> np.ndarray:
+    """Symmetrise, de-duplicate and sort an undirected pair list -> int32 [2, E].
+    ``assume_unique``: the pairs are known to be distinct (only the sort is needed)."""
     u = np.asarray(u, np.int64)
     v = np.asarray(v, np.int64)
     if drop_loops:
         keep = u != v
         u, v = u[keep], v[keep]
     key = np.concatenate([u * n + v, v * n + u])
-    key = np.unique(key)
-    return np.stack([key // n, key % n]).astype(np.int32)
+    if assume_unique:
+        key.sort(kind="stable")                 # two long sorted-ish runs: timsort territory
+    else:
+        key = np.unique(key)
+    out = np.empty((2, key.shape[0]), np.int32)
+    np.floor_divide(key, n, out=out[0], casting="unsafe")
+    np.remainder(key, n, out=out[1], casting="unsafe")
+    return out
 
 
 def add_self_loops(edge_index: np.ndarray, n: int | None = None) -> np.ndarray:
@@ -77,8 +85,13 @@ def add_self_loops(edge_index: np.ndarray, n: int | None = None) -> np.ndarray:
         n = int(ei.max()) + 1
     keep = ei[0] != ei[1]
     key = np.concatenate([ei[0][keep] * n + ei[1][keep], np.arange(n, dtype=np.int64) * (n + 1)])
-    key = np.unique(key)
-    return np.stack([key // n, key % n]).astype(np.int32)
+    key.sort(kind="stable")
+    if key.size > 1:
+        key = key[np.concatenate([[True], key[1:] != key[:-1]])]
+    out = np.empty((2, key.shape[0]), np.int32)
+    np.floor_divide(key, n, out=out[0], casting="unsafe")
+    np.remainder(key, n, out=out[1], casting="unsafe")
+    return out
 
 
 def _patch_isolated(rng, edge_index: np.ndarray, n: int) -> np.ndarray:
@@ -131,7 +144,8 @@ def sbm(n: int, blocks: int, p_in: float, p_out: float, seed: int = 0, patch: bo
     keep = blk[i] != blk[j]
     us.append(i[keep])
     vs.append(j[keep])
-    ei = coalesce_undirected(np.concatenate(us), np.concatenate(vs), n)
+    # positions inside one triangle are distinct and inter-block pairs never fall inside a block
+    ei = coalesce_undirected(np.concatenate(us), np.concatenate(vs), n, assume_unique=True)
     return _patch_isolated(rng, ei, n) if patch else ei
 
 

@@ -55,6 +55,8 @@ enum {
 typedef struct cbm_format {
     int32_t n;
     int32_t n_levels;
+    int32_t is_symmetric;   /* 1 if the input pattern equals its transpose (A_hat^T = A_hat) */
+    int32_t reserved;
     int64_t nnz;            /* delta non-zeros = weight of the arborescence */
     int64_t nnz_a;          /* non-zeros of the input matrix after de-duplication */
     int64_t n_candidates;   /* edges of the distance graph, root edges included */

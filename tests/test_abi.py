@@ -33,9 +33,9 @@ def test_libraries_export_every_declared_symbol():
 
 
 def test_struct_mirror_layout():
-    # struct cbm_format: 2 x int32, 4 x int64, 7 pointers
-    assert C.sizeof(_lib.CbmFormat) == 8 + 32 + 56
-    assert _lib.CbmFormat.rowptr.offset == 40
+    # struct cbm_format: 4 x int32, 4 x int64, 7 pointers
+    assert C.sizeof(_lib.CbmFormat) == 16 + 32 + 56
+    assert _lib.CbmFormat.rowptr.offset == 48
 
 
 def test_shim_exports_the_reference_extension_names():

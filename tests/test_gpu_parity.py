@@ -299,3 +299,39 @@ def test_c_abi_status_codes_on_device_calls():
     assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), n, d, d, d, 0, None) == 3
     torch.cuda.synchronize()
     assert (y == 0).all()
+
+
+def test_two_layer_gcn_forward_backward_matches_dense(orc):
+    """The GCN epoch harness (Linear -> CBM aggregate -> ReLU -> Linear -> CBM aggregate, cross
+    entropy) against the same model written with a dense normalised adjacency in torch."""
+    from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
+    n, f_in, hidden, classes = 300, 37, 128, 41
+    ei_np = graphs.add_self_loops(graphs.sbm(n, 6, 0.3, 0.02, seed=11), n)
+    ei = torch.from_numpy(ei_np)
+    say("gcn harness")
+    op = build_operator(ei, alpha=2, normalized=True)
+    assert op.n_levels >= 2
+    torch.manual_seed(1)
+    model = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op), CBMGCNLayer(hidden, classes, op)).cuda()
+    x = torch.randn((n, f_in), generator=torch.Generator().manual_seed(2)).cuda()
+    y = torch.randint(0, classes, (n,), generator=torch.Generator().manual_seed(3)).cuda()
+    loss = torch.nn.functional.cross_entropy(model(x), y)
+    loss.backward()
+    a = torch.from_numpy(orc.dense_adjacency(np.stack([ei_np[1], ei_np[0]]), n)).double().cuda()
+    m = a.sum(dim=1).pow(-0.5)
+    a_hat = m[:, None] * a * m[None, :]
+    w1 = model.first_layer.lin.weight.detach().double().requires_grad_(True)
+    w2 = model.last_layer.lin.weight.detach().double().requires_grad_(True)
+    ref = a_hat @ ((a_hat @ (x.double() @ w1.t())).relu() @ w2.t())
+    ref_loss = torch.nn.functional.cross_entropy(ref, y)
+    ref_loss.backward()
+    assert abs(float(loss) - float(ref_loss)) <= 1e-4 * abs(float(ref_loss))
+    for got, want in ((model.first_layer.lin.weight.grad, w1.grad), (model.last_layer.lin.weight.grad, w2.grad)):
+        assert float((got.double() - want).abs().max() / want.abs().max()) <= 1e-3
+    # the CSR-baseline model computes the same thing
+    vals = op.col_multiplier[ei[0].long()] * op.col_multiplier[ei[1].long()]
+    fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, vals, x.device)
+    torch.manual_seed(1)
+    base = TwoLayerGCN(CSRGCNLayer(f_in, hidden, fwd, fwd), CSRGCNLayer(hidden, classes, fwd, fwd)).cuda()
+    base_loss = torch.nn.functional.cross_entropy(base(x), y)
+    assert abs(float(base_loss) - float(loss)) <= 1e-5 * abs(float(loss))
