@@ -238,7 +238,10 @@ def alpha_sweep_bench(args):
         b_spmm, b_prop, b_csr = algorithmic_bytes(n, mat.nnz, d, int(w.normalized), tree_edges, mat.n_levels, mat.nnz_a)
         step(); torch.cuda.synchronize()
         rows.append({"alpha": alpha, "compression_ratio": mat.compression_ratio(), "nnz_delta": mat.nnz,
-                     "tree_levels": mat.n_levels, "tree_edges": tree_edges, "cbm_ms": ms, "delta_spmm_ms": spmm_ms,
+                     "tree_levels": mat.n_levels, "tree_edges": tree_edges,
+                     "level_widths": {"first": np.diff(mat.level_off.numpy())[:12].tolist(),
+                                      "histogram": {int(k): int(v) for k, v in zip(*np.unique(np.diff(mat.level_off.numpy()), return_counts=True))} if mat.n_levels <= 64 or True else None},
+                     "cbm_ms": ms, "delta_spmm_ms": spmm_ms,
                      "propagate_ms": ms - spmm_ms, "cbm_GBps": (b_spmm + b_prop) / ms / 1e6,
                      "speedup_vs_gpu_csr": csr_ms / ms, "build_s": t_build, "build_phases": mat.build_seconds,
                      "max_rel_err_vs_gpu_csr": float((yd - ycsr).abs().max() / ycsr.abs().max())})

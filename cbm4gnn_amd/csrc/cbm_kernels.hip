@@ -17,6 +17,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "../../include/cbm_hip.h"
 
 namespace {
@@ -271,34 +273,49 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
             if (i < n) nxt = fetch(i);
 
             float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (int pos = start; pos < end; pos += kStep * U) {
-                float x[U][4];
-                float f[U];
+            // One gather round = UU instructions of kStep entries each.  Every load of a round is
+            // unconditional -- entries past the end of the row are clamped to its last entry and
+            // get coefficient 0 -- so the index loads, then the X-row loads, are all in flight
+            // together; a branch or an exec mask around each load would serialise them.  Short
+            // remainders take a shorter round instead of mostly clamped instructions.
+            auto round = [&](auto uu_tag, int pos) {
+                constexpr int UU = decltype(uu_tag)::value;
+                uint32_t p[UU];
+                float f[UU];
+                float x[UU][4];
 #pragma unroll
-                for (int u = 0; u < U; u++) {
+                for (int u = 0; u < UU; u++) {
                     const int k = pos + u * kStep + sub;
-                    f[u] = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) x[u][e] = 0.0f;
-                    if (k < end) {
-                        const uint32_t p = idx[k];
-                        const uint32_t c = PACKED ? (p & 0x7fffffffu) : p;
-                        if constexpr (PACKED) {
-                            if (val) f[u] = val[k];        // streamed +-m[col]
-                            else {
-                                const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
-                                f[u] = __uint_as_float(mag ^ (p & 0x80000000u));
-                            }
-                        } else {
-                            f[u] = val ? val[k] : 1.0f;
-                        }
-                        load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
-                    }
+                    const int kc = min(k, end - 1);
+                    p[u] = idx[kc];
+                    if (val) f[u] = val[kc];
+                    else f[u] = 1.0f;
+                    if (k >= end) f[u] = 0.0f;
                 }
 #pragma unroll
-                for (int u = 0; u < U; u++)
+                for (int u = 0; u < UU; u++) {
+                    const uint32_t c = PACKED ? (p[u] & 0x7fffffffu) : p[u];
+                    if constexpr (PACKED) {
+                        if (!val) {                        // no streamed coefficients: sign bit, optional m gather
+                            const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
+                            const float g = __uint_as_float(mag ^ (p[u] & 0x80000000u));
+                            f[u] = f[u] == 0.0f ? 0.0f : g;
+                        }
+                    }
+                    load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < UU; u++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) acc[e] = fmaf(f[u], x[u][e], acc[e]);
+            };
+            int pos = start;
+            while (pos < end) {
+                const int rem = end - pos;
+                if (rem > (U / 2) * kStep) { round(std::integral_constant<int, U>{}, pos); pos += U * kStep; }
+                else if (rem > (U / 4) * kStep) { round(std::integral_constant<int, U / 2>{}, pos); pos += (U / 2) * kStep; }
+                else if (rem > kStep) { round(std::integral_constant<int, U / 4>{}, pos); pos += (U / 4) * kStep; }
+                else { round(std::integral_constant<int, 1>{}, pos); pos += kStep; }
             }
 #pragma unroll
             for (int off = LPE; off < kWave; off <<= 1)
@@ -391,6 +408,61 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_narrow_levels(
         }
         __threadfence();
         __syncthreads();
+    }
+}
+
+// A run of levels that all hold ONE row is a chain: row k's parent is row k - 1 of the run.  One
+// thread per feature column carries the running value in a register down the chain, so the only
+// dependency between levels is an add; the rows of Y it needs are independent loads and are
+// fetched kChainDepth levels ahead.  The 64 row ids (and their m) of a stretch come in with one
+// coalesced load and are broadcast with v_readlane.  Arithmetic per level is exactly that of
+// propagate_row.
+constexpr int kChainDepth = 16;
+constexpr int kMinChain = 4;               // shorter runs of single-row levels stay with the other kernels
+
+template <bool NORM>
+__global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
+    const int32_t* __restrict__ parent, const int32_t* __restrict__ order, int first, int count,
+    const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;          // feature column of this thread
+    const bool live = j < d;                                      // whole waves beyond d were not launched
+    const int jj = live ? j : 0;                                  // dead lanes load column 0 and store nothing
+    const int v0 = order[first];
+    const int u0 = parent[v0];
+    float run = Y[(int64_t)u0 * ldy + jj];                         // final value of the row above the chain
+    float mu = NORM ? m[u0] : 1.0f;
+    for (int base = 0; base < count; base += kWave) {
+        const int cnt = min(kWave, count - base);
+        int my_v = 0;
+        float my_m = 1.0f;
+        if (lane < cnt) {
+            my_v = order[first + base + lane];
+            if constexpr (NORM) my_m = m[my_v];
+        }
+        for (int k = 0; k < cnt; k += kChainDepth) {
+            float z[kChainDepth];
+            // unconditional loads (past the end of the stretch: its last row again), so that all
+            // kChainDepth of them are in flight before the first is needed
+#pragma unroll
+            for (int u = 0; u < kChainDepth; u++)
+                z[u] = Y[(int64_t)bcast_i(my_v, min(k + u, cnt - 1)) * ldy + jj];
+#pragma unroll
+            for (int u = 0; u < kChainDepth; u++) {
+                if (k + u < cnt) {
+                    const int v = bcast_i(my_v, k + u);
+                    if constexpr (NORM) {
+                        const float mv = bcast_f(my_m, k + u);
+                        const float inv_mu = 1.0f / mu;
+                        run = (j < dv) ? fmaf(run, inv_mu, z[u]) * mv : (z[u] + run / mu) * mv;
+                        mu = mv;
+                    } else {
+                        run = z[u] + run;
+                    }
+                    if (live) Y[(int64_t)v * ldy + j] = run;
+                }
+            }
+        }
     }
 }
 
@@ -551,9 +623,27 @@ int launch_propagate(const int32_t* parent, const int32_t* order, const int32_t*
     int l = 1;
     while (l < n_levels) {
         const int width = lo[l + 1] - lo[l];
+        auto chain_end = [&](int from) {                   // end of the run of single-row levels at `from`
+            int e = from;
+            while (e < n_levels && lo[e + 1] - lo[e] == 1) e++;
+            return e;
+        };
+        if (width == 1) {                                  // a chain of single-row levels
+            const int l_end = chain_end(l);
+            if (l_end - l >= kMinChain) {
+                const int waves = (d + kWave - 1) / kWave;
+                const int wpb = waves < kNarrowWaves ? waves : kNarrowWaves;
+                const dim3 grid((waves + wpb - 1) / wpb), cblock(kWave * wpb);
+                hipLaunchKernelGGL((propagate_chain<NORM>), grid, cblock, 0, s, parent, order, lo[l], l_end - l, m, Y,
+                                   d, dv, ldy);
+                l = l_end;
+                continue;
+            }
+        }
         if (width <= kNarrowWidth) {
-            int l_end = l + 1;
-            while (l_end < n_levels && lo[l_end + 1] - lo[l_end] <= kNarrowWidth) l_end++;
+            int l_end = l + 1;                             // extend over narrow levels, but leave chains to the chain kernel
+            while (l_end < n_levels && lo[l_end + 1] - lo[l_end] <= kNarrowWidth &&
+                   chain_end(l_end) - l_end < kMinChain) l_end++;
             if (l_end - l >= 2) {
                 const dim3 grid(1, t.grid_y), nblock(kWave * kNarrowWaves);
 #define LAUNCH(V, C, F)                                                                                 \

@@ -184,14 +184,42 @@ def test_update_only_entry_points(orc):
         assert torch.equal(y, y2)
 
 
-def test_deep_narrow_tree_uses_multi_level_kernel(orc):
-    # 64-deep staircase chain: runs of width-1 levels go through the single-workgroup kernel
-    ei = graphs.sbm_with_chain(n=1500, blocks=24, p_in=1.0, mean_deg=80.0, chain=64, base=48, seed=0)
+def test_narrow_levels_use_the_single_workgroup_kernel(orc):
+    # a hand-made tree: 40 levels of 3 rows each under one root child (narrow, but not a chain)
+    n, d = 121, 72
+    parent = np.full(n, -1, np.int64)
+    for v in range(1, n):
+        parent[v] = 0 if v <= 3 else v - 3
+    kids = [[] for _ in range(n + 1)]
+    for v in range(n):
+        kids[n if parent[v] < 0 else parent[v]].append(v)
+    mst_col = torch.tensor(sum(kids, []), dtype=torch.int32)
+    mst_row = torch.tensor(np.concatenate([[0], np.cumsum([len(k) for k in kids])]), dtype=torch.int32)
+    from cbm import cbm_mkl_cpp as cbm_
+    rng = np.random.default_rng(0)
+    z = rng.standard_normal((n, d)).astype(np.float32)
+    m = (rng.random(n).astype(np.float32) + 0.5)
+    say("narrow levels, plain")
+    y = torch.from_numpy(z.copy()).cuda()
+    cbm_.omp_s_update_csr_int32(mst_row, mst_col, y)
+    assert np.array_equal(y.cpu().numpy(), orc.update_plain(mst_row.numpy(), mst_col.numpy(), z.copy()))
+    say("narrow levels, normalised")
+    y = torch.from_numpy(z.copy()).cuda()
+    cbm_.omp_s_fused_update_csr_int32(mst_row, mst_col, torch.from_numpy(m), y)
+    assert np.array_equal(y.cpu().numpy(), orc.update_fused(mst_row.numpy(), mst_col.numpy(), m, z.copy()))
+
+
+def test_deep_chain_uses_the_chain_kernel(orc):
+    # 150-deep staircase chain: the run of single-row levels goes through the chain kernel
+    # (register-carried running row, more than two 64-level stretches)
+    ei = graphs.sbm_with_chain(n=1500, blocks=24, p_in=1.0, mean_deg=80.0, chain=150, base=48, seed=0)
     n = 1500
-    for normalized, d in ((False, 512), (True, 96), (False, 10)):
+    for normalized, d in ((False, 512), (True, 96), (True, 41), (False, 10), (True, 1100)):
         e2 = graphs.add_self_loops(ei, n) if normalized else ei
         mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
-        assert mat.n_levels >= 65
+        assert mat.n_levels >= 151
+        widths = np.diff(mat.level_off.numpy())
+        assert (widths[-120:] == 1).all()
         say("deep chain", normalized, d, "levels", mat.n_levels)
         x = np.random.default_rng(1).standard_normal((n, d)).astype(np.float32)
         got = gpu_product(mat, x, normalized)
