@@ -389,24 +389,40 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void propagate_level(
 }
 
 // A run of narrow levels [l_beg, l_end) handled by ONE workgroup: its 16 waves share each level's
-// rows and meet at a barrier between levels.  Column tiles (grid.y) are independent of each
-// other, so every tile is its own single workgroup.
+// rows (at most kNarrowWidth = 64, so at most 4 per wave) and meet at a barrier between levels.
+// The (row, parent) pairs of the NEXT level do not depend on Y, so each wave fetches them before
+// the barrier; after it only the two Y rows are on the critical path.  All waves of a workgroup
+// share one L1, so a workgroup-scope fence orders the stores of one level before the loads of
+// the next.  Column tiles (grid.y) are independent: every tile is its own single workgroup.
 template <int VEC, int CH, bool NORM, bool FULL>
 __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_narrow_levels(
     const int32_t* __restrict__ parent, const int32_t* __restrict__ order,
     const int32_t* __restrict__ level_off, int l_beg, int l_end, const float* __restrict__ m,
     float* __restrict__ Y, int d, int dv, int64_t ldy) {
+    constexpr int kPerWave = kNarrowWidth / kNarrowWaves;        // rows of a level one wave may own
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
-    for (int l = l_beg; l < l_end; l++) {
-        const int beg = level_off[l], end = level_off[l + 1];
-        for (int i = beg + wave; i < end; i += kNarrowWaves) {
-            const int v = __builtin_amdgcn_readfirstlane(order[i]);
-            const int u = __builtin_amdgcn_readfirstlane(parent[v]);
-            propagate_row<VEC, CH, NORM, FULL>(v, u, m, Y, d, dv, ldy, col0);
+    // lane t < kPerWave of a wave holds the wave's t-th row of the level (and its parent)
+    auto fetch = [&](int l, int& v, int& u) {
+        v = -1; u = -1;
+        if (l < l_end && lane < kPerWave) {
+            const int i = level_off[l] + wave + kNarrowWaves * lane;
+            if (i < level_off[l + 1]) { v = order[i]; u = parent[v]; }
         }
-        __threadfence();
+    };
+    int my_v, my_u;
+    fetch(l_beg, my_v, my_u);
+    for (int l = l_beg; l < l_end; l++) {
+        const int cur_v = my_v, cur_u = my_u;
+        fetch(l + 1, my_v, my_u);
+#pragma unroll
+        for (int t = 0; t < kPerWave; t++) {
+            const int v = bcast_i(cur_v, t);
+            if (v < 0) break;
+            propagate_row<VEC, CH, NORM, FULL>(v, bcast_i(cur_u, t), m, Y, d, dv, ldy, col0);
+        }
+        __threadfence_block();
         __syncthreads();
     }
 }
