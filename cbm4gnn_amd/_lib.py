@@ -13,7 +13,6 @@ from .build import HIP_LIB, HOST_LIB
 
 CBM_OK = 0
 CBM_PROP_SCALE_ROOTS = 1
-CBM_PROP_PERSISTENT = 2
 
 
 class CbmLibraryError(RuntimeError):

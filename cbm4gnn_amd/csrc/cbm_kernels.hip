@@ -1,16 +1,19 @@
 // HIP kernels (gfx950 / CDNA4) and C-ABI launchers of the CBM multiply.
 //
-// Two bandwidth-bound kernels, no MFMA:
-//   (1) delta SpMM      Z = D * diag(m) * X      one 64-lane wavefront per row, lanes span the
-//                       feature columns (float4 / float2 / float per lane so that one load
-//                       instruction fetches a whole contiguous row of X); the row's packed
-//                       indices are fetched 64 at a time with one coalesced load and broadcast
-//                       lane by lane through v_readlane into scalar registers, so every X-row
-//                       load has a scalar base address.
-//   (2) tree propagate  Y[v] (+)= Y[parent(v)]   level-synchronous over a host-computed
-//                       (level, id) ordering: one launch per wide level, one single-workgroup
-//                       launch per run of narrow levels.
-// The same SpMM template without the sign bit is the plain CSR baseline.
+// Bandwidth-bound gather / stream kernels, 64-wide wavefronts, no MFMA, no atomics:
+//   (1)  spmm_slab_per_xcd    delta SpMM  Z = D * diag(m) * X  for feature widths that split into
+//                             128- or 256-byte slabs: one slab per XCD (so an XCD's L2 only ever
+//                             sees its slab of X), persistent waves walking a longest-first row
+//                             schedule, 8 lanes per delta entry, 64 entries in flight per wave.
+//        spmm_wave_per_row    the same product for any other width or alignment: one wave per
+//                             row, lanes span the feature columns, packed indices broadcast with
+//                             v_readlane so X-row addresses are scalar.
+//   (2)  propagate_level / propagate_narrow_levels / propagate_chain / scale_level0
+//                             tree propagation  Y[v] (+)= Y[parent(v)]  level-synchronously over a
+//                             host-computed (level, id) ordering: one launch per wide level, one
+//                             single-workgroup launch per run of narrow levels, one
+//                             register-carried launch per chain of single-row levels.
+// The SpMM templates without the sign bit (PACKED = false) are the plain CSR baseline.
 //
 // What each launcher replaces in the reference is stated in include/cbm_hip.h.
 #include <hip/hip_runtime.h>
@@ -23,7 +26,9 @@
 
 namespace {
 
-// Tunables (overridable with -D for sweeps; the defaults are what measurements on MI355X chose).
+// Tunables (overridable with -D for sweeps; the defaults are what measurements on MI355X chose:
+// 2, 8 or 16 waves per workgroup, 4 or 16 loads in flight and no XCD remap were all within +-3 %
+// or slower on the 100k-node power-law workload).
 #ifndef CBM_WAVES_PER_BLOCK
 #define CBM_WAVES_PER_BLOCK 4
 #endif
@@ -32,9 +37,6 @@ namespace {
 #endif
 #ifndef CBM_XCD_REMAP
 #define CBM_XCD_REMAP 1
-#endif
-#ifndef CBM_NT_STORE
-#define CBM_NT_STORE 0
 #endif
 
 constexpr int kWave = 64;
@@ -68,13 +70,7 @@ __device__ __forceinline__ void load_vec(const float* __restrict__ p, float (&v)
 
 template <int VEC>
 __device__ __forceinline__ void store_vec(float* __restrict__ p, const float (&v)[VEC]) {
-    if constexpr (CBM_NT_STORE) {
-        typedef float vf __attribute__((ext_vector_type(VEC)));
-        vf t;
-#pragma unroll
-        for (int e = 0; e < VEC; e++) t[e] = v[e];
-        __builtin_nontemporal_store(t, reinterpret_cast<vf*>(p));
-    } else if constexpr (VEC == 4) {
+    if constexpr (VEC == 4) {
         *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
     } else if constexpr (VEC == 2) {
         *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
@@ -590,6 +586,7 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
     if (sched && !aligned(sched, 16)) return CBM_ERR_SHAPE;
+    if (X == Z) return CBM_ERR_SHAPE;                    // rows of X are gathered while rows of Z are written
     if (n == 0 || d == 0) return CBM_OK;
     const int4* sc = reinterpret_cast<const int4*>(sched);
     if (const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z)) {
@@ -754,7 +751,7 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
     if (!parent || !order || !level_off_dev || !level_off_host || !Y) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldy)) return rc;
     if (int rc = validate_levels(level_off_host, n_levels, n)) return rc;
-    if (flags & CBM_PROP_PERSISTENT) return CBM_ERR_UNSUPPORTED;
+    if (flags & ~CBM_PROP_SCALE_ROOTS) return CBM_ERR_UNSUPPORTED;
     if (n == 0 || d == 0) return CBM_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return m ? launch_propagate<true>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s)

@@ -38,8 +38,7 @@ enum {
 
 /* flags of cbm_propagate_f32 / cbm_spmm_update_f32 */
 enum {
-    CBM_PROP_SCALE_ROOTS = 1, /* normalised only: first do Y[r,:] *= m[r] for children of the root */
-    CBM_PROP_PERSISTENT = 2   /* one persistent kernel walking the levels instead of per-level launches */
+    CBM_PROP_SCALE_ROOTS = 1  /* normalised only: first do Y[r,:] *= m[r] for children of the root */
 };
 
 /* The CBM format as built on the host.  All arrays are malloc'd by cbm_build_host and are

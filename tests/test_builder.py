@@ -173,3 +173,38 @@ def test_graph_generators_are_pinned():
         if name == "c1":
             from cbm4gnn_amd.utility import check_edge_index
             check_edge_index(torch.from_numpy(w.edge_index).long())
+
+
+def test_row_schedule_properties():
+    from cbm4gnn_amd.cbm import schedule_rows
+    rng = np.random.default_rng(0)
+    n = 500
+    lens = np.concatenate([rng.integers(0, 70, n - 5), [0, 64, 65, 700, 129]])
+    rowptr = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    parent = torch.tensor(rng.integers(-1, n, n), dtype=torch.int32)
+    m = torch.tensor(rng.random(n) + 0.5, dtype=torch.float32)
+    plain = schedule_rows(rowptr).numpy()
+    scaled = schedule_rows(rowptr, parent, m).numpy()
+    for s in (plain, scaled):
+        rows = s[:, 2]
+        assert sorted(rows.tolist()) == list(range(n))                      # a permutation
+        assert np.array_equal(s[:, 0], rowptr.numpy()[:-1][rows]) and np.array_equal(s[:, 1], rowptr.numpy()[1:][rows])
+        rounds = (lens[rows] + 63) // 64
+        assert (np.diff(rounds) <= 0).all()                                 # longest first
+        for r in np.unique(rounds):
+            assert (np.diff(rows[rounds == r]) > 0).all()                   # stable inside a bucket
+    assert (plain[:, 3].view(np.float32) == 1.0).all()
+    want = np.where(parent.numpy()[scaled[:, 2]] < 0, m.numpy()[scaled[:, 2]], np.float32(1.0))
+    assert np.array_equal(scaled[:, 3].view(np.float32), want.astype(np.float32))
+    assert _lib.host_lib().cbm_schedule_rows(None, None, None, 3, None) == 1
+
+
+def test_graphs_with_empty_rows_single_node_and_self_loop_only(orc):
+    # node 3 has no edge at all (its row is empty), node 0 only a self loop
+    ei = torch.tensor([[0, 1, 2, 4, 2], [0, 2, 1, 2, 4]], dtype=torch.int32)
+    mat = cbm_matrix(ei, None, alpha=0)
+    assert mat.num_rows == 5 and mat.nnz_a == 5
+    assert np.diff(mat.rowptr.numpy())[3] == 0
+    assert orc.check_format(ei.numpy(), 5, mat.rowptr.numpy(), _u32(mat.idx), mat.mst_row.numpy(), mat.mst_col.numpy())
+    one = cbm_matrix(torch.tensor([[0], [0]], dtype=torch.int32), None, alpha=0, normalized=True)
+    assert one.num_rows == 1 and one.nnz == 1 and one.n_levels == 1 and float(one.col_multiplier[0]) == 1.0

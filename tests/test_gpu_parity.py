@@ -363,3 +363,28 @@ def test_two_layer_gcn_forward_backward_matches_dense(orc):
     base = TwoLayerGCN(CSRGCNLayer(f_in, hidden, fwd, fwd), CSRGCNLayer(hidden, classes, fwd, fwd)).cuda()
     base_loss = torch.nn.functional.cross_entropy(base(x), y)
     assert abs(float(base_loss) - float(loss)) <= 1e-5 * abs(float(loss))
+
+
+def test_degenerate_shapes(orc):
+    # empty rows, a single-row matrix, d = 1, more slabs than rows
+    ei = np.array([[0, 1, 2, 4, 2], [0, 2, 1, 2, 4]], np.int32)      # row 3 is empty
+    for d in (1, 32, 256):
+        say("degenerate", d)
+        x = np.random.default_rng(d).standard_normal((5, d)).astype(np.float32)
+        for normalized in (False, True):
+            if normalized:
+                e2 = graphs.add_self_loops(ei, 5)                     # no zero degrees under normalisation
+            else:
+                e2 = ei
+            mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
+            got = gpu_product(mat, x, normalized)
+            assert orc.max_rel_err(got, orc.dense_product(e2, 5, x, normalized)) <= 1e-6
+            if not normalized:
+                assert (got[3] == 0).all()
+    one = cbm_matrix(torch.tensor([[0], [0]], dtype=torch.int32), None, alpha=0)
+    x = torch.arange(64, dtype=torch.float32).reshape(1, 64).cuda()
+    y = torch.empty_like(x)
+    one.omp_mkl_csr_spmm_update(x, y)
+    assert torch.equal(x, y)
+    with pytest.raises(ValueError):
+        one.omp_mkl_csr_spmm_update(x, x)                             # in place is refused
