@@ -183,6 +183,51 @@ class cbm_matrix:
         self._transposed = None
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
 
+    # ------------------------------------------------------------------ on-disk cache --------
+    _SAVED_ARRAYS = ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col")
+    FORMAT_VERSION = 1
+
+    def save(self, path):
+        """Write the built format to ``path`` (NumPy ``.npz``, no pickled objects).  The reference
+        has no serialisation: every run rebuilds (``cbm_message_passing.py:22-25``)."""
+        arrays = {k: getattr(self, k).numpy() for k in self._SAVED_ARRAYS}
+        if self.col_multiplier is not None:
+            arrays["col_multiplier"] = self.col_multiplier.numpy()
+        if self._edge_index_cpu is not None:                      # needed to build the transposed operator
+            arrays["edge_index"] = self._edge_index_cpu.numpy()
+        meta = np.array([self.FORMAT_VERSION, self.num_rows, self.alpha, int(self.normalized), self.nnz, self.nnz_a,
+                         self.n_candidates, self.n_levels, int(self.is_symmetric)], np.int64)
+        np.savez(path, meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
+
+    @classmethod
+    def load(cls, path):
+        """Inverse of ``save``; runs no builder.  Consistency of the arrays is checked."""
+        with np.load(path, allow_pickle=False) as z:
+            meta = z["meta"].tolist()
+            if meta[0] != cls.FORMAT_VERSION:
+                raise ValueError(f"unsupported CBM file version {meta[0]}")
+            self = cls.__new__(cls)
+            (_, self.num_rows, self.alpha, normalized, self.nnz, self.nnz_a, self.n_candidates, self.n_levels,
+             symmetric) = meta
+            self.normalized, self.is_symmetric = bool(normalized), bool(symmetric)
+            self.deltas_format = str(z["deltas_format"])
+            for k in cls._SAVED_ARRAYS:
+                setattr(self, k, torch.from_numpy(z[k].copy()))
+            self.col_multiplier = torch.from_numpy(z["col_multiplier"].copy()) if "col_multiplier" in z.files else None
+            self._edge_index_cpu = torch.from_numpy(z["edge_index"].copy()) if "edge_index" in z.files else None
+        n = self.num_rows
+        ok = (self.rowptr.numel() == n + 1 and int(self.rowptr[-1]) == self.nnz == self.idx.numel()
+              and self.parent.numel() == n and self.order.numel() == n and self.level_off.numel() == self.n_levels + 1
+              and int(self.level_off[-1]) == n and self.mst_row.numel() == n + 2 and self.mst_col.numel() == n
+              and (self.col_multiplier is None) == (not self.normalized)
+              and (self.is_symmetric or self._edge_index_cpu is not None))
+        if not ok:
+            raise ValueError(f"{path} does not hold a consistent CBM format")
+        self.build_seconds = None
+        self._deltas, self._dev, self._transposed = None, {}, None
+        self.stream_coefficients = True
+        return self
+
     # ------------------------------------------------------------------ format views --------
     def columns(self):
         """Delta column indices (int64) and signs (+1/-1, fp32), unpacked from ``idx``."""

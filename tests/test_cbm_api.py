@@ -114,3 +114,29 @@ def test_symmetry_flag_and_transpose():
     assert torch.equal(t.deltas.to_dense(), c.deltas.to_dense().t()) or t.nnz <= 4
     und = cbm_matrix(torch.from_numpy(graphs.erdos_renyi(10, 0.5, 1)), None)
     assert und.is_symmetric and und.transposed() is und
+
+
+def test_save_and_load_round_trip(tmp_path):
+    ei = torch.from_numpy(graphs.add_self_loops(graphs.erdos_renyi(60, 0.2, 5), 60))
+    directed = torch.tensor([[0, 1, 2, 2], [1, 2, 0, 1]], dtype=torch.int32)
+    for edge_index, normalized in ((ei, True), (ei, False), (directed, True)):
+        a = cbm_matrix(edge_index, None, alpha=2, normalized=normalized)
+        path = str(tmp_path / "m.npz")
+        a.save(path)
+        b = cbm_matrix.load(path)
+        for name in ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col"):
+            assert torch.equal(getattr(a, name), getattr(b, name)), name
+        assert (a.col_multiplier is None) == (b.col_multiplier is None)
+        if normalized:
+            assert torch.equal(a.col_multiplier, b.col_multiplier)
+        for name in ("num_rows", "alpha", "normalized", "nnz", "nnz_a", "n_candidates", "n_levels", "is_symmetric"):
+            assert getattr(a, name) == getattr(b, name), name
+        assert torch.equal(a.deltas.to_dense(), b.deltas.to_dense())
+        assert b.check_format(edge_index)
+        if not b.is_symmetric:
+            assert torch.equal(b.transposed().rowptr, a.transposed().rowptr)
+    bad = dict(np.load(path))
+    bad["order"] = bad["order"][:-1]
+    np.savez(str(tmp_path / "bad.npz"), **bad)
+    with pytest.raises(ValueError):
+        cbm_matrix.load(str(tmp_path / "bad.npz"))

@@ -388,3 +388,17 @@ def test_degenerate_shapes(orc):
     assert torch.equal(x, y)
     with pytest.raises(ValueError):
         one.omp_mkl_csr_spmm_update(x, x)                             # in place is refused
+
+
+def test_alpha_tuner_reports_every_alpha_and_picks_the_fastest():
+    from cbm4gnn_amd.tuner import tune_alpha
+    w = graphs.workload("c2", scale=0.25)
+    say("alpha tuner")
+    best, rows = tune_alpha(w.edge_index, 64, alphas=(0, 4, 10_000), normalized=True, iters=10, warmup=2)
+    assert [r["alpha"] for r in rows] == [0, 4, 10_000]
+    assert rows[-1]["tree_levels"] == 1 and rows[-1]["compression_ratio"] < 1.0      # flat tree: delta = A
+    assert rows[0]["compression_ratio"] > 1.2
+    assert all(r["max_rel_err_vs_gpu_csr"] <= 1e-3 for r in rows)
+    assert best in (0, 4, 10_000)
+    fastest = min(r["cbm_ms"] for r in rows)
+    assert next(r for r in rows if r["alpha"] == best)["cbm_ms"] <= 1.02 * fastest
