@@ -1,5 +1,6 @@
-"""Full-size checks at the benchmark workload (100k nodes, d=256), where the CPU oracle is too
-slow to run per test: size-independent properties plus one CPU CSR product as the anchor."""
+"""Full-size checks at the benchmark workloads, where the CPU oracle is too slow to run per test:
+size-independent properties (linearity, determinism, exactness on integer features, agreement
+with the plain CSR product) plus one CPU CSR product as the anchor."""
 import sys
 
 import numpy as np
@@ -81,3 +82,61 @@ def test_full_size_plain_integer_features_exact(c3):
         got = torch.empty_like(x)
         mat.omp_mkl_csr_spmm_update(x, got)
         assert torch.equal(got, want)
+
+
+def test_alpha_sweep_graph_full_size_deep_chain_exact():
+    """132,534 nodes, 82.5 M non-zeros, a 2000-level chain, d = 512, plain operator, integer
+    features: every partial sum is an exact integer, so the CBM product (delta SpMM, 9 wide levels,
+    narrow levels, the 1986-level chain kernel) must equal the CSR product bit for bit."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c5")
+    print("[gpu-case] c5 full size, building", flush=True); sys.stdout.flush()
+    ei = torch.from_numpy(w.edge_index)
+    mat = cbm_matrix(ei, None, alpha=0)
+    assert mat.n_levels >= 2001 and mat.compression_ratio() > 2.0
+    x = torch.randint(0, 3, (w.n, 512), generator=torch.Generator().manual_seed(1)).float().cuda()
+    order = np.lexsort((w.edge_index[1], w.edge_index[0]))
+    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(w.edge_index[0], minlength=w.n))]).astype(np.int32)).cuda()
+    col = torch.from_numpy(w.edge_index[1][order].astype(np.int32)).cuda()
+    want = torch.empty_like(x)
+    csr_spmm(rp, col, None, x, want)
+    print("[gpu-case] c5 full size, multiply", flush=True); sys.stdout.flush()
+    got = torch.empty_like(x)
+    mat.omp_mkl_csr_spmm_update(x, got)
+    assert torch.equal(got, want)
+    # the deepest chain row really is the sum of ~2050 columns
+    deep = int(mat.order[-1])
+    assert float(got[deep].max()) > 1000.0
+    # and on real-valued features: within the plain-CSR tolerance, linear, deterministic
+    a = torch.randn((w.n, 512), generator=torch.Generator().manual_seed(2)).cuda()
+    ya = torch.empty_like(a); mat.omp_mkl_csr_spmm_update(a, ya)
+    csr_spmm(rp, col, None, a, want)
+    assert float((ya - want).abs().max() / want.abs().max()) <= 1e-3
+    yb = torch.empty_like(a); mat.omp_mkl_csr_spmm_update(a, yb)
+    assert torch.equal(ya, yb)
+
+
+def test_gcn_graph_full_size_against_gpu_csr():
+    """232,965 nodes, 114 M non-zeros (the GCN epoch workload), normalised, d = 128 and d = 41."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c4")
+    print("[gpu-case] c4 full size, building", flush=True); sys.stdout.flush()
+    ei = torch.from_numpy(w.edge_index)
+    mat = cbm_matrix(ei, None, alpha=2, normalized=True)
+    m = mat.col_multiplier
+    order = np.lexsort((w.edge_index[1], w.edge_index[0]))
+    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(w.edge_index[0], minlength=w.n))]).astype(np.int32)).cuda()
+    col = torch.from_numpy(w.edge_index[1][order].astype(np.int32)).cuda()
+    val = (m[torch.from_numpy(w.edge_index[0][order].astype(np.int64))] * m[torch.from_numpy(w.edge_index[1][order].astype(np.int64))]).cuda()
+    for d in (128, 41):
+        print("[gpu-case] c4 full size, d", d, flush=True); sys.stdout.flush()
+        x = torch.randn((w.n, d), generator=torch.Generator().manual_seed(d)).cuda()
+        want = torch.empty_like(x)
+        csr_spmm(rp, col, val, x, want)
+        got = _mul(mat, x)
+        assert float((got - want).abs().max() / want.abs().max()) <= 1e-3
+        ones = _mul(mat, torch.ones_like(x))
+        # rows of D^-1/2 (A+I) D^-1/2 applied to the all-ones vector: sum_j m_i m_j over neighbours, < sqrt(deg_i) * max m
+        assert float(ones.min()) > 0.0 and torch.isfinite(ones).all()
