@@ -47,10 +47,10 @@ HIP_SYMBOLS = {
     "cbm_set_spmm_kernel": (C.c_int, [C.c_int]),
     "cbm_spmm_summation_groups": (C.c_int, [_I32, _I64, _I64, _P, _P]),
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),
-    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
-    "cbm_spmm_update_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
-    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_update_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
 }
 
 _host = None

@@ -66,6 +66,20 @@ def _check_f32_matrix(t, name, n=None):
         raise ValueError(f"{name} has overlapping rows (stride {t.stride(0)} < width {t.size(1)})")
 
 
+# Rows with fewer delta entries than this on average do not repay the slab-major copy of X
+_MIN_ENTRIES_PER_ROW_FOR_RELAYOUT = 24
+
+
+def _workspace(x, nnz):
+    """Device scratch for the slab-major copy of ``x`` (n * d floats), or None when the copy
+    would not pay off or the width is not one the slab kernel takes.  Allocated from torch's
+    stream-ordered caching allocator, so handing it to an asynchronous launch is safe."""
+    n, d = x.shape
+    if d % 32 != 0 or n == 0 or nnz < _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT * n:
+        return None
+    return torch.empty(n * d, dtype=torch.float32, device=x.device)
+
+
 def _ld(t):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
 
@@ -352,13 +366,14 @@ class cbm_matrix:
         if yd.device != xd.device:
             raise ValueError("rhs and dst are on different devices")
         st = self._device_arrays(xd.device)
+        ws = _workspace(xd, self.nnz)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None,
                 _ptr(st["parent"]) if scale_roots else None,
                 _ptr(st["sched_scaled"] if (scale_roots and use_m) else st["sched"]), _ptr(xd), _ptr(yd),
-                n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
+                _ptr(ws), n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
         _lib.check(rc, "cbm_spmm_f32")
         if yd is not y:
             y.copy_(yd)
@@ -398,12 +413,13 @@ class cbm_matrix:
         if yd.data_ptr() == xd.data_ptr():
             raise ValueError("dst must not alias rhs")
         st = self._device_arrays(xd.device)
+        ws = _workspace(xd, self.nnz)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None, _ptr(st["parent"]),
                 _ptr(st["sched_scaled"] if use_m else st["sched"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
-                _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
+                _ptr(xd), _ptr(yd), _ptr(ws), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
         _lib.check(rc, "cbm_spmm_update_f32")
         if yd is not y:
             y.copy_(yd)
@@ -520,7 +536,8 @@ def csr_spmm(rowptr, col, val, x, y, sched=None):
         raise RuntimeError("lhs_val (NOT torch::kFloat32)")
     if not (x.is_cuda and y.is_cuda and rowptr.is_cuda and col.is_cuda):
         raise ValueError("csr_spmm expects device tensors")
+    ws = _workspace(x, col.numel())
     with torch.cuda.device(x.device):
-        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), _ptr(sched), _ptr(x), _ptr(y),
+        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), _ptr(sched), _ptr(x), _ptr(y), _ptr(ws),
                                          n, x.size(1), _ld(x), _ld(y), _stream(x.device))
     _lib.check(rc, "csr_spmm_f32")

@@ -35,6 +35,9 @@ namespace {
 #ifndef CBM_UNROLL_CH1
 #define CBM_UNROLL_CH1 8
 #endif
+#ifndef CBM_SLAB_ROUNDS
+#define CBM_SLAB_ROUNDS 8                  // load instructions in flight per wave in the slab kernel
+#endif
 #ifndef CBM_XCD_REMAP
 #define CBM_XCD_REMAP 1
 #endif
@@ -219,7 +222,11 @@ template <int LPE, bool PACKED, int U>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
-    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int64_t ldx, int64_t ldz) {
+    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int64_t x_slab_stride,
+    int64_t x_row_stride, int64_t ldz) {
+    // X is addressed as X[slab * x_slab_stride + row * x_row_stride + column in slab]: the caller's
+    // row-major matrix (slab stride = slab width, row stride = ldx) or the slab-major copy made by
+    // relayout_slabs (slab stride = n * slab width, row stride = slab width).
     constexpr int kSlab = LPE * 4;                         // floats per slab
     constexpr int kStep = kWave / LPE;                     // entries per wave instruction
     const int lane = threadIdx.x & (kWave - 1);
@@ -245,7 +252,7 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
         }
     }
     for (int slab = slab0; slab < n_slabs; slab += slab_step) {
-        const float* __restrict__ Xs = X + slab * kSlab + li * 4;
+        const float* __restrict__ Xs = X + slab * x_slab_stride + li * 4;
         float* __restrict__ Zs = Z + slab * kSlab + li * 4;
         // row descriptor {start, end, row, bits(left scale)} fetched one row ahead of its use
         auto fetch = [&](int i) -> int4 {
@@ -298,7 +305,7 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
                             f[u] = f[u] == 0.0f ? 0.0f : g;
                         }
                     }
-                    load_vec<4>(Xs + (int64_t)c * ldx, x[u]);
+                    load_vec<4>(Xs + (int64_t)c * x_row_stride, x[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < UU; u++)
@@ -327,6 +334,20 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
             }
         }
     }
+}
+
+// Slab-major copy of X: W[s][r][0 .. slab) = X[r][s * slab .. (s + 1) * slab).  With the caller's
+// row-major X a slab's lines sit a whole row (a power of two for the usual widths) apart, which
+// maps them onto a fraction of an XCD's L2 channels; in the copy they are consecutive lines.
+// One thread per float4.
+__global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n,
+                                                      int d4, int slab4, int64_t ldx) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (int64_t)n * d4) return;
+    const int r = (int)(t / d4), q = (int)(t % d4);
+    const int s = q / slab4, w = q % slab4;
+    const float4 v = *reinterpret_cast<const float4*>(X + (int64_t)r * ldx + 4 * q);
+    *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * slab4 + w) * 4) = v;
 }
 
 // coef[k] = +-m[col(k)]: the packed entries expanded once so the SpMM can stream coefficients.
@@ -580,8 +601,8 @@ int resident_groups_per_xcd(K kernel) {
 
 template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, const float* m,
-                const int32_t* parent, const int32_t* sched, const float* X, float* Z, int32_t n, int32_t d,
-                int64_t ldx, int64_t ldz, hipStream_t s) {
+                const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace, int32_t n,
+                int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
     if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
@@ -591,8 +612,16 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
     const int4* sc = reinterpret_cast<const int4*>(sched);
     if (const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z)) {
         const int n_slabs = d / (lpe * 4);
-        static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, 8>);
-        static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, 8>);
+        const float* Xg = X;                              // what the gather reads
+        int64_t x_slab_stride = lpe * 4, x_row_stride = ldx;
+        if (workspace && aligned(workspace, 16) && workspace != Z && workspace != X) {
+            const int64_t units = (int64_t)n * (d / 4);
+            hipLaunchKernelGGL(relayout_slabs, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, X, workspace, n,
+                               d / 4, lpe, ldx);
+            Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
+        }
+        static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>);
+        static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>);
         int G = lpe == 8 ? g8 : g16;
         if (G > 0) {
             // no more waves than rows: with fewer rows than resident waves shrink the grid
@@ -601,11 +630,11 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
             if (G > need) G = need;
             const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
             if (lpe == 8)
-                hipLaunchKernelGGL((spmm_slab_per_xcd<8, PACKED, 8>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   X, Z, n, n_slabs, ldx, ldz);
+                hipLaunchKernelGGL((spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
+                                   Xg, Z, n, n_slabs, x_slab_stride, x_row_stride, ldz);
             else
-                hipLaunchKernelGGL((spmm_slab_per_xcd<16, PACKED, 8>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   X, Z, n, n_slabs, ldx, ldz);
+                hipLaunchKernelGGL((spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
+                                   Xg, Z, n, n_slabs, x_slab_stride, x_row_stride, ldz);
             return check_launch();
         }
     }
@@ -708,11 +737,11 @@ const char* cbm_status_string(int status) {
 }
 
 int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
-                 const int32_t* parent, const int32_t* row_sched, const float* X, float* Z, int32_t n, int32_t d,
-                 int64_t ldx, int64_t ldz, void* stream) {
+                 const int32_t* parent, const int32_t* row_sched, const float* X, float* Z, float* workspace,
+                 int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
     if (!idx && n > 0) return CBM_ERR_NULL;
     if (coef && !m) return CBM_ERR_NULL;                 // coef is the expansion of m, not a substitute
-    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, n, d, ldx, ldz,
+    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, workspace, n, d, ldx, ldz,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -739,10 +768,11 @@ int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_
 }
 
 int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_sched,
-                 const float* X, float* Y, int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream) {
+                 const float* X, float* Y, float* workspace, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
+                 void* stream) {
     if (!col && n > 0) return CBM_ERR_NULL;
     return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_sched,
-                              X, Y, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
+                              X, Y, workspace, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
 }
 
 int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t* level_off_dev,
@@ -760,11 +790,11 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
 
 int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
                         const int32_t* parent, const int32_t* row_sched, const int32_t* order, const int32_t* level_off_dev,
-                        const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, int32_t n,
-                        int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
+                        const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, float* workspace,
+                        int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, n, d, ldx, ldy, stream);
+    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, workspace, n, d, ldx, ldy, stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,

@@ -126,11 +126,15 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * cbm_extensions.cpp:910-940, folded into the producer).  row_sched, if not NULL, is the row
  * schedule written by cbm_schedule_rows (4 int32 per row, 16-byte aligned): rows are then
  * processed in that order, rowptr is not read (may be NULL) and the left scale comes from it.
+ * workspace, if not NULL, is caller-owned device memory for n * d floats (16-byte aligned, disjoint
+ * from X and Z): widths the slab kernel takes are first copied there slab-major, so that the
+ * gathered 128-byte lines of a slab are consecutive in memory instead of a row apart; the result
+ * is bit-identical, the copy pays off when rows have more than a few entries.
  * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
 int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
                  const int32_t* parent_dev, const int32_t* row_sched_dev, const float* X_dev, float* Z_dev,
-                 int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
+                 float* workspace_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
  *   m == NULL : Y[v,:] += Y[parent[v],:]
@@ -155,14 +159,14 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, cons
                         const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
                         const int32_t* order_dev,
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
-                        const float* X_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
-                        int32_t flags, void* stream);
+                        const float* X_dev, float* Y_dev, float* workspace_dev, int32_t n, int32_t d,
+                        int64_t ldx, int64_t ldy, int32_t flags, void* stream);
 
 /* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
 int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, const float* val_dev,
-                 const int32_t* row_sched_dev, const float* X_dev, float* Y_dev, int32_t n, int32_t d,
-                 int64_t ldx, int64_t ldy, void* stream);
+                 const int32_t* row_sched_dev, const float* X_dev, float* Y_dev, float* workspace_dev,
+                 int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream);
 
 #ifdef __cplusplus
 }

@@ -315,16 +315,17 @@ def test_c_abi_status_codes_on_device_calls():
     rp = torch.zeros(n + 1, dtype=torch.int32, device="cuda"); idx = torch.zeros(1, dtype=torch.int32, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
     say("status codes")
-    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), n, d, d, d, None) == 1
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), n, d, d - 1, d, None) == 3
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), n, d, d, d, None) == 1   # coef without m
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), n, d, d, d, None) == 0   # empty rows -> zeros
+    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), None, n, d, d, d, None) == 1
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, n, d, d - 1, d, None) == 3
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), None, n, d, d, d, None) == 1   # coef without m
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(x), None, n, d, d, d, None) == 3   # in place
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, n, d, d, d, None) == 0   # empty rows -> zeros
     lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
     par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
     lo = (C.c_int32 * 2)(0, n)
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 0
-    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), n, d, d, d, 0, None) == 3
+    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), None, n, d, d, d, 0, None) == 3
     torch.cuda.synchronize()
     assert (y == 0).all()
 
