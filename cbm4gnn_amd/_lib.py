@@ -13,6 +13,7 @@ from .build import HIP_LIB, HOST_LIB
 
 CBM_OK = 0
 CBM_PROP_SCALE_ROOTS = 1
+CBM_SPMM_WORKSPACE_READY = 1
 
 
 class CbmLibraryError(RuntimeError):
@@ -46,11 +47,13 @@ HIP_SYMBOLS = {
     "cbm_status_string": (C.c_char_p, [C.c_int]),
     "cbm_set_spmm_kernel": (C.c_int, [C.c_int]),
     "cbm_spmm_summation_groups": (C.c_int, [_I32, _I64, _I64, _P, _P]),
+    "cbm_spmm_workspace_floats": (C.c_int64, [_I32, _I32, _I64, _I64, _P, _P]),
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),
-    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
+    "cbm_relayout_slabs_f32": (C.c_int, [_P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
-    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
 }
 
 _host = None

@@ -32,7 +32,7 @@ from . import _lib
 
 warnings.filterwarnings("ignore", message="Sparse CSR tensor support is in beta state", category=UserWarning)
 
-__all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels", "schedule_rows"]
+__all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels", "schedule_rows", "relayout_slabs"]
 
 
 def _ptr(t):
@@ -70,14 +70,15 @@ def _check_f32_matrix(t, name, n=None):
 _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT = 24
 
 
-def _workspace(x, nnz):
-    """Device scratch for the slab-major copy of ``x`` (n * d floats), or None when the copy
-    would not pay off or the width is not one the slab kernel takes.  Allocated from torch's
+def _workspace(x, y, nnz):
+    """Device scratch for the slab-major copy of ``x``, or None when the library would not use it
+    for this shape or the rows are too short for the copy to pay off.  Allocated from torch's
     stream-ordered caching allocator, so handing it to an asynchronous launch is safe."""
     n, d = x.shape
-    if d % 32 != 0 or n == 0 or nnz < _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT * n:
+    if n == 0 or nnz < _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT * n:
         return None
-    return torch.empty(n * d, dtype=torch.float32, device=x.device)
+    floats = _lib.hip_lib().cbm_spmm_workspace_floats(n, d, _ld(x), _ld(y), _ptr(x), _ptr(y))
+    return torch.empty(floats, dtype=torch.float32, device=x.device) if floats > 0 else None
 
 
 def _ld(t):
@@ -194,6 +195,7 @@ class cbm_matrix:
         self._deltas = None
         self._dev = {}
         self.stream_coefficients = True     # False: gather m[col] in the kernel, 4 B/entry less device memory
+        self.relayout = True                # False: gather from the caller's row-major X, no n*d scratch per call
         self._transposed = None
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
 
@@ -240,6 +242,7 @@ class cbm_matrix:
         self.build_seconds = None
         self._deltas, self._dev, self._transposed = None, {}, None
         self.stream_coefficients = True
+        self.relayout = True
         return self
 
     # ------------------------------------------------------------------ format views --------
@@ -352,7 +355,7 @@ class cbm_matrix:
         return t.to("cuda"), True
 
     # ------------------------------------------------------------------ kernels -------------
-    def _run_spmm(self, x, y, use_m, scale_roots):
+    def _run_spmm(self, x, y, use_m, scale_roots, workspace=None, workspace_ready=False):
         n = self.num_rows
         _check_f32_matrix(x, "rhs", n)
         _check_f32_matrix(y, "dst", n)
@@ -366,14 +369,15 @@ class cbm_matrix:
         if yd.device != xd.device:
             raise ValueError("rhs and dst are on different devices")
         st = self._device_arrays(xd.device)
-        ws = _workspace(xd, self.nnz)
+        ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None,
                 _ptr(st["parent"]) if scale_roots else None,
                 _ptr(st["sched_scaled"] if (scale_roots and use_m) else st["sched"]), _ptr(xd), _ptr(yd),
-                _ptr(ws), n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
+                _ptr(ws), _lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0, n, x.size(1), _ld(xd), _ld(yd),
+                _stream(xd.device))
         _lib.check(rc, "cbm_spmm_f32")
         if yd is not y:
             y.copy_(yd)
@@ -413,7 +417,7 @@ class cbm_matrix:
         if yd.data_ptr() == xd.data_ptr():
             raise ValueError("dst must not alias rhs")
         st = self._device_arrays(xd.device)
-        ws = _workspace(xd, self.nnz)
+        ws = _workspace(xd, yd, self.nnz) if self.relayout else None
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
@@ -522,6 +526,20 @@ class CBMMatmul(torch.autograd.Function):
         return gx, None, None
 
 
+def relayout_slabs(x):
+    """Slab-major copy of ``x`` for ``cbm_spmm_f32(..., CBM_SPMM_WORKSPACE_READY)``, or None when the
+    library makes no such copy for this shape."""
+    n, d = x.shape
+    floats = _lib.hip_lib().cbm_spmm_workspace_floats(n, d, _ld(x), d, _ptr(x), _ptr(x))
+    if floats <= 0:
+        return None
+    ws = torch.empty(floats, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.hip_lib().cbm_relayout_slabs_f32(_ptr(x), _ptr(ws), n, d, _ld(x), _stream(x.device))
+    _lib.check(rc, "cbm_relayout_slabs_f32")
+    return ws
+
+
 def csr_spmm(rowptr, col, val, x, y, sched=None):
     """Plain CSR SpMM ``y = A @ x`` on the GPU: the hand-written baseline the CBM multiply is
     measured against (role of ``omp_s_spmm_csr_int32``, ``cbm_extensions.cpp:1707-1755``).
@@ -536,8 +554,8 @@ def csr_spmm(rowptr, col, val, x, y, sched=None):
         raise RuntimeError("lhs_val (NOT torch::kFloat32)")
     if not (x.is_cuda and y.is_cuda and rowptr.is_cuda and col.is_cuda):
         raise ValueError("csr_spmm expects device tensors")
-    ws = _workspace(x, col.numel())
+    ws = _workspace(x, y, col.numel())
     with torch.cuda.device(x.device):
         rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), _ptr(sched), _ptr(x), _ptr(y), _ptr(ws),
-                                         n, x.size(1), _ld(x), _ld(y), _stream(x.device))
+                                         0, n, x.size(1), _ld(x), _ld(y), _stream(x.device))
     _lib.check(rc, "csr_spmm_f32")

@@ -561,6 +561,10 @@ inline int pick_slab_lanes(int d, int64_t ld_a, int64_t ld_b, const void* pa, co
     return (n_slabs % kXcds == 0 || kXcds % n_slabs == 0) ? lpe : 0;
 }
 
+// The slab-major copy of X pays off for 128-byte slabs (8 lanes per entry); with 256-byte slabs
+// it measured within +-3 %.
+constexpr int kRelayoutLanes = 8;
+
 #define CBM_DISPATCH_TILING(T, LAUNCH)                                              \
     do {                                                                            \
         if ((T).full) { CBM_DISPATCH_VC(T, true, LAUNCH); }                         \
@@ -599,10 +603,18 @@ int resident_groups_per_xcd(K kernel) {
     return (cus / kXcds) * per_cu;
 }
 
+inline void launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int lpe, int64_t ldx,
+                            hipStream_t s) {
+    const int64_t units = (int64_t)n * (d / 4);
+    hipLaunchKernelGGL(relayout_slabs, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, X, workspace, n, d / 4,
+                       lpe, ldx);
+}
+
 template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, const float* m,
-                const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace, int32_t n,
-                int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
+                const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
+                int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
+    if (flags & ~CBM_SPMM_WORKSPACE_READY) return CBM_ERR_UNSUPPORTED;
     if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
@@ -610,15 +622,17 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
     if (X == Z) return CBM_ERR_SHAPE;                    // rows of X are gathered while rows of Z are written
     if (n == 0 || d == 0) return CBM_OK;
     const int4* sc = reinterpret_cast<const int4*>(sched);
-    if (const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z)) {
+    const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z);
+    if (!lpe && (flags & CBM_SPMM_WORKSPACE_READY)) return CBM_ERR_SHAPE;
+    if (lpe) {
         const int n_slabs = d / (lpe * 4);
         const float* Xg = X;                              // what the gather reads
         int64_t x_slab_stride = lpe * 4, x_row_stride = ldx;
-        if (workspace && aligned(workspace, 16) && workspace != Z && workspace != X) {
-            const int64_t units = (int64_t)n * (d / 4);
-            hipLaunchKernelGGL(relayout_slabs, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, X, workspace, n,
-                               d / 4, lpe, ldx);
+        if (workspace && lpe == kRelayoutLanes && aligned(workspace, 16) && workspace != Z && workspace != X) {
+            if (!(flags & CBM_SPMM_WORKSPACE_READY)) launch_relayout(X, workspace, n, d, lpe, ldx, s);
             Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
+        } else if (flags & CBM_SPMM_WORKSPACE_READY) {
+            return CBM_ERR_SHAPE;                         // told to read a copy that this shape never makes
         }
         static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>);
         static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>);
@@ -738,11 +752,20 @@ const char* cbm_status_string(int status) {
 
 int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
                  const int32_t* parent, const int32_t* row_sched, const float* X, float* Z, float* workspace,
-                 int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
+                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
     if (!idx && n > 0) return CBM_ERR_NULL;
     if (coef && !m) return CBM_ERR_NULL;                 // coef is the expansion of m, not a substitute
-    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, workspace, n, d, ldx, ldz,
+    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, workspace, flags, n, d, ldx, ldz,
                              static_cast<hipStream_t>(stream));
+}
+
+int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, void* stream) {
+    if (!X || !workspace) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (pick_slab_lanes(d, ldx, d, X, workspace) != kRelayoutLanes || X == workspace) return CBM_ERR_SHAPE;
+    if (n == 0) return CBM_OK;
+    launch_relayout(X, workspace, n, d, kRelayoutLanes, ldx, static_cast<hipStream_t>(stream));
+    return check_launch();
 }
 
 int cbm_set_spmm_kernel(int kind) {
@@ -754,6 +777,11 @@ int cbm_set_spmm_kernel(int kind) {
 int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
     const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z);
     return lpe ? kWave / lpe : 1;
+}
+
+int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
+    if (n <= 0 || d <= 0) return 0;
+    return pick_slab_lanes(d, ldx, ldz, X, Z) == kRelayoutLanes ? (int64_t)n * d : 0;
 }
 
 int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_t nnz, void* stream) {
@@ -768,11 +796,11 @@ int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_
 }
 
 int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_sched,
-                 const float* X, float* Y, float* workspace, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
-                 void* stream) {
+                 const float* X, float* Y, float* workspace, int32_t flags, int32_t n, int32_t d, int64_t ldx,
+                 int64_t ldy, void* stream) {
     if (!col && n > 0) return CBM_ERR_NULL;
     return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_sched,
-                              X, Y, workspace, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
+                              X, Y, workspace, flags, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
 }
 
 int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t* level_off_dev,
@@ -794,7 +822,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float*
                         int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, workspace, n, d, ldx, ldy, stream);
+    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, workspace, 0, n, d, ldx, ldy, stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,

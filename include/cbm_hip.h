@@ -36,6 +36,11 @@ enum {
     CBM_ERR_UNSUPPORTED = 6  /* valid request this build does not implement        */
 };
 
+/* flags of cbm_spmm_f32 / csr_spmm_f32 */
+enum {
+    CBM_SPMM_WORKSPACE_READY = 1 /* workspace already holds cbm_relayout_slabs_f32(X): do not copy again */
+};
+
 /* flags of cbm_propagate_f32 / cbm_spmm_update_f32 */
 enum {
     CBM_PROP_SCALE_ROOTS = 1  /* normalised only: first do Y[r,:] *= m[r] for children of the root */
@@ -114,6 +119,10 @@ int cbm_set_spmm_kernel(int kind);
  * summation order bit for bit.  No reference counterpart (MKL does not document its order). */
 int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
 
+/* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 can use for this
+ * shape (n * d when the slab-major copy of X applies, else 0).  The workspace stays optional. */
+int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
+
 /* coef[k] = +-m[column of entry k] for the packed entries idx[0 .. nnz): the delta VALUES of the
  * reference's normalised builder (cbm_extensions.cpp:504-585), expanded on the device once so
  * that cbm_spmm_f32 can stream them instead of gathering m[col] per entry.  Optional. */
@@ -134,7 +143,14 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
 int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
                  const int32_t* parent_dev, const int32_t* row_sched_dev, const float* X_dev, float* Z_dev,
-                 float* workspace_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
+                 float* workspace_dev, int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz,
+                 void* stream);
+
+/* The slab-major copy of X that cbm_spmm_f32 / csr_spmm_f32 make into their workspace, as a call
+ * of its own: several multiplies by different matrices with the SAME X can then share one copy
+ * (pass the workspace with CBM_SPMM_WORKSPACE_READY).  CBM_ERR_SHAPE if
+ * cbm_spmm_workspace_floats is 0 for this shape. */
+int cbm_relayout_slabs_f32(const float* X_dev, float* workspace_dev, int32_t n, int32_t d, int64_t ldx, void* stream);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
  *   m == NULL : Y[v,:] += Y[parent[v],:]
@@ -166,7 +182,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, cons
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
 int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, const float* val_dev,
                  const int32_t* row_sched_dev, const float* X_dev, float* Y_dev, float* workspace_dev,
-                 int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream);
+                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream);
 
 #ifdef __cplusplus
 }

@@ -315,11 +315,12 @@ def test_c_abi_status_codes_on_device_calls():
     rp = torch.zeros(n + 1, dtype=torch.int32, device="cuda"); idx = torch.zeros(1, dtype=torch.int32, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
     say("status codes")
-    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), None, n, d, d, d, None) == 1
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, n, d, d - 1, d, None) == 3
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), None, n, d, d, d, None) == 1   # coef without m
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(x), None, n, d, d, d, None) == 3   # in place
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, n, d, d, d, None) == 0   # empty rows -> zeros
+    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d - 1, d, None) == 3
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1   # coef without m
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(x), None, 0, n, d, d, d, None) == 3   # in place
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 0   # empty rows -> zeros
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 1, n, d, d, d, None) == 3   # d = 4 never has a slab-major copy
     lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
     par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
@@ -403,3 +404,23 @@ def test_alpha_tuner_reports_every_alpha_and_picks_the_fastest():
     assert best in (0, 4, 10_000)
     fastest = min(r["cbm_ms"] for r in rows)
     assert next(r for r in rows if r["alpha"] == best)["cbm_ms"] <= 1.02 * fastest
+
+
+def test_shared_slab_major_copy(orc):
+    """cbm_relayout_slabs_f32 once, then two different matrices multiply the same X from it."""
+    from cbm4gnn_amd.cbm import relayout_slabs
+    n, d = 600, 128
+    ei = graphs.add_self_loops(graphs.sbm(n, 6, 0.3, 0.01, seed=4), n)
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(4)).cuda()
+    say("shared relayout")
+    ws = relayout_slabs(x)
+    assert ws is not None and ws.numel() == n * d
+    # the copy is what it says: W[s][r][:] = X[r][32 s : 32 s + 32]
+    assert torch.equal(ws.view(d // 32, n, 32).permute(1, 0, 2).reshape(n, d), x)
+    for alpha in (0, 1000):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=True)
+        want = torch.empty_like(x); mat._run_spmm(x, want, use_m=True, scale_roots=True)
+        got = torch.empty_like(x); mat._run_spmm(torch.zeros_like(x), got, use_m=True, scale_roots=True,
+                                                 workspace=ws, workspace_ready=True)     # X itself is not read
+        assert torch.equal(got, want)
+    assert relayout_slabs(torch.zeros((n, 41), device="cuda")) is None
