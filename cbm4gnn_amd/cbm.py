@@ -347,7 +347,7 @@ class cbm_matrix:
         self._device_arrays(device)
         return self
 
-    def _stage(self, t, like=None):
+    def _stage(self, t):
         """(device tensor, needs_copy_back).  CPU tensors are staged through the current GPU."""
         if t.is_cuda:
             return t, False

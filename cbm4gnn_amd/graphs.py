@@ -283,8 +283,9 @@ def workload(name: str, seed: int = 0, scale: float = 1.0) -> Workload:
     if name == "c4":
         n = max(500, int(232_965 * scale)); blocks = 50
         blk = n / blocks
-        p_in = min(1.0, 0.9 * 490.0 * min(1.0, scale) / (blk - 1.0)) if scale < 1.0 else 0.9 * 490.0 / (blk - 1.0)
-        p_out = 0.1 * 490.0 * min(1.0, scale) / (n - blk)
+        mean_deg = 490.0 * min(1.0, scale)                   # 90 % of it inside the block
+        p_in = min(1.0, 0.9 * mean_deg / (blk - 1.0))
+        p_out = 0.1 * mean_deg / (n - blk)
         ei = add_self_loops(sbm(n, blocks, p_in, p_out, seed), n)
         return Workload("c4", ei, n, 602, True, (2,), "normal",
                         "SBM 50 blocks, mean degree ~490 (90% intra), A+I normalised, GCN 602-128-41")
