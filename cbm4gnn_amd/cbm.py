@@ -354,6 +354,13 @@ class cbm_matrix:
         _require_gpu()
         return t.to("cuda"), True
 
+    def summation_groups(self, x, y=None):
+        """Interleaved partial sums per output element that the next multiply of ``x`` into ``y``
+        keeps (1 = entries accumulate strictly in order); lets a checker reproduce the fp32 order."""
+        y = x if y is None else y
+        use_ws = self.relayout and x.size(0) > 0 and self.nnz >= _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT * x.size(0)
+        return int(_lib.hip_lib().cbm_spmm_summation_groups(x.size(1), _ld(x), _ld(y), _ptr(x), _ptr(y), int(use_ws)))
+
     # ------------------------------------------------------------------ kernels -------------
     def _run_spmm(self, x, y, use_m, scale_roots, workspace=None, workspace_ready=False):
         n = self.num_rows
@@ -527,10 +534,10 @@ class CBMMatmul(torch.autograd.Function):
 
 
 def relayout_slabs(x):
-    """Slab-major copy of ``x`` for ``cbm_spmm_f32(..., CBM_SPMM_WORKSPACE_READY)``, or None when the
-    library makes no such copy for this shape."""
+    """Slab-major copy of ``x`` for ``cbm_spmm_f32(..., CBM_SPMM_WORKSPACE_READY)`` (None for an
+    empty matrix)."""
     n, d = x.shape
-    floats = _lib.hip_lib().cbm_spmm_workspace_floats(n, d, _ld(x), d, _ptr(x), _ptr(x))
+    floats = _lib.hip_lib().cbm_relayout_floats(n, d)
     if floats <= 0:
         return None
     ws = torch.empty(floats, dtype=torch.float32, device=x.device)

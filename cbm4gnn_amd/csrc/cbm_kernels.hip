@@ -222,8 +222,11 @@ template <int LPE, bool PACKED, int U>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
-    const float* __restrict__ X, float* __restrict__ Z, int n, int n_slabs, int64_t x_slab_stride,
-    int64_t x_row_stride, int64_t ldz) {
+    const float* __restrict__ X, float* __restrict__ Z, int n, int d, int vec_out, int n_slabs,
+    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz) {
+    // d is the true feature width: slabs may reach past it (odd widths are zero-padded in the
+    // slab-major copy) and nothing is stored beyond column d; vec_out says that rows of Z are
+    // float4-addressable.
     // X is addressed as X[slab * x_slab_stride + row * x_row_stride + column in slab]: the caller's
     // row-major matrix (slab stride = slab width, row stride = ldx) or the slab-major copy made by
     // relayout_slabs (slab stride = n * slab width, row stride = slab width).
@@ -330,24 +333,46 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 #pragma unroll
                         for (int e = 0; e < 4; e++) acc[e] *= row_scale;
                 }
-                store_vec<4>(Zs + (int64_t)row * ldz, acc);
+                const int col = slab * kSlab + li * 4;
+                float* __restrict__ zr = Zs + (int64_t)row * ldz;
+                if (vec_out) {
+                    if (col < d) store_vec<4>(zr, acc);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (col + e < d) zr[e] = acc[e];
+                }
             }
         }
     }
 }
 
-// Slab-major copy of X: W[s][r][0 .. slab) = X[r][s * slab .. (s + 1) * slab).  With the caller's
-// row-major X a slab's lines sit a whole row (a power of two for the usual widths) apart, which
-// maps them onto a fraction of an XCD's L2 channels; in the copy they are consecutive lines.
-// One thread per float4.
-__global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n,
-                                                      int d4, int slab4, int64_t ldx) {
+// Slab-major copy of X: W[s][r][0 .. 32) = X[r][32 s .. 32 s + 32), zero where the column is >= d
+// (n_slabs * 32 may exceed d).  With the caller's row-major X a slab's lines sit a whole row (a
+// power of two for the usual widths) apart, which maps them onto a fraction of an XCD's L2
+// channels, and rows of odd widths are not line-aligned at all; in the copy the lines of a slab
+// are consecutive and aligned.  One thread per float4 of the copy.
+template <bool VEC_IN>
+__global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n, int d,
+                                                      int n_slabs, int64_t ldx) {
+    constexpr int kSlab4 = 8;                              // float4 per 128-byte slab
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= (int64_t)n * d4) return;
-    const int r = (int)(t / d4), q = (int)(t % d4);
-    const int s = q / slab4, w = q % slab4;
-    const float4 v = *reinterpret_cast<const float4*>(X + (int64_t)r * ldx + 4 * q);
-    *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * slab4 + w) * 4) = v;
+    const int row4 = n_slabs * kSlab4;
+    if (t >= (int64_t)n * row4) return;
+    const int r = (int)(t / row4), q = (int)(t % row4);
+    const int s = q / kSlab4, w = q % kSlab4;
+    const int col = 4 * q;
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const float* __restrict__ src = X + (int64_t)r * ldx + col;
+    if constexpr (VEC_IN) {
+        if (col < d) v = *reinterpret_cast<const float4*>(src);
+    } else {
+        if (col + 0 < d) v.x = src[0];
+        if (col + 1 < d) v.y = src[1];
+        if (col + 2 < d) v.z = src[2];
+        if (col + 3 < d) v.w = src[3];
+    }
+    *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * kSlab4 + w) * 4) = v;
 }
 
 // coef[k] = +-m[col(k)]: the packed entries expanded once so the SpMM can stream coefficients.
@@ -548,22 +573,47 @@ inline Tiling pick_tiling(int d, int64_t ld_a, int64_t ld_b, const void* pa, con
 // SpMM kernel choice: 0 = automatic, 1 = always one wave per row, 2 = slabs whenever the shape allows
 int g_spmm_kernel = 0;
 
-// Lanes per delta entry of the slab kernel (8 -> 128-byte slabs, 16 -> 256-byte slabs), or 0 when
-// the wave-per-row kernel should run: d must split into whole slabs whose count divides, or is a
-// multiple of, the 8 XCDs, and rows must be float4-addressable.  A wider slab is taken only when
-// it still leaves one slab per XCD.
-inline int pick_slab_lanes(int d, int64_t ld_a, int64_t ld_b, const void* pa, const void* pb) {
-    if (g_spmm_kernel == 1) return 0;
-    if (d % 32 != 0 || ld_a % 4 != 0 || ld_b % 4 != 0 || !aligned(pa, 16) || !aligned(pb, 16)) return 0;
-    int lpe = 8;
-    if (d % 64 == 0 && d / 64 >= kXcds) lpe = 16;
-    const int n_slabs = d / (lpe * 4);
-    return (n_slabs % kXcds == 0 || kXcds % n_slabs == 0) ? lpe : 0;
+// How a multiply of feature width d runs.
+struct SlabPlan {
+    int lpe = 0;            // lanes per delta entry: 8 -> 128-byte slabs, 16 -> 256-byte slabs, 0 -> one wave per row
+    int n_slabs = 0;        // slabs the kernel walks (odd widths: padded count)
+    bool relayout = false;  // the gather reads the slab-major copy in the workspace
+    bool vec_out = false;   // rows of Z are float4-addressable
+};
+
+// Slabs of the slab-major copy: ceil(d / 32), rounded up to 1, 2, 4 or 8 when below 8 so that
+// the XCDs sharing a slab split evenly.
+inline int padded_slab_count(int d) {
+    int ns = (d + 31) / 32;
+    if (ns < kXcds) { int q = 1; while (q < ns) q *= 2; ns = q; }
+    return ns;
 }
 
-// The slab-major copy of X pays off for 128-byte slabs (8 lanes per entry); with 256-byte slabs
-// it measured within +-3 %.
-constexpr int kRelayoutLanes = 8;
+// Widths that split into whole 128- or 256-byte slabs whose count divides, or is a multiple of,
+// the 8 XCDs run on the slab kernel directly (a wider slab is taken only when it still leaves
+// one slab per XCD; the slab-major copy pays off for 128-byte slabs only: with 256-byte slabs it
+// measured within +-3 %).  Any other width or alignment runs on the slab kernel through the
+// zero-padded slab-major copy when the caller brought a workspace, else one wave per row.
+// force_copy: the caller already made the copy (always 128-byte slabs, padded count).
+inline SlabPlan plan_slabs(int d, int64_t ldx, int64_t ldz, const void* X, const void* Z, bool have_workspace,
+                           bool force_copy) {
+    SlabPlan p;
+    if (g_spmm_kernel == 1 && !force_copy) return p;
+    const bool x_vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16);
+    p.vec_out = d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16);
+    if (!force_copy && d % 32 == 0 && x_vec && p.vec_out) {
+        int lpe = 8;
+        if (d % 64 == 0 && d / 64 >= kXcds) lpe = 16;
+        const int ns = d / (lpe * 4);
+        if (ns % kXcds == 0 || kXcds % ns == 0) {
+            p.lpe = lpe; p.n_slabs = ns; p.relayout = have_workspace && lpe == 8;
+            return p;
+        }
+    }
+    if (!have_workspace && !force_copy) return p;
+    p.lpe = 8; p.n_slabs = padded_slab_count(d); p.relayout = true;
+    return p;
+}
 
 #define CBM_DISPATCH_TILING(T, LAUNCH)                                              \
     do {                                                                            \
@@ -603,11 +653,16 @@ int resident_groups_per_xcd(K kernel) {
     return (cus / kXcds) * per_cu;
 }
 
-inline void launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int lpe, int64_t ldx,
-                            hipStream_t s) {
-    const int64_t units = (int64_t)n * (d / 4);
-    hipLaunchKernelGGL(relayout_slabs, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, X, workspace, n, d / 4,
-                       lpe, ldx);
+inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s) {
+    const int ns = padded_slab_count(d);
+    const int64_t blocks = ((int64_t)n * ns * 8 + 255) / 256;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    const dim3 grid((unsigned)blocks), block(256);
+    if (d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16))
+        hipLaunchKernelGGL(relayout_slabs<true>, grid, block, 0, s, X, workspace, n, d, ns, ldx);
+    else
+        hipLaunchKernelGGL(relayout_slabs<false>, grid, block, 0, s, X, workspace, n, d, ns, ldx);
+    return CBM_OK;
 }
 
 template <bool PACKED>
@@ -620,19 +675,20 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
     if (int rc = check_matrix(n, d, ldz)) return rc;
     if (sched && !aligned(sched, 16)) return CBM_ERR_SHAPE;
     if (X == Z) return CBM_ERR_SHAPE;                    // rows of X are gathered while rows of Z are written
+    const bool ready = (flags & CBM_SPMM_WORKSPACE_READY) != 0;
+    const bool have_ws = workspace && aligned(workspace, 16) && workspace != Z && workspace != X;
+    if (ready && !have_ws) return CBM_ERR_NULL;
     if (n == 0 || d == 0) return CBM_OK;
     const int4* sc = reinterpret_cast<const int4*>(sched);
-    const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z);
-    if (!lpe && (flags & CBM_SPMM_WORKSPACE_READY)) return CBM_ERR_SHAPE;
-    if (lpe) {
-        const int n_slabs = d / (lpe * 4);
+    const SlabPlan plan = plan_slabs(d, ldx, ldz, X, Z, have_ws, ready);
+    if (plan.lpe) {
+        const int lpe = plan.lpe, n_slabs = plan.n_slabs;
         const float* Xg = X;                              // what the gather reads
         int64_t x_slab_stride = lpe * 4, x_row_stride = ldx;
-        if (workspace && lpe == kRelayoutLanes && aligned(workspace, 16) && workspace != Z && workspace != X) {
-            if (!(flags & CBM_SPMM_WORKSPACE_READY)) launch_relayout(X, workspace, n, d, lpe, ldx, s);
+        if (plan.relayout) {
+            if (!ready)
+                if (int rc = launch_relayout(X, workspace, n, d, ldx, s)) return rc;
             Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
-        } else if (flags & CBM_SPMM_WORKSPACE_READY) {
-            return CBM_ERR_SHAPE;                         // told to read a copy that this shape never makes
         }
         static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>);
         static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>);
@@ -643,14 +699,16 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
             const int need = (n + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
             if (G > need) G = need;
             const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
+            const int vec_out = plan.vec_out ? 1 : 0;
             if (lpe == 8)
                 hipLaunchKernelGGL((spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   Xg, Z, n, n_slabs, x_slab_stride, x_row_stride, ldz);
+                                   Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz);
             else
                 hipLaunchKernelGGL((spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   Xg, Z, n, n_slabs, x_slab_stride, x_row_stride, ldz);
+                                   Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz);
             return check_launch();
         }
+        if (ready) return CBM_ERR_LAUNCH;                 // no occupancy information: cannot honour the copy
     }
     const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
     const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
@@ -762,10 +820,15 @@ int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, con
 int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, void* stream) {
     if (!X || !workspace) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
-    if (pick_slab_lanes(d, ldx, d, X, workspace) != kRelayoutLanes || X == workspace) return CBM_ERR_SHAPE;
-    if (n == 0) return CBM_OK;
-    launch_relayout(X, workspace, n, d, kRelayoutLanes, ldx, static_cast<hipStream_t>(stream));
+    if (!aligned(workspace, 16) || X == workspace) return CBM_ERR_SHAPE;
+    if (n == 0 || d == 0) return CBM_OK;
+    if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream))) return rc;
     return check_launch();
+}
+
+int64_t cbm_relayout_floats(int32_t n, int32_t d) {
+    if (n <= 0 || d <= 0) return 0;
+    return (int64_t)n * padded_slab_count(d) * 32;
 }
 
 int cbm_set_spmm_kernel(int kind) {
@@ -774,14 +837,15 @@ int cbm_set_spmm_kernel(int kind) {
     return CBM_OK;
 }
 
-int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
-    const int lpe = pick_slab_lanes(d, ldx, ldz, X, Z);
-    return lpe ? kWave / lpe : 1;
+int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z, int32_t have_workspace) {
+    const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, have_workspace != 0, false);
+    return p.lpe ? kWave / p.lpe : 1;
 }
 
 int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
     if (n <= 0 || d <= 0) return 0;
-    return pick_slab_lanes(d, ldx, ldz, X, Z) == kRelayoutLanes ? (int64_t)n * d : 0;
+    const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, true, false);
+    return p.relayout ? (int64_t)n * p.n_slabs * 32 : 0;
 }
 
 int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_t nnz, void* stream) {

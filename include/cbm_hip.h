@@ -117,10 +117,14 @@ int cbm_set_spmm_kernel(int kind);
  * entries of a row are accumulated strictly in order; g > 1 = entry k goes to partial sum
  * k mod g and the g sums are added as a balanced tree).  Lets a checker reproduce the fp32
  * summation order bit for bit.  No reference counterpart (MKL does not document its order). */
-int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
+int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev,
+                              int32_t have_workspace);
 
-/* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 can use for this
- * shape (n * d when the slab-major copy of X applies, else 0).  The workspace stays optional. */
+/* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 use for this shape when
+ * given one: the size of the slab-major copy of X (n rows x 128-byte slabs, the slab count
+ * rounded up for odd widths), or 0 where the copy is not made (256-byte slabs: d a multiple of 64
+ * and >= 512, float4-addressable rows).  The workspace stays optional: without it, widths that
+ * are a multiple of 32 gather from the row-major X and all others take one wavefront per row. */
 int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
 
 /* coef[k] = +-m[column of entry k] for the packed entries idx[0 .. nnz): the delta VALUES of the
@@ -135,10 +139,13 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * cbm_extensions.cpp:910-940, folded into the producer).  row_sched, if not NULL, is the row
  * schedule written by cbm_schedule_rows (4 int32 per row, 16-byte aligned): rows are then
  * processed in that order, rowptr is not read (may be NULL) and the left scale comes from it.
- * workspace, if not NULL, is caller-owned device memory for n * d floats (16-byte aligned, disjoint
- * from X and Z): widths the slab kernel takes are first copied there slab-major, so that the
- * gathered 128-byte lines of a slab are consecutive in memory instead of a row apart; the result
- * is bit-identical, the copy pays off when rows have more than a few entries.
+ * workspace, if not NULL, is caller-owned device memory of cbm_spmm_workspace_floats() floats
+ * (16-byte aligned, disjoint from X and Z): X is first copied there slab-major (zero-padded to
+ * whole 128-byte slabs), so that the gathered lines of a slab are consecutive in memory instead of
+ * a row apart and odd widths (d = 41, 602, unaligned rows) run on the slab kernel too.  For widths
+ * that are a multiple of 32 the result is bit-identical with and without it; for other widths the
+ * fp32 summation order differs (see cbm_spmm_summation_groups).  The copy pays off when rows
+ * have more than a few entries.
  * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
 int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
@@ -148,9 +155,10 @@ int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float
 
 /* The slab-major copy of X that cbm_spmm_f32 / csr_spmm_f32 make into their workspace, as a call
  * of its own: several multiplies by different matrices with the SAME X can then share one copy
- * (pass the workspace with CBM_SPMM_WORKSPACE_READY).  CBM_ERR_SHAPE if
- * cbm_spmm_workspace_floats is 0 for this shape. */
+ * (pass the workspace with CBM_SPMM_WORKSPACE_READY; the multiply then reads only the copy).
+ * Any width; workspace holds cbm_relayout_floats(n, d) floats. */
 int cbm_relayout_slabs_f32(const float* X_dev, float* workspace_dev, int32_t n, int32_t d, int64_t ldx, void* stream);
+int64_t cbm_relayout_floats(int32_t n, int32_t d);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
  *   m == NULL : Y[v,:] += Y[parent[v],:]

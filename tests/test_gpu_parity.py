@@ -31,11 +31,18 @@ def _need_gpu():
     _lib.hip_lib()
 
 
-def groups_for(d, ld=None):
-    """Partial sums per output element the SpMM keeps for contiguous, 16-byte aligned [*, d]
-    matrices (1 = strictly in order); the oracle reproduces that order bit for bit."""
+def groups_for(d, ld=None, workspace=False):
+    """Partial sums per output element the SpMM keeps for 16-byte aligned [*, d] matrices of row
+    stride ld (1 = strictly in order), with or without a workspace for the slab-major copy of X;
+    the oracle reproduces that order bit for bit."""
     ld = d if ld is None else ld
-    return int(_lib.hip_lib().cbm_spmm_summation_groups(d, ld, ld, C.c_void_p(256), C.c_void_p(256)))
+    return int(_lib.hip_lib().cbm_spmm_summation_groups(d, ld, ld, C.c_void_p(256), C.c_void_p(256), int(workspace)))
+
+
+def mat_groups(mat, d, ld=None):
+    """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough."""
+    n = mat.num_rows
+    return groups_for(d, ld, workspace=mat.relayout and mat.nnz >= 24 * n)
 
 
 def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None):
@@ -45,7 +52,7 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None):
     val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
     return orc.spmm_update(mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32),
                            mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads,
-                           groups=groups_for(x.shape[1]) if groups is None else groups)
+                           groups=mat_groups(mat, x.shape[1]) if groups is None else groups)
 
 
 @pytest.fixture(params=["auto", "wave-per-row"])
@@ -86,11 +93,14 @@ def test_golden_integer_products_bit_exact(golden, case, alpha):
 def test_widths_against_oracle(orc, d, normalized, spmm_kernel):
     n = 700
     ei = graphs.add_self_loops(graphs.sbm(n, 10, 0.3, 0.01, seed=d), n)
-    say("widths", d, normalized, spmm_kernel, "groups", groups_for(d))
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=normalized)
+    say("widths", d, normalized, spmm_kernel, "groups", mat_groups(mat, d))
     assert mat.n_levels >= 2 and (mat.idx < 0).any()
-    if spmm_kernel == "auto" and d in (64, 128, 256, 512):
-        assert groups_for(d) > 1                           # these widths really take the slab kernel
+    if spmm_kernel == "auto":
+        assert mat_groups(mat, d) > 1                      # every width takes the slab kernel (rows are long enough)
+        assert groups_for(d) == (1 if d % 32 else groups_for(d, workspace=True))   # without a workspace only multiples of 32
+    else:
+        assert mat_groups(mat, d) == 1
     x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
     got = gpu_product(mat, x, normalized)
     want = oracle_product(orc, mat, ei, n, x, normalized)
@@ -102,6 +112,10 @@ def test_widths_against_oracle(orc, d, normalized, spmm_kernel):
         mat2 = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
         mat2.stream_coefficients = False
         assert np.array_equal(gpu_product(mat2, x, True), got)
+    mat.relayout = False                                   # no workspace: row-major gather / one wave per row
+    got2 = gpu_product(mat, x, normalized)
+    assert np.array_equal(got2, oracle_product(orc, mat, ei, n, x, normalized))
+    assert orc.max_rel_err(got2, got) <= 1e-5
 
 
 @pytest.mark.parametrize("name,scale,alphas", [("c1", 1.0, (0,)), ("c2", 0.5, (0, 8)), ("c3", 0.05, (0, 16))])
@@ -130,7 +144,7 @@ def test_workloads_against_oracle(orc, name, scale, alphas, spmm_kernel):
         csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(ei[1][order].astype(np.int32)).cuda(),
                  None if vals is None else torch.from_numpy(vals).cuda(), torch.from_numpy(x).cuda(), yd)
         assert orc.max_rel_err(yd.cpu().numpy(), csr) <= 1e-5
-        g = groups_for(x.shape[1])
+        g = groups_for(x.shape[1], workspace=ei.shape[1] >= 24 * w.n)
         assert np.array_equal(yd.cpu().numpy(), csr if g == 1 else orc.csr_spmm(rp, ei[1][order], vals, x, threads=4, groups=g))
 
 
@@ -165,7 +179,7 @@ def test_update_only_entry_points(orc):
         col, sign = mat.columns()
         m = orc.col_multiplier(ei, n) if normalized else None
         val = (sign.numpy() * (m[col.numpy()] if normalized else 1)).astype(np.float32)
-        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=groups_for(d))
+        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=mat_groups(mat, d))
         assert np.array_equal(z.cpu().numpy(), z_ref)
         # update alone on that Z == the oracle's walk (plain or fused) on the same Z
         y = z.clone()
@@ -243,7 +257,7 @@ def test_strided_rows_and_cpu_staging(orc):
     say("strided, slab kernel")                                 # d = 64 with ld = 68 / 72: float4-addressable
     d2 = 64
     x2 = np.random.default_rng(3).standard_normal((n, d2)).astype(np.float32)
-    want2 = oracle_product(orc, mat, ei, n, x2, False, groups=groups_for(d2, 68))
+    want2 = oracle_product(orc, mat, ei, n, x2, False, groups=mat_groups(mat, d2, 68))
     xbig = torch.zeros((n, 68), device="cuda"); xbig[:, :d2] = torch.from_numpy(x2).cuda()
     ybig = torch.full((n, 72), 7.0, device="cuda")
     mat.omp_mkl_csr_spmm_update(xbig[:, :d2], ybig[:, :d2])
@@ -284,6 +298,7 @@ def test_shim_functions_match_cbm_matrix(orc):
     say("shim")
     for normalized in (False, True):
         c = cbm_matrix(ei, None, alpha=2, normalized=normalized)
+        c.relayout = False                                 # the shim brings no workspace: same summation order
         want = gpu_product(c, x.numpy(), normalized)
         mul = c.col_multiplier
         data = (cbm_.from_coo_int32_t_v2_(ei[0], ei[1], torch.ones(ei.size(1)), mul, n, n, 2) if normalized
@@ -320,7 +335,7 @@ def test_c_abi_status_codes_on_device_calls():
     assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1   # coef without m
     assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(x), None, 0, n, d, d, d, None) == 3   # in place
     assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 0   # empty rows -> zeros
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 1, n, d, d, d, None) == 3   # d = 4 never has a slab-major copy
+    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 1, n, d, d, d, None) == 1   # WORKSPACE_READY without a workspace
     lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
     par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
@@ -423,4 +438,9 @@ def test_shared_slab_major_copy(orc):
         got = torch.empty_like(x); mat._run_spmm(torch.zeros_like(x), got, use_m=True, scale_roots=True,
                                                  workspace=ws, workspace_ready=True)     # X itself is not read
         assert torch.equal(got, want)
-    assert relayout_slabs(torch.zeros((n, 41), device="cuda")) is None
+    # odd width: the copy is zero-padded to whole slabs (41 -> 2 slabs of 32)
+    x41 = torch.randn((n, 41), generator=torch.Generator().manual_seed(5)).cuda()
+    w41 = relayout_slabs(x41)
+    assert w41.numel() == n * 64
+    back = w41.view(2, n, 32).permute(1, 0, 2).reshape(n, 64)
+    assert torch.equal(back[:, :41], x41) and float(back[:, 41:].abs().max()) == 0.0
