@@ -88,6 +88,11 @@ public:
                 const int32_t e = h;
                 const int32_t w = node_[e].key;
                 heap_[u] = meld(node_[e].lc, node_[e].rc);            // pop
+                // An edge inside the (contracted) component is dropped outright.  Charging its
+                // reduced weight and discounting the rest of the heap by it, as for any other
+                // popped edge, would cancel out with the next pop of this heap, and the one-edge
+                // "cycle" it would record expands to nothing.
+                if (find(edges_[e].u) == u) continue;
                 if (heap_[u] >= 0) node_[heap_[u]].lazy -= w;        // remaining keys become reduced costs
                 Q[qi] = e; path[qi++] = u; seen[u] = s;
                 res += w;
