@@ -46,15 +46,16 @@ HIP_SYMBOLS = {
     "cbm_version": (C.c_char_p, []),
     "cbm_status_string": (C.c_char_p, [C.c_int]),
     "cbm_set_spmm_kernel": (C.c_int, [C.c_int]),
+    "cbm_set_spmm_occupancy": (C.c_int, [C.c_int]),
     "cbm_spmm_summation_groups": (C.c_int, [_I32, _I64, _I64, _P, _P, _I32]),
     "cbm_relayout_floats": (C.c_int64, [_I32, _I32]),
     "cbm_spmm_workspace_floats": (C.c_int64, [_I32, _I32, _I64, _I64, _P, _P]),
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),
-    "cbm_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_relayout_slabs_f32": (C.c_int, [_P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
-    "cbm_spmm_update_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
-    "csr_spmm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "csr_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
 }
 
 _host = None

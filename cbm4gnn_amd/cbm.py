@@ -379,7 +379,7 @@ class cbm_matrix:
         ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
-                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
+                _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None,
                 _ptr(st["parent"]) if scale_roots else None,
                 _ptr(st["sched_scaled"] if (scale_roots and use_m) else st["sched"]), _ptr(xd), _ptr(yd),
@@ -427,7 +427,7 @@ class cbm_matrix:
         ws = _workspace(xd, yd, self.nnz) if self.relayout else None
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
-                _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None,
+                _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
                 _ptr(st["coef"]) if use_m else None, _ptr(st["parent"]),
                 _ptr(st["sched_scaled"] if use_m else st["sched"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
                 _ptr(xd), _ptr(yd), _ptr(ws), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
@@ -563,6 +563,6 @@ def csr_spmm(rowptr, col, val, x, y, sched=None):
         raise ValueError("csr_spmm expects device tensors")
     ws = _workspace(x, y, col.numel())
     with torch.cuda.device(x.device):
-        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), _ptr(val), _ptr(sched), _ptr(x), _ptr(y), _ptr(ws),
+        rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), col.numel(), _ptr(val), _ptr(sched), _ptr(x), _ptr(y), _ptr(ws),
                                          0, n, x.size(1), _ld(x), _ld(y), _stream(x.device))
     _lib.check(rc, "csr_spmm_f32")

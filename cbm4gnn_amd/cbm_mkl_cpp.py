@@ -105,7 +105,7 @@ def _csr_spmm(row_b, row_e, col, val, rhs, dst_dev, dev):
     # be handed out again by the caching allocator and overwritten by the next upload
     x = rhs.to(dev)
     rowptr_d, col_d, val_d = rowptr.to(dev), col.to(dev).contiguous(), val.to(dev).contiguous()
-    rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr_d), _ptr(col_d), _ptr(val_d), None, _ptr(x), _ptr(dst_dev), None,
+    rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr_d), _ptr(col_d), col_d.numel(), _ptr(val_d), None, _ptr(x), _ptr(dst_dev), None,
                                      0, n, x.size(1), _ld(x), _ld(dst_dev), _stream(dev))
     _lib.check(rc, "csr_spmm_f32")
 

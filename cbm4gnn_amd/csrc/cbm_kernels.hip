@@ -192,13 +192,10 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
             }
         }
     }
-    if constexpr (PACKED) {
-        if (m && parent)                           // child of the root: left scaling, final value
 #pragma unroll
-            for (int c = 0; c < CH; c++)
+    for (int c = 0; c < CH; c++)                   // 1.0f unless a child of the root (left scaling)
 #pragma unroll
-                for (int v = 0; v < VEC; v++) acc[c][v] *= root_scale;
-    }
+        for (int v = 0; v < VEC; v++) acc[c][v] *= root_scale;
     float* __restrict__ zr = Z + (int64_t)row * ldz + col0;
 #pragma unroll
     for (int c = 0; c < CH; c++)
@@ -216,9 +213,20 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
 // that many consecutive entries of the same row at once; each group keeps its own partial sum
 // (entries k = g mod (64 / LPE), in order) and the partial sums are added by a xor-shuffle tree
 // at the end of the row.  The price: index (and coefficient) arrays are streamed once per slab.
-// Coefficients: `coef` (streamed, +-m[col] precomputed) if given, else m[col] gathered, else +-1.
+// Where an entry's coefficient comes from is a template parameter, so that the gather rounds hold
+// no branch at all (with run-time tests of `val` and `m` between the loads of a round the plain
+// +-1 variant ran latency-bound: 6.2 ms at 8 wavefronts per SIMD, 9.1 ms at 4, on a matrix the
+// streamed variant multiplies in 5.9 ms):
+//   kCoefStream: val[k] streamed (the CSR values, or +-m[col] precomputed by expand_coef)
+//   kCoefSign:   +-1 from bit 31 of the index (plain CSR columns have it clear: +1)
+//   kCoefSignM:  +-m[col], m gathered per entry
+// Bit 31 is masked off the column in every mode.  PACKED only names the instantiation the packed
+// delta format runs on (kernel traces then tell CBM launches from CSR baseline launches) and
+// enables the left scale read from m when no row schedule is given.
 // ---------------------------------------------------------------------------------------------
-template <int LPE, bool PACKED, int U>
+constexpr int kCoefStream = 0, kCoefSign = 1, kCoefSignM = 2;
+
+template <int LPE, bool PACKED, int COEF, int U>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
@@ -294,19 +302,17 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
                     const int k = pos + u * kStep + sub;
                     const int kc = min(k, end - 1);
                     p[u] = idx[kc];
-                    if (val) f[u] = val[kc];
-                    else f[u] = 1.0f;
-                    if (k >= end) f[u] = 0.0f;
+                    if constexpr (COEF == kCoefStream) {
+                        f[u] = val[kc];
+                        if (k >= end) f[u] = 0.0f;
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < UU; u++) {
-                    const uint32_t c = PACKED ? (p[u] & 0x7fffffffu) : p[u];
-                    if constexpr (PACKED) {
-                        if (!val) {                        // no streamed coefficients: sign bit, optional m gather
-                            const uint32_t mag = m ? __float_as_uint(m[c]) : 0x3f800000u;
-                            const float g = __uint_as_float(mag ^ (p[u] & 0x80000000u));
-                            f[u] = f[u] == 0.0f ? 0.0f : g;
-                        }
+                    const uint32_t c = p[u] & 0x7fffffffu;
+                    if constexpr (COEF != kCoefStream) {
+                        const uint32_t mag = COEF == kCoefSignM ? __float_as_uint(m[c]) : 0x3f800000u;
+                        f[u] = pos + u * kStep + sub < end ? __uint_as_float(mag ^ (p[u] & 0x80000000u)) : 0.0f;
                     }
                     load_vec<4>(Xs + (int64_t)c * x_row_stride, x[u]);
                 }
@@ -328,11 +334,8 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
             if (sub == 0) {
-                if constexpr (PACKED) {
-                    if (m && parent)
 #pragma unroll
-                        for (int e = 0; e < 4; e++) acc[e] *= row_scale;
-                }
+                for (int e = 0; e < 4; e++) acc[e] *= row_scale;      // 1.0f unless a child of the root
                 const int col = slab * kSlab + li * 4;
                 float* __restrict__ zr = Zs + (int64_t)row * ldz;
                 if (vec_out) {
@@ -589,29 +592,30 @@ inline int padded_slab_count(int d) {
     return ns;
 }
 
-// Widths that split into whole 128- or 256-byte slabs whose count divides, or is a multiple of,
-// the 8 XCDs run on the slab kernel directly (a wider slab is taken only when it still leaves
-// one slab per XCD; the slab-major copy pays off for 128-byte slabs only: with 256-byte slabs it
-// measured within +-3 %).  Any other width or alignment runs on the slab kernel through the
-// zero-padded slab-major copy when the caller brought a workspace, else one wave per row.
-// force_copy: the caller already made the copy (always 128-byte slabs, padded count).
+// With a workspace every width runs on 128-byte slabs read from the slab-major copy (zero-padded
+// for widths that are not a multiple of 32).  Without one, widths that split into whole 128- or
+// 256-byte slabs whose count divides, or is a multiple of, the 8 XCDs gather from the row-major X
+// (a 256-byte slab is taken when that still leaves one slab per XCD: d = 512, 1024, ...), and any
+// other width or alignment takes one wavefront per row.  Measured at d = 512 / 1024 on an MI355X:
+// 128-byte slabs from the copy beat 256-byte slabs from the row-major X by 5-18 % (copy included)
+// on graphs with N >= 100 000 and tie on a 12 000-row graph.
+// force_copy: the caller already made the copy.
 inline SlabPlan plan_slabs(int d, int64_t ldx, int64_t ldz, const void* X, const void* Z, bool have_workspace,
                            bool force_copy) {
     SlabPlan p;
     if (g_spmm_kernel == 1 && !force_copy) return p;
     const bool x_vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16);
     p.vec_out = d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16);
-    if (!force_copy && d % 32 == 0 && x_vec && p.vec_out) {
+    if (have_workspace || force_copy) {
+        p.lpe = 8; p.n_slabs = padded_slab_count(d); p.relayout = true;
+        return p;
+    }
+    if (d % 32 == 0 && x_vec && p.vec_out) {
         int lpe = 8;
         if (d % 64 == 0 && d / 64 >= kXcds) lpe = 16;
         const int ns = d / (lpe * 4);
-        if (ns % kXcds == 0 || kXcds % ns == 0) {
-            p.lpe = lpe; p.n_slabs = ns; p.relayout = have_workspace && lpe == 8;
-            return p;
-        }
+        if (ns % kXcds == 0 || kXcds % ns == 0) { p.lpe = lpe; p.n_slabs = ns; }
     }
-    if (!have_workspace && !force_copy) return p;
-    p.lpe = 8; p.n_slabs = padded_slab_count(d); p.relayout = true;
     return p;
 }
 
@@ -642,7 +646,22 @@ inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
     return CBM_OK;
 }
 
-// Workgroups per XCD of the persistent slab kernel: as many as are resident at once.
+// Wavefronts per SIMD the persistent slab kernel is launched with (a workgroup is one wavefront on
+// each of a CU's 4 SIMDs).  Every wavefront keeps 8 KB of gathered lines in flight while it is inside
+// a long row; at the 6-7 wavefronts the registers allow, a 32-CU XCD has more lines in flight than
+// its 4 MB L2 holds.  Short rows spend more of their time outside the gather rounds and need the
+// extra wavefronts.  Measured on an MI355X with 128-byte slabs: rows averaging 190-490 entries are
+// fastest at 3-4 (3-8 % over 6-8), rows averaging 45 entries at 5-6 (4 costs 7 %, 3 costs 20 %);
+// 256-byte slabs are fastest at 3-4 on every graph tried.
+int g_spmm_occupancy = 0;                                  // 0 = automatic
+inline int slab_waves_per_simd(int64_t nnz, int32_t n, int lpe) {
+    if (g_spmm_occupancy > 0) return g_spmm_occupancy;
+    if (lpe == 16) return 4;
+    return nnz >= (int64_t)128 * n ? 4 : 6;
+}
+
+// Workgroups per XCD of the persistent slab kernel that are resident at once, and workgroups per
+// XCD that give one wavefront per SIMD.
 template <class K>
 int resident_groups_per_xcd(K kernel) {
     int dev = 0, cus = 0, per_cu = 0;
@@ -651,6 +670,26 @@ int resident_groups_per_xcd(K kernel) {
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kWave * kWavesPerBlock, 0) != hipSuccess) return 0;
     if (cus < kXcds || per_cu < 1) return 0;
     return (cus / kXcds) * per_cu;
+}
+
+// Resident workgroups per XCD of each slab kernel instantiation, queried once.
+template <bool PACKED>
+int slab_kernel_groups(int lpe, int coef_mode) {
+    static const int g[2][3] = {
+        {resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefStream, CBM_SLAB_ROUNDS>),
+         resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSign, CBM_SLAB_ROUNDS>),
+         resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>)},
+        {resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefStream, CBM_SLAB_ROUNDS>),
+         resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSign, CBM_SLAB_ROUNDS>),
+         resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>)}};
+    return g[lpe == 8 ? 0 : 1][coef_mode];
+}
+
+inline int groups_per_xcd_per_wave() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return cus / kXcds;
 }
 
 inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s) {
@@ -666,7 +705,7 @@ inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t 
 }
 
 template <bool PACKED>
-int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, const float* m,
+int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* val, const float* m,
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
     if (flags & ~CBM_SPMM_WORKSPACE_READY) return CBM_ERR_UNSUPPORTED;
@@ -690,22 +729,30 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, const float* val, co
                 if (int rc = launch_relayout(X, workspace, n, d, ldx, s)) return rc;
             Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
         }
-        static const int g8 = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>);
-        static const int g16 = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>);
-        int G = lpe == 8 ? g8 : g16;
+        const int coef_mode = val ? kCoefStream : (m ? kCoefSignM : kCoefSign);
+        static const int per_wave = groups_per_xcd_per_wave();
+        int G = slab_kernel_groups<PACKED>(lpe, coef_mode);
         if (G > 0) {
+            const int cap = per_wave * slab_waves_per_simd(nnz, n, lpe);
+            if (cap > 0 && G > cap) G = cap;
             // no more waves than rows: with fewer rows than resident waves shrink the grid
             const int share = n_slabs >= kXcds ? 1 : kXcds / n_slabs;
             const int need = (n + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
             if (G > need) G = need;
             const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
             const int vec_out = plan.vec_out ? 1 : 0;
-            if (lpe == 8)
-                hipLaunchKernelGGL((spmm_slab_per_xcd<8, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz);
-            else
-                hipLaunchKernelGGL((spmm_slab_per_xcd<16, PACKED, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, val, m, parent,
-                                   Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz);
+#define LAUNCH_SLAB(L, CF)                                                                                     \
+    hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, CF, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, \
+                       val, m, parent, Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz)
+            switch (lpe * 4 + coef_mode) {
+                case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream); break;
+                case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign); break;
+                case 8 * 4 + kCoefSignM: LAUNCH_SLAB(8, kCoefSignM); break;
+                case 16 * 4 + kCoefStream: LAUNCH_SLAB(16, kCoefStream); break;
+                case 16 * 4 + kCoefSign: LAUNCH_SLAB(16, kCoefSign); break;
+                default: LAUNCH_SLAB(16, kCoefSignM); break;
+            }
+#undef LAUNCH_SLAB
             return check_launch();
         }
         if (ready) return CBM_ERR_LAUNCH;                 // no occupancy information: cannot honour the copy
@@ -808,12 +855,12 @@ const char* cbm_status_string(int status) {
     }
 }
 
-int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
+int cbm_spmm_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m, const float* coef,
                  const int32_t* parent, const int32_t* row_sched, const float* X, float* Z, float* workspace,
                  int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
     if (!idx && n > 0) return CBM_ERR_NULL;
     if (coef && !m) return CBM_ERR_NULL;                 // coef is the expansion of m, not a substitute
-    return launch_spmm<true>(rowptr, idx, coef, m, parent, row_sched, X, Z, workspace, flags, n, d, ldx, ldz,
+    return launch_spmm<true>(rowptr, idx, nnz, coef, m, parent, row_sched, X, Z, workspace, flags, n, d, ldx, ldz,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -829,6 +876,12 @@ int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t 
 int64_t cbm_relayout_floats(int32_t n, int32_t d) {
     if (n <= 0 || d <= 0) return 0;
     return (int64_t)n * padded_slab_count(d) * 32;
+}
+
+int cbm_set_spmm_occupancy(int waves_per_simd) {
+    if (waves_per_simd < 0 || waves_per_simd > 8) return CBM_ERR_SHAPE;
+    g_spmm_occupancy = waves_per_simd;
+    return CBM_OK;
 }
 
 int cbm_set_spmm_kernel(int kind) {
@@ -859,11 +912,11 @@ int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_
     return check_launch();
 }
 
-int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, const float* val, const int32_t* row_sched,
+int csr_spmm_f32(const int32_t* rowptr, const int32_t* col, int64_t nnz, const float* val, const int32_t* row_sched,
                  const float* X, float* Y, float* workspace, int32_t flags, int32_t n, int32_t d, int64_t ldx,
                  int64_t ldy, void* stream) {
     if (!col && n > 0) return CBM_ERR_NULL;
-    return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), val, nullptr, nullptr, row_sched,
+    return launch_spmm<false>(rowptr, reinterpret_cast<const uint32_t*>(col), nnz, val, nullptr, nullptr, row_sched,
                               X, Y, workspace, flags, n, d, ldx, ldy, static_cast<hipStream_t>(stream));
 }
 
@@ -880,13 +933,13 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
              : launch_propagate<false>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s);
 }
 
-int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, const float* m, const float* coef,
+int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m, const float* coef,
                         const int32_t* parent, const int32_t* row_sched, const int32_t* order, const int32_t* level_off_dev,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, float* workspace,
                         int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, m, coef, parent, row_sched, X, Y, workspace, 0, n, d, ldx, ldy, stream);
+    int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, Y, workspace, 0, n, d, ldx, ldy, stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,

@@ -113,6 +113,11 @@ const char* cbm_status_string(int status);
  * counterpart. */
 int cbm_set_spmm_kernel(int kind);
 
+/* Resident wavefronts per SIMD of the slab SpMM kernel for later calls of this process: 0 =
+ * automatic (default: 4 when rows average 256 entries or more, else 6), 1..8 = fixed.  A tuning
+ * hook; no reference counterpart. */
+int cbm_set_spmm_occupancy(int waves_per_simd);
+
 /* How many interleaved partial sums the SpMM keeps per output element for this shape (1 = the
  * entries of a row are accumulated strictly in order; g > 1 = entry k goes to partial sum
  * k mod g and the g sums are added as a balanced tree).  Lets a checker reproduce the fp32
@@ -122,9 +127,8 @@ int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X
 
 /* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 use for this shape when
  * given one: the size of the slab-major copy of X (n rows x 128-byte slabs, the slab count
- * rounded up for odd widths), or 0 where the copy is not made (256-byte slabs: d a multiple of 64
- * and >= 512, float4-addressable rows).  The workspace stays optional: without it, widths that
- * are a multiple of 32 gather from the row-major X and all others take one wavefront per row. */
+ * rounded up for odd widths).  The workspace stays optional: without it, widths that are a
+ * multiple of 32 gather from the row-major X and all others take one wavefront per row. */
 int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
 
 /* coef[k] = +-m[column of entry k] for the packed entries idx[0 .. nnz): the delta VALUES of the
@@ -142,14 +146,15 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * workspace, if not NULL, is caller-owned device memory of cbm_spmm_workspace_floats() floats
  * (16-byte aligned, disjoint from X and Z): X is first copied there slab-major (zero-padded to
  * whole 128-byte slabs), so that the gathered lines of a slab are consecutive in memory instead of
- * a row apart and odd widths (d = 41, 602, unaligned rows) run on the slab kernel too.  For widths
- * that are a multiple of 32 the result is bit-identical with and without it; for other widths the
- * fp32 summation order differs (see cbm_spmm_summation_groups).  The copy pays off when rows
- * have more than a few entries.
+ * a row apart and odd widths (d = 41, 602, unaligned rows) run on the slab kernel too.  The fp32
+ * summation order with and without it can differ (cbm_spmm_summation_groups reports both).  The
+ * copy pays off when rows have more than a few entries.
+ * nnz is the number of entries (rowptr[n]); it only sizes the launch (long rows run with fewer
+ * resident wavefronts, see cbm_set_spmm_occupancy) and may be 0 if unknown.
  * Replaces the mkl_sparse_s_create_csr + mkl_sparse_s_mm pair of every *_spmm_update function
  * (cbm_extensions.cpp:678-704, :875-900, :1133-1159, :1251-1277); overwrites Z (beta = 0). */
-int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
-                 const int32_t* parent_dev, const int32_t* row_sched_dev, const float* X_dev, float* Z_dev,
+int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz, const float* m_dev,
+                 const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev, const float* X_dev, float* Z_dev,
                  float* workspace_dev, int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz,
                  void* stream);
 
@@ -179,7 +184,7 @@ int cbm_propagate_f32(const int32_t* parent_dev, const int32_t* order_dev, const
 /* Y = A_hat * X in one call: cbm_spmm_f32 followed by cbm_propagate_f32 on the same stream.
  * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);
  * m != NULL replaces seq_/omp_s_fused_spmm_update_csr_int32_ (:845-996, :1224-1374). */
-int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev,
+int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz, const float* m_dev,
                         const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
                         const int32_t* order_dev,
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
@@ -188,7 +193,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, cons
 
 /* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
-int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, const float* val_dev,
+int csr_spmm_f32(const int32_t* rowptr_dev, const int32_t* col_dev, int64_t nnz, const float* val_dev,
                  const int32_t* row_sched_dev, const float* X_dev, float* Y_dev, float* workspace_dev,
                  int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldy, void* stream);
 

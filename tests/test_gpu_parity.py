@@ -98,7 +98,9 @@ def test_widths_against_oracle(orc, d, normalized, spmm_kernel):
     assert mat.n_levels >= 2 and (mat.idx < 0).any()
     if spmm_kernel == "auto":
         assert mat_groups(mat, d) > 1                      # every width takes the slab kernel (rows are long enough)
-        assert groups_for(d) == (1 if d % 32 else groups_for(d, workspace=True))   # without a workspace only multiples of 32
+        assert groups_for(d, workspace=True) == 8           # 128-byte slabs from the slab-major copy
+        # without a workspace only multiples of 32 run on slabs; 256-byte slabs (4 groups) where 8 of them fit
+        assert groups_for(d) == (1 if d % 32 else (4 if d % 64 == 0 and d >= 512 else 8))
     else:
         assert mat_groups(mat, d) == 1
     x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
@@ -330,18 +332,18 @@ def test_c_abi_status_codes_on_device_calls():
     rp = torch.zeros(n + 1, dtype=torch.int32, device="cuda"); idx = torch.zeros(1, dtype=torch.int32, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
     say("status codes")
-    assert lib.cbm_spmm_f32(None, p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d - 1, d, None) == 3
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, p(x), None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1   # coef without m
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(x), None, 0, n, d, d, d, None) == 3   # in place
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 0   # empty rows -> zeros
-    assert lib.cbm_spmm_f32(p(rp), p(idx), None, None, None, None, p(x), p(y), None, 1, n, d, d, d, None) == 1   # WORKSPACE_READY without a workspace
+    assert lib.cbm_spmm_f32(None, p(idx), 0, None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1
+    assert lib.cbm_spmm_f32(p(rp), p(idx), 0, None, None, None, None, p(x), p(y), None, 0, n, d, d - 1, d, None) == 3
+    assert lib.cbm_spmm_f32(p(rp), p(idx), 0, None, p(x), None, None, p(x), p(y), None, 0, n, d, d, d, None) == 1   # coef without m
+    assert lib.cbm_spmm_f32(p(rp), p(idx), 0, None, None, None, None, p(x), p(x), None, 0, n, d, d, d, None) == 3   # in place
+    assert lib.cbm_spmm_f32(p(rp), p(idx), 0, None, None, None, None, p(x), p(y), None, 0, n, d, d, d, None) == 0   # empty rows -> zeros
+    assert lib.cbm_spmm_f32(p(rp), p(idx), 0, None, None, None, None, p(x), p(y), None, 1, n, d, d, d, None) == 1   # WORKSPACE_READY without a workspace
     lo = (C.c_int32 * 2)(0, n - 1)                      # does not cover n rows
     par = torch.full((n,), -1, dtype=torch.int32, device="cuda"); order = torch.arange(n, dtype=torch.int32, device="cuda")
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 3
     lo = (C.c_int32 * 2)(0, n)
     assert lib.cbm_propagate_f32(p(par), p(order), p(rp), lo, 1, None, p(y), n, d, d, 0, None) == 0
-    assert lib.cbm_spmm_update_f32(p(rp), p(idx), None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), None, n, d, d, d, 0, None) == 3
+    assert lib.cbm_spmm_update_f32(p(rp), p(idx), 0, None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), None, n, d, d, d, 0, None) == 3
     torch.cuda.synchronize()
     assert (y == 0).all()
 
@@ -444,3 +446,27 @@ def test_shared_slab_major_copy(orc):
     assert w41.numel() == n * 64
     back = w41.view(2, n, 32).permute(1, 0, 2).reshape(n, 64)
     assert torch.equal(back[:, :41], x41) and float(back[:, 41:].abs().max()) == 0.0
+
+
+def test_launch_size_does_not_change_results(orc):
+    """The slab kernel is persistent: how many wavefronts it is launched with (automatic from the
+    mean row length, or fixed through cbm_set_spmm_occupancy) changes which wavefront computes a
+    row, never the order in which a row's entries are summed."""
+    lib = _lib.hip_lib()
+    n = 3000
+    ei = graphs.add_self_loops(graphs.sbm(n, 3, 0.3, 0.002, seed=6), n)       # rows average ~300 entries
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=True)
+    assert mat.nnz_a >= 256 * n
+    x = torch.randn((n, 128), generator=torch.Generator().manual_seed(6)).cuda()
+    say("occupancy hook")
+    want = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, want)
+    assert lib.cbm_set_spmm_occupancy(9) == 3 and lib.cbm_set_spmm_occupancy(-1) == 3
+    try:
+        for waves in (1, 3, 8):
+            assert lib.cbm_set_spmm_occupancy(waves) == 0
+            got = torch.full_like(x, float("nan")); mat.omp_mkl_csr_fused_spmm_update(x, got)
+            assert torch.equal(got, want), waves
+    finally:
+        assert lib.cbm_set_spmm_occupancy(0) == 0
+    ref = oracle_product(orc, mat, ei, n, x.cpu().numpy(), True)
+    assert np.array_equal(want.cpu().numpy(), ref)
