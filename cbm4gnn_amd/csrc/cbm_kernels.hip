@@ -289,23 +289,28 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
             float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             // One gather round = UU instructions of kStep entries each.  Every load of a round is
             // unconditional -- entries past the end of the row are clamped to its last entry and
-            // get coefficient 0 -- so the index loads, then the X-row loads, are all in flight
-            // together; a branch or an exec mask around each load would serialise them.  Short
-            // remainders take a shorter round instead of mostly clamped instructions.
+            // get coefficient 0 -- so the X-row loads are all in flight together; a branch or an
+            // exec mask around each load would serialise them.  Short remainders take a shorter
+            // round instead of mostly clamped instructions.
             auto round = [&](auto uu_tag, int pos) {
                 constexpr int UU = decltype(uu_tag)::value;
                 uint32_t p[UU];
                 float f[UU];
                 float x[UU][4];
+                // The round's entries come in with ONE coalesced load (lane l fetches entry pos + l,
+                // clamped) and reach their lane group through the LDS crossbar.  UU per-group loads of
+                // the same few addresses cost the texture addresser about half of what the X loads
+                // cost: 3-15 % of the kernel time on the workloads measured.
+                const int k = pos + lane;
+                const int kc = min(k, end - 1);
+                const uint32_t p_all = idx[kc];
+                float f_all = 0.0f;
+                if constexpr (COEF == kCoefStream) f_all = val[kc];
+                if constexpr (COEF == kCoefStream) f_all = k < end ? f_all : 0.0f;
 #pragma unroll
                 for (int u = 0; u < UU; u++) {
-                    const int k = pos + u * kStep + sub;
-                    const int kc = min(k, end - 1);
-                    p[u] = idx[kc];
-                    if constexpr (COEF == kCoefStream) {
-                        f[u] = val[kc];
-                        if (k >= end) f[u] = 0.0f;
-                    }
+                    p[u] = __shfl(p_all, u * kStep + sub, kWave);
+                    if constexpr (COEF == kCoefStream) f[u] = __shfl(f_all, u * kStep + sub, kWave);
                 }
 #pragma unroll
                 for (int u = 0; u < UU; u++) {
