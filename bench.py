@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # runs of `bench.py --probe` scaled by a plain copy of known size (FETCH_SIZE x 2.00, WRITE_SIZE
 # x 1.00 on this part); keyed by (workload, alpha, d).  Counters cannot be read from inside this
 # process, so a configuration that was not profiled reports null.
-MEASURED_TRAFFIC_BYTES = {("c3", 16, 256): 2.33e9 + 0.1024e9}
+MEASURED_TRAFFIC_BYTES = {("c3", 16, 256): 2.32e9 + 0.1024e9}
 
 
 def algorithmic_bytes(n, nnz, d, norm, tree_edges, levels, n_edges_a):
@@ -368,7 +368,7 @@ def main():
         "kernel_ms": {"relayout_slabs": relayout_ms, "delta_spmm": spmm_ms, "propagate": prop_ms},
         "gpu_csr_ms": csr_ms, "gpu_csr_GBps": b_csr / (csr_ms * 1e-3) / 1e9, "speedup_vs_gpu_csr": csr_ms / span_ms,
         "max_rel_err_vs_gpu_csr": err_vs_csr,
-        "roofline": {"bound": "hbm", "kernel": "spmm_slab_per_xcd" if d % 32 == 0 else "spmm_wave_per_row", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "spmm_slab_per_xcd" if (ws is not None or d % 32 == 0) else "spmm_wave_per_row", "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, alpha, d)) if args.scale == 1.0 else None,
                      "algorithmic_bytes": b_spmm, "avg_launch_ms": spmm_ms},
