@@ -321,8 +321,8 @@ def main():
     # the dominant kernel alone (delta SpMM gather), same launch as inside the step; where the step
     # first copies X slab-major, that copy is made once here and timed on its own
     zd = torch.empty_like(xd)
-    from cbm4gnn_amd.cbm import _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT as min_entries
-    ws = relayout_slabs(xd) if (mat.relayout and nnz >= min_entries * n) else None
+    from cbm4gnn_amd.cbm import _wants_workspace
+    ws = relayout_slabs(xd) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
     relayout_ms = 0.0
     if ws is not None:
         _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd), args.steps, args.warmup, torch)

@@ -1,19 +1,21 @@
 // HIP kernels (gfx950 / CDNA4) and C-ABI launchers of the CBM multiply.
 //
 // Bandwidth-bound gather / stream kernels, 64-wide wavefronts, no MFMA, no atomics:
-//   (1)  spmm_slab_per_xcd    delta SpMM  Z = D * diag(m) * X  for feature widths that split into
-//                             128- or 256-byte slabs: one slab per XCD (so an XCD's L2 only ever
-//                             sees its slab of X), persistent waves walking a longest-first row
-//                             schedule, 8 lanes per delta entry, 64 entries in flight per wave.
-//        spmm_wave_per_row    the same product for any other width or alignment: one wave per
-//                             row, lanes span the feature columns, packed indices broadcast with
-//                             v_readlane so X-row addresses are scalar.
+//   (1)  spmm_slab_per_xcd    delta SpMM  Z = D * diag(m) * X  with the feature dimension cut into
+//                             128-byte slabs (256-byte on the row-major path of wide d): one slab per
+//                             XCD (so an XCD's L2 only ever sees its slab of X), persistent waves
+//                             walking a longest-first row schedule, 8 lanes per delta entry, 64
+//                             entries in flight per wave.  Any width when the caller brings a
+//                             workspace for the slab-major copy of X (relayout_slabs).
+//        spmm_wave_per_row    the same product without a workspace for widths that are not a
+//                             multiple of 32: one wave per row, lanes span the feature columns,
+//                             packed indices broadcast with v_readlane so X-row addresses are scalar.
 //   (2)  propagate_level / propagate_narrow_levels / propagate_chain / scale_level0
 //                             tree propagation  Y[v] (+)= Y[parent(v)]  level-synchronously over a
 //                             host-computed (level, id) ordering: one launch per wide level, one
 //                             single-workgroup launch per run of narrow levels, one
 //                             register-carried launch per chain of single-row levels.
-// The SpMM templates without the sign bit (PACKED = false) are the plain CSR baseline.
+// The SpMM instantiations with PACKED = false are the plain CSR baseline.
 //
 // What each launcher replaces in the reference is stated in include/cbm_hip.h.
 #include <hip/hip_runtime.h>
@@ -155,12 +157,13 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
                 my_cf = val ? val[base + lane] : 1.0f;
             }
         }
-        int k = 0;
-        for (; k + U <= cnt; k += U) {
+        // U X-row loads in flight; in the last, partial group the surplus loads repeat the row of
+        // the last entry with coefficient 0 (a branch around each load would serialise them)
+        for (int k = 0; k < cnt; k += U) {
             float x[U][CH][VEC];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const float* __restrict__ xr = X + (int64_t)bcast_i(my_col, k + u) * ldx + col0;
+                const float* __restrict__ xr = X + (int64_t)bcast_i(my_col, min(k + u, cnt - 1)) * ldx + col0;
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     if (FULL || col0 + c * kWave * VEC < d) load_vec<VEC>(xr + c * kWave * VEC, x[u][c]);
@@ -171,24 +174,11 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const float f = bcast_f(my_cf, k + u);
+                const float f = k + u < cnt ? bcast_f(my_cf, min(k + u, cnt - 1)) : 0.0f;
 #pragma unroll
                 for (int c = 0; c < CH; c++)
 #pragma unroll
                     for (int v = 0; v < VEC; v++) acc[c][v] = fmaf(f, x[u][c][v], acc[c][v]);
-            }
-        }
-        for (; k < cnt; k++) {
-            const float* __restrict__ xr = X + (int64_t)bcast_i(my_col, k) * ldx + col0;
-            const float f = bcast_f(my_cf, k);
-#pragma unroll
-            for (int c = 0; c < CH; c++) {
-                if (FULL || col0 + c * kWave * VEC < d) {
-                    float x[VEC];
-                    load_vec<VEC>(xr + c * kWave * VEC, x);
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[c][v] = fmaf(f, x[v], acc[c][v]);
-                }
             }
         }
     }
@@ -656,13 +646,15 @@ inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
 // a long row; at the 6-7 wavefronts the registers allow, a 32-CU XCD has more lines in flight than
 // its 4 MB L2 holds.  Short rows spend more of their time outside the gather rounds and need the
 // extra wavefronts.  Measured on an MI355X with 128-byte slabs: rows averaging 190-490 entries are
-// fastest at 3-4 (3-8 % over 6-8), rows averaging 45 entries at 5-6 (4 costs 7 %, 3 costs 20 %);
-// 256-byte slabs are fastest at 3-4 on every graph tried.
+// fastest at 3-4 (3-8 % over 6-8), rows averaging 45 entries at 5-6 (4 costs 7 %, 3 costs 20 %),
+// rows averaging 13 entries at the register limit (6 costs 7 %); 256-byte slabs are fastest at
+// 3-4 on every graph tried.
 int g_spmm_occupancy = 0;                                  // 0 = automatic
 inline int slab_waves_per_simd(int64_t nnz, int32_t n, int lpe) {
     if (g_spmm_occupancy > 0) return g_spmm_occupancy;
     if (lpe == 16) return 4;
-    return nnz >= (int64_t)128 * n ? 4 : 6;
+    if (nnz >= (int64_t)128 * n) return 4;
+    return nnz >= (int64_t)32 * n ? 6 : 8;                 // 8: every wavefront the registers allow
 }
 
 // Workgroups per XCD of the persistent slab kernel that are resident at once, and workgroups per

@@ -114,7 +114,8 @@ const char* cbm_status_string(int status);
 int cbm_set_spmm_kernel(int kind);
 
 /* Resident wavefronts per SIMD of the slab SpMM kernel for later calls of this process: 0 =
- * automatic (default: 4 when rows average 256 entries or more, else 6), 1..8 = fixed.  A tuning
+ * automatic (default: 4 when rows average 128 entries or more, 6 from 32, else all the registers
+ * allow), 1..8 = fixed.  A tuning
  * hook; no reference counterpart. */
 int cbm_set_spmm_occupancy(int waves_per_simd);
 

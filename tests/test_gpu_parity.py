@@ -39,10 +39,16 @@ def groups_for(d, ld=None, workspace=False):
     return int(_lib.hip_lib().cbm_spmm_summation_groups(d, ld, ld, C.c_void_p(256), C.c_void_p(256), int(workspace)))
 
 
+def brings_workspace(relayout, nnz, n, d, ld=None):
+    """The Python layer's rule: a workspace when rows average >= 24 entries, or when the width would
+    otherwise run one wavefront per row."""
+    return bool(relayout) and n > 0 and (nnz >= 24 * n or groups_for(d, ld) == 1)
+
+
 def mat_groups(mat, d, ld=None):
     """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough."""
     n = mat.num_rows
-    return groups_for(d, ld, workspace=mat.relayout and mat.nnz >= 24 * n)
+    return groups_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, n, d, ld))
 
 
 def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None):
@@ -146,7 +152,7 @@ def test_workloads_against_oracle(orc, name, scale, alphas, spmm_kernel):
         csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(ei[1][order].astype(np.int32)).cuda(),
                  None if vals is None else torch.from_numpy(vals).cuda(), torch.from_numpy(x).cuda(), yd)
         assert orc.max_rel_err(yd.cpu().numpy(), csr) <= 1e-5
-        g = groups_for(x.shape[1], workspace=ei.shape[1] >= 24 * w.n)
+        g = groups_for(x.shape[1], workspace=brings_workspace(True, ei.shape[1], w.n, x.shape[1]))
         assert np.array_equal(yd.cpu().numpy(), csr if g == 1 else orc.csr_spmm(rp, ei[1][order], vals, x, threads=4, groups=g))
 
 
