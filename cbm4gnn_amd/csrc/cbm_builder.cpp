@@ -18,7 +18,8 @@
 //   * |row_i ^ row_j| is streamed row by row with a sparse accumulator and only admissible pairs
 //     are kept; the reference materialises all of A*A^T with mkl_sparse_syrk (:46-65).
 //   * the arborescence is found by an own implementation of Tarjan's O(m log n) algorithm
-//     (meldable leftist heaps with lazy keys, union-find with rollback for the expansion).
+//     (sorted runs merged through small heaps, lazy reduced costs, union-find with rollback
+//     for the expansion).
 //   * the normalisation vector is NOT folded into delta values here; kernels apply it.
 #include <algorithm>
 #include <cstdint>
@@ -37,43 +38,54 @@ struct CandEdge { int32_t u, v, w; };
 
 // ---------------------------------------------------------------------------------------------
 // Minimum spanning arborescence (Tarjan 1977 / Camerini-Fratta-Maffioli 1979 expansion).
+//
+// The edges entering a (contracted) node are kept as a k-way merge instead of a meldable heap:
+// every original node's incoming edges form one run, sorted once by (weight, edge id); a
+// contracted node owns the runs of its members and a small binary heap over the runs' current
+// heads.  Popping the cheapest entering edge advances one run (sequential memory) and sifts
+// one entry of a heap that fits the L1 cache; contracting a cycle moves the smaller heaps
+// into the largest.  Reduced costs are lazy: an offset per contracted node plus an offset per
+// run that absorbs the difference when the run changes owner.  Ties go to the smaller edge id,
+// so the result does not depend on the order in which heaps were merged.
 // ---------------------------------------------------------------------------------------------
 class Arborescence {
 public:
     Arborescence(int32_t n, const std::vector<CandEdge>& edges, int threads)
-        : n_(n), threads_(threads), edges_(edges), node_(edges.size()), heap_(n, -1), uf_(n, -1) {}
+        : n_(n), threads_(threads), edges_(edges), uf_(n, -1), fast_(n) {}
 
     // Returns total weight; par[v] = tail of the edge entering v (par[root] = -1).
     int64_t run(int32_t root, std::vector<int32_t>& par) {
         const int64_t m = (int64_t)edges_.size();
-        // One heap per head node, built without a single meld: the node's incoming edges sorted
-        // by (weight, id) and chained through the LEFT child is a valid leftist heap (every right
-        // child is empty), and the sorts run in parallel.
+        // runs: edges grouped by head, each group sorted by (weight, id); weight and tail are
+        // copied next to the id so that walking a run never touches edges_
+        run_beg_.assign(n_ + 1, 0);
+        for (int64_t e = 0; e < m; e++) run_beg_[edges_[e].v + 1]++;
+        for (int32_t v = 0; v < n_; v++) run_beg_[v + 1] += run_beg_[v];
+        run_id_.resize(m); run_w_.resize(m); run_tail_.resize(m);
         {
-            std::vector<int64_t> cnt(n_ + 1, 0);
-            for (int64_t e = 0; e < m; e++) cnt[edges_[e].v + 1]++;
-            for (int32_t v = 0; v < n_; v++) cnt[v + 1] += cnt[v];
-            std::vector<int32_t> ids(m);
-            {
-                std::vector<int64_t> fill(cnt.begin(), cnt.end() - 1);
-                for (int64_t e = 0; e < m; e++) ids[fill[edges_[e].v]++] = (int32_t)e;
-            }
-#pragma omp parallel for schedule(dynamic, 64) num_threads(threads_)
-            for (int32_t v = 0; v < n_; v++) {
-                const int64_t b = cnt[v], e = cnt[v + 1];
-                if (b == e) continue;
-                std::sort(ids.begin() + b, ids.begin() + e, [&](int32_t x, int32_t y) {
-                    return edges_[x].w != edges_[y].w ? edges_[x].w < edges_[y].w : x < y;
-                });
-                for (int64_t k = b; k < e; k++) {
-                    Node& nd = node_[ids[k]];
-                    nd.key = edges_[ids[k]].w; nd.lazy = 0;
-                    nd.lc = k + 1 < e ? ids[k + 1] : -1; nd.rc = -1; nd.rank = 1;
-                }
-                heap_[v] = ids[b];
-            }
+            std::vector<int64_t> fill(run_beg_.begin(), run_beg_.end() - 1);
+            for (int64_t e = 0; e < m; e++) run_id_[fill[edges_[e].v]++] = (int32_t)e;
         }
-        std::vector<int32_t> seen(n_, -1), path(n_), Q(n_), in(n_, -1);
+#pragma omp parallel for schedule(dynamic, 64) num_threads(threads_)
+        for (int32_t v = 0; v < n_; v++) {
+            const int64_t b = run_beg_[v], e = run_beg_[v + 1];
+            std::sort(run_id_.begin() + b, run_id_.begin() + e, [&](int32_t x, int32_t y) {
+                return edges_[x].w != edges_[y].w ? edges_[x].w < edges_[y].w : x < y;
+            });
+            for (int64_t k = b; k < e; k++) { run_w_[k] = edges_[run_id_[k]].w; run_tail_[k] = edges_[run_id_[k]].u; }
+        }
+        pos_.assign(run_beg_.begin(), run_beg_.end() - 1);
+        run_off_.assign(n_, 0);
+        queue_.assign(n_, {});
+        queue_of_.resize(n_);
+        queue_off_.assign(n_, 0);
+        for (int32_t v = 0; v < n_; v++) {
+            fast_[v] = v;
+            queue_of_[v] = v;
+            if (run_beg_[v] < run_beg_[v + 1]) queue_[v].push_back({(int64_t)run_w_[run_beg_[v]], run_id_[run_beg_[v]], v});
+        }
+
+        std::vector<int32_t> seen(n_, -1), path(n_), Q(n_), in(n_, -1), members;
         seen[root] = root;
         int64_t res = 0;
         struct Cycle { int32_t node; int32_t time; int32_t eb, ee; };
@@ -82,28 +94,31 @@ public:
         for (int32_t s = 0; s < n_; s++) {
             int32_t u = s, qi = 0;
             while (seen[u] < 0) {
-                int32_t h = heap_[u];
-                if (h < 0) return -1;                   // node not reachable from the root
-                push_down(h);
-                const int32_t e = h;
-                const int32_t w = node_[e].key;
-                heap_[u] = meld(node_[e].lc, node_[e].rc);            // pop
-                // An edge inside the (contracted) component is dropped outright.  Charging its
-                // reduced weight and discounting the rest of the heap by it, as for any other
-                // popped edge, would cancel out with the next pop of this heap, and the one-edge
-                // "cycle" it would record expands to nothing.
-                if (find(edges_[e].u) == u) continue;
-                if (heap_[u] >= 0) node_[heap_[u]].lazy -= w;        // remaining keys become reduced costs
+                const int32_t q = queue_of_[u];
+                std::vector<Head>& heap = queue_[q];
+                if (heap.empty()) return -1;             // node not reachable from the root
+                const Head top = heap[0];
+                const int32_t e = top.id;
+                const int64_t w = top.key + queue_off_[q];            // reduced cost of e
+                const int32_t tail = run_tail_[pos_[top.run]];
+                advance(heap, top.run);                                // pop
+                // An edge inside the (contracted) node is dropped outright.  Charging its reduced
+                // cost and discounting the rest of the queue by it, as for any other popped edge,
+                // would cancel out with the next pop, and the one-edge "cycle" it would record
+                // expands to nothing.
+                if (find_fast(tail) == u) continue;
+                queue_off_[q] -= w;                                    // remaining keys become reduced costs
                 Q[qi] = e; path[qi++] = u; seen[u] = s;
                 res += w;
-                u = find(edges_[e].u);
+                u = find_fast(tail);
                 if (seen[u] == s) {                      // closed a cycle: contract it into u
-                    int32_t cyc = -1;
                     const int32_t end = qi, time = (int32_t)hist_.size();
+                    members.clear();
                     int32_t x;
-                    do { x = path[--qi]; cyc = meld(cyc, heap_[x]); } while (join(u, x));
-                    u = find(u);
-                    heap_[u] = cyc; seen[u] = -1;
+                    do { x = path[--qi]; members.push_back(queue_of_[x]); } while (join(u, x));
+                    u = find_fast(u);
+                    queue_of_[u] = merge_queues(members);
+                    seen[u] = -1;
                     cycles.push_back({u, time, (int32_t)cyc_edges.size(), (int32_t)cyc_edges.size() + (end - qi)});
                     for (int32_t i = qi; i < end; i++) cyc_edges.push_back(Q[i]);
                 }
@@ -123,46 +138,93 @@ public:
     }
 
 private:
-    struct Node { int32_t key, lazy, lc, rc; int32_t rank; };   // one cache line holds three
+    struct Head { int64_t key; int32_t id, run; };              // head of a run; key excludes the owner's offset
+    static bool before(const Head& a, const Head& b) { return a.key != b.key ? a.key < b.key : a.id < b.id; }
+
     int32_t n_;
     int threads_;
     const std::vector<CandEdge>& edges_;
-    std::vector<Node> node_;                                   // index = edge id
-    std::vector<int32_t> heap_;
-    std::vector<int32_t> uf_;                                  // <0: -size, else parent
+    std::vector<int64_t> run_beg_, pos_;                        // per original node: its run and the next unread entry
+    std::vector<int32_t> run_id_, run_w_, run_tail_;            // per run entry: edge id, weight, tail
+    std::vector<int64_t> run_off_;                              // per run: offset relative to its owner's
+    std::vector<std::vector<Head>> queue_;                      // binary min-heaps over run heads
+    std::vector<int32_t> queue_of_;                             // per representative: index of its queue
+    std::vector<int64_t> queue_off_;                            // per queue: offset of every key in it
+    std::vector<int32_t> uf_;                                   // <0: -size, else parent (no compression: undoable)
+    std::vector<int32_t> fast_;                                 // the same sets with path halving, for the forward pass
     std::vector<std::pair<int32_t, int32_t>> hist_;
 
-    void push_down(int32_t a) {
-        Node& nd = node_[a];
-        const int32_t z = nd.lazy;
-        if (z) {
-            nd.key += z;
-            if (nd.lc >= 0) node_[nd.lc].lazy += z;
-            if (nd.rc >= 0) node_[nd.rc].lazy += z;
-            nd.lazy = 0;
+    static void sift_down(std::vector<Head>& h, size_t i) {
+        const size_t n = h.size();
+        const Head x = h[i];
+        for (;;) {
+            size_t c = 2 * i + 1;
+            if (c >= n) break;
+            if (c + 1 < n && before(h[c + 1], h[c])) c++;
+            if (!before(h[c], x)) break;
+            h[i] = h[c];
+            i = c;
         }
+        h[i] = x;
     }
-    // Leftist heap meld; the right spine is O(log size) so the recursion is shallow.  Ties are
-    // broken towards the smaller edge id, which makes the result independent of meld order.
-    int32_t meld(int32_t a, int32_t b) {
-        if (a < 0) return b;
-        if (b < 0) return a;
-        push_down(a); push_down(b);
-        if (node_[a].key > node_[b].key || (node_[a].key == node_[b].key && a > b)) std::swap(a, b);
-        Node& na = node_[a];
-        na.rc = meld(na.rc, b);
-        const int32_t rl = na.lc >= 0 ? node_[na.lc].rank : 0, rr = node_[na.rc].rank;
-        if (rl < rr) std::swap(na.lc, na.rc);
-        na.rank = (na.rc >= 0 ? node_[na.rc].rank : 0) + 1;
-        return a;
+    static void sift_up(std::vector<Head>& h, size_t i) {
+        const Head x = h[i];
+        while (i > 0) {
+            const size_t p = (i - 1) / 2;
+            if (!before(x, h[p])) break;
+            h[i] = h[p];
+            i = p;
+        }
+        h[i] = x;
+    }
+    // The run at the top of the heap moves on to its next entry (or leaves the heap).
+    void advance(std::vector<Head>& h, int32_t run) {
+        const int64_t k = ++pos_[run];
+        if (k < run_beg_[run + 1]) {
+            h[0] = {(int64_t)run_w_[k] + run_off_[run], run_id_[k], run};
+        } else {
+            h[0] = h.back();
+            h.pop_back();
+            if (h.empty()) return;
+        }
+        sift_down(h, 0);
+    }
+    // All queues in `which` (distinct) become one: the smaller ones are moved into the largest.
+    int32_t merge_queues(const std::vector<int32_t>& which) {
+        int32_t base = which[0];
+        for (int32_t q : which) if (queue_[q].size() > queue_[base].size()) base = q;
+        std::vector<Head>& dst = queue_[base];
+        const size_t before_size = dst.size();
+        for (int32_t q : which) {
+            if (q == base) continue;
+            const int64_t delta = queue_off_[q] - queue_off_[base];
+            for (Head hd : queue_[q]) {
+                hd.key += delta;
+                run_off_[hd.run] += delta;
+                dst.push_back(hd);
+            }
+            std::vector<Head>().swap(queue_[q]);
+        }
+        const size_t added = dst.size() - before_size;
+        if (added * 8 > dst.size()) {
+            for (size_t i = dst.size() / 2; i-- > 0;) sift_down(dst, i);   // rebuild
+        } else {
+            for (size_t i = before_size; i < dst.size(); i++) sift_up(dst, i);
+        }
+        return base;
     }
     int32_t find(int32_t x) const { while (uf_[x] >= 0) x = uf_[x]; return x; }
+    int32_t find_fast(int32_t x) {
+        while (fast_[x] != x) { fast_[x] = fast_[fast_[x]]; x = fast_[x]; }
+        return x;
+    }
     bool join(int32_t a, int32_t b) {
         a = find(a); b = find(b);
         if (a == b) return false;
         if (uf_[a] > uf_[b]) std::swap(a, b);
         hist_.push_back({a, uf_[a]}); hist_.push_back({b, uf_[b]});
         uf_[a] += uf_[b]; uf_[b] = a;
+        fast_[b] = a;                                            // same representative in both structures
         return true;
     }
     void rollback(int32_t t) {
