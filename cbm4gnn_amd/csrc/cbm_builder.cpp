@@ -101,7 +101,7 @@ public:
                 const int32_t e = top.id;
                 const int64_t w = top.key + queue_off_[q];            // reduced cost of e
                 const int32_t tail = run_tail_[pos_[top.run]];
-                advance(heap, top.run);                                // pop
+                advance(heap, top.run, u);                             // pop
                 // An edge inside the (contracted) node is dropped outright.  Charging its reduced
                 // cost and discounting the rest of the queue by it, as for any other popped edge,
                 // would cancel out with the next pop, and the one-edge "cycle" it would record
@@ -177,10 +177,15 @@ private:
         }
         h[i] = x;
     }
-    // The run at the top of the heap moves on to its next entry (or leaves the heap).
-    void advance(std::vector<Head>& h, int32_t run) {
-        const int64_t k = ++pos_[run];
-        if (k < run_beg_[run + 1]) {
+    // The run at the top of the heap moves on to its next entry (or leaves the heap).  Entries
+    // whose tail already lies inside the owner `u` are skipped on the way: they stay internal
+    // for good and would only be dropped when they reached the top.
+    void advance(std::vector<Head>& h, int32_t run, int32_t u) {
+        const int64_t end = run_beg_[run + 1];
+        int64_t k = pos_[run] + 1;
+        while (k < end && find_fast(run_tail_[k]) == u) k++;
+        pos_[run] = k;
+        if (k < end) {
             h[0] = {(int64_t)run_w_[k] + run_off_[run], run_id_[k], run};
         } else {
             h[0] = h.back();
