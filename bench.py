@@ -137,7 +137,7 @@ def gcn_epoch_bench(args):
     hidden, classes = 128, 41
     ei = torch.from_numpy(w.edge_index)
     t0 = time.perf_counter()
-    op = build_operator(ei, alpha=alpha, normalized=True)
+    op = build_operator(ei, alpha=alpha, normalized=True, builder=args.builder)
     t_build = time.perf_counter() - t0
     dev = torch.device("cuda:0")
     op.to(dev)
@@ -227,7 +227,7 @@ def alpha_sweep_bench(args):
     alphas = [args.alpha] if args.alpha is not None else list(w.alphas)
     for alpha in alphas:
         t0 = time.perf_counter()
-        mat = cbm_matrix(ei, None, alpha=alpha, normalized=w.normalized)
+        mat = cbm_matrix(ei, None, alpha=alpha, normalized=w.normalized, builder=args.builder)
         t_build = time.perf_counter() - t0
         mat.to(xd.device)
         step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
@@ -265,6 +265,8 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--builder", choices=("host", "gpu"), default="host",
+                    help="where the format builder computes its row intersections (same format either way)")
     ap.add_argument("--probe", action="store_true",
                     help="counter run: 3 multiplies and 3 plain device copies of X (known size, for scaling "
                          "FETCH_SIZE / WRITE_SIZE), no timing, no JSON")
@@ -296,7 +298,7 @@ def main():
     d = args.d or w.d
     t_gen = time.perf_counter() - t0
     t0 = time.perf_counter()
-    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized)
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder)
     t_build = time.perf_counter() - t0
     n, nnz, n_edges = w.n, mat.nnz, mat.nnz_a
     norm = int(w.normalized)
@@ -372,7 +374,7 @@ def main():
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, alpha, d)) if args.scale == 1.0 else None,
                      "algorithmic_bytes": b_spmm, "avg_launch_ms": spmm_ms},
-        "host_s": {"generate": t_gen, "build_format": t_build},
+        "host_s": {"generate": t_gen, "build_format": t_build, "builder": args.builder, "build_phases": mat.build_seconds},
     }
     if not args.no_cpu:
         cpu, y_cpu = cpu_baseline(w, mat, x.numpy())

@@ -41,6 +41,11 @@ HOST_SYMBOLS = {
     "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
     "cbm_build_host_timings": (None, [C.POINTER(C.c_double)]),
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
+    "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),
+    "cbm_builder_arrays": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
+                                     C.POINTER(_P), C.POINTER(_I64)]),
+    "cbm_builder_finish": (C.c_int, [_P, _I32, _P, _I64, C.POINTER(CbmFormat)]),
+    "cbm_builder_free": (None, [_P]),
 }
 HIP_SYMBOLS = {
     "cbm_version": (C.c_char_p, []),
@@ -56,6 +61,8 @@ HIP_SYMBOLS = {
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "csr_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
+    "cbm_row_intersections_groups": (C.c_int, [_I32]),
+    "cbm_row_intersections": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _P, _I32, _P, _P, _I64, _P, _P]),
 }
 
 _host = None

@@ -149,10 +149,72 @@ def tree_levels(mst_row: np.ndarray, mst_col: np.ndarray):
     return parent.astype(np.int32), order.astype(np.int32), level_off.astype(np.int32)
 
 
+def _first_pair_capacity(nnz):
+    """Room for admissible pairs in the first pass of the GPU row intersections (12 B each); they
+    rarely outnumber the entries of the matrix, and a second, exactly sized pass runs if they do."""
+    return max(1 << 16, int(nnz))
+
+
+def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
+    """Staged build (``cbm_builder_*``) with ``cbm_row_intersections`` on the current HIP device.
+    Returns (status, seconds spent on upload + kernel + download)."""
+    import time
+    _require_gpu()
+    host, hip = _lib.host_lib(), _lib.hip_lib()
+    handle = C.c_void_p()
+    rc = host.cbm_builder_create(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()), ei_cpu.size(1), n, threads,
+                                 C.byref(handle))
+    if rc:
+        return rc, 0.0
+    try:
+        ptrs = [C.c_void_p() for _ in range(6)]
+        nnz = C.c_int64()
+        rc = host.cbm_builder_arrays(handle, *[C.byref(p) for p in ptrs], C.byref(nnz))
+        if rc:
+            return rc, 0.0
+        t0 = time.perf_counter()
+        dev = torch.device("cuda", torch.cuda.current_device())
+
+        def up(ptr, count, ctype, dtype):
+            a = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(ctype)), shape=(max(count, 1),))[:count]
+            return torch.from_numpy(a).to(dev)                      # borrowed host memory, copied by .to()
+
+        rowptr = up(ptrs[0], n + 1, C.c_int64, np.int64)
+        col = up(ptrs[1], nnz.value, C.c_int32, np.int32)
+        colptr_t = up(ptrs[2], n + 1, C.c_int64, np.int64)
+        row_t = up(ptrs[3], nnz.value, C.c_int32, np.int32)
+        after = up(ptrs[4], nnz.value, C.c_int64, np.int64)
+        row_nnz = up(ptrs[5], n, C.c_int32, np.int32)
+        groups = int(hip.cbm_row_intersections_groups(n))
+        counters = torch.zeros(groups * n, dtype=torch.int32, device=dev)
+        capacity = _first_pair_capacity(nnz.value)
+        while True:
+            ticket = torch.zeros(1, dtype=torch.int32, device=dev)
+            count = torch.zeros(1, dtype=torch.int64, device=dev)
+            pairs = torch.empty((capacity, 3), dtype=torch.int32, device=dev)
+            with torch.cuda.device(dev):
+                rc = hip.cbm_row_intersections(_ptr(rowptr), _ptr(col), _ptr(colptr_t), _ptr(row_t), _ptr(after),
+                                               _ptr(row_nnz), n, alpha, _ptr(counters), groups, _ptr(ticket), _ptr(pairs),
+                                               capacity, _ptr(count), _stream(dev))
+            if rc:
+                return rc, 0.0
+            found = int(count.item())                               # synchronises
+            if found <= capacity:
+                break
+            del pairs
+            capacity = found                                        # exact size, second pass
+        pairs_host = pairs[:found].cpu().contiguous()
+        t_pairs = time.perf_counter() - t0
+        rc = host.cbm_builder_finish(handle, alpha, _ptr(pairs_host) if found else None, found, C.byref(fmt))
+        return rc, t_pairs
+    finally:
+        host.cbm_builder_free(handle)
+
+
 class cbm_matrix:
 
     def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
-                 deltas_format="csr", threads=0):
+                 deltas_format="csr", threads=0, builder="host"):
         ei = torch.as_tensor(edge_index)
         if ei.dim() != 2 or ei.size(0) != 2:
             raise ValueError("Edge index should have shape (2, num_edges)")
@@ -170,14 +232,23 @@ class cbm_matrix:
         self.normalized = bool(normalized)
         self.deltas_format = deltas_format if deltas_format in ("csr", "coo") else "csr"
 
+        # builder: "host" = everything on the CPU; "gpu" = the row intersections (the dominant cost
+        # for large graphs) on the GPU, the rest on the CPU.  Both give the same format.
+        if builder not in ("host", "gpu"):
+            raise ValueError('builder must be "host" or "gpu"')
         fmt = _lib.CbmFormat()
-        rc = _lib.host_lib().cbm_build_host(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()),
-                                            ei_cpu.size(1), n, self.alpha, int(threads), C.byref(fmt))
+        if builder == "gpu":
+            rc, t_pairs = _build_with_gpu_intersections(ei_cpu, n, self.alpha, int(threads), fmt)
+        else:
+            rc, t_pairs = _lib.host_lib().cbm_build_host(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()),
+                                                         ei_cpu.size(1), n, self.alpha, int(threads), C.byref(fmt)), None
         try:
             _lib.check(rc, "cbm_build_host")
             t4 = (C.c_double * 4)()
             _lib.host_lib().cbm_build_host_timings(t4)
             self.build_seconds = dict(zip(("csr", "candidates", "arborescence", "deltas"), list(t4)))
+            if t_pairs is not None:
+                self.build_seconds["gpu_intersections"] = t_pairs       # upload + kernel + download, before "candidates"
 
             def take(ptr, count, dtype):
                 return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))

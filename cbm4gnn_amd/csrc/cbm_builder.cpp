@@ -245,165 +245,195 @@ template <class T> T* dup_array(const std::vector<T>& v) {
     return p;
 }
 
-}  // namespace
 
-// seconds spent by the last cbm_build_host call of this thread in: CSR + transpose, candidate
-// edges, arborescence, tree arrays + deltas
-thread_local double g_last_timings[4] = {0, 0, 0, 0};
+// The input matrix as the stages of the build see it.
+struct Graph {
+    int32_t N = 0;
+    int64_t nnzA = 0;
+    bool symmetric = false;
+    std::vector<int64_t> rp, tp;         // CSR offsets of A and of A^T
+    std::vector<int32_t> ci, tr;         // columns of A (ascending per row), rows of A^T (ascending per column)
+    std::vector<int32_t> nnz;            // entries per row of A
+    std::vector<int64_t> after;          // per entry k = (r, c) of A: first position in tr of a row id > r inside column c
+};
 
-extern "C" {
-
-void cbm_build_host_timings(double* out4) {
-    if (out4) for (int i = 0; i < 4; i++) out4[i] = g_last_timings[i];
+// COO -> CSR(A) with sorted unique columns, and its transpose.
+int build_graph(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int threads, Graph& g) {
+    g.N = N;
+    std::vector<int64_t>& rp = g.rp; std::vector<int32_t>& ci = g.ci; std::vector<int32_t>& nnz = g.nnz;
+    std::vector<int64_t>& tp = g.tp; std::vector<int32_t>& tr = g.tr;
+    rp.assign(N + 1, 0);
+    for (int64_t k = 0; k < E; k++) {
+        if (row[k] < 0 || row[k] >= N || col[k] < 0 || col[k] >= N) return CBM_ERR_SHAPE;
+        rp[row[k] + 1]++;
+    }
+    for (int32_t r = 0; r < N; r++) rp[r + 1] += rp[r];
+    ci.resize(E);
+    {
+        std::vector<int64_t> fill(rp.begin(), rp.end() - 1);
+        for (int64_t k = 0; k < E; k++) ci[fill[row[k]]++] = col[k];
+    }
+    nnz.resize(N);
+#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
+    for (int32_t r = 0; r < N; r++) {
+        auto b = ci.begin() + rp[r], e = ci.begin() + rp[r + 1];
+        std::sort(b, e);
+        nnz[r] = (int32_t)(std::unique(b, e) - b);
+    }
+    {   // compact duplicates away
+        int64_t w = 0;
+        for (int32_t r = 0; r < N; r++) {
+            const int64_t b = rp[r];
+            rp[r] = w;
+            if (w != b) std::memmove(&ci[w], &ci[b], sizeof(int32_t) * (size_t)nnz[r]);
+            w += nnz[r];
+        }
+        rp[N] = w;
+        ci.resize(w);
+    }
+    g.nnzA = rp[N];
+    tp.assign(N + 1, 0);
+    for (int64_t k = 0; k < g.nnzA; k++) tp[ci[k] + 1]++;
+    for (int32_t c = 0; c < N; c++) tp[c + 1] += tp[c];
+    tr.resize(g.nnzA);
+    g.after.resize(g.nnzA);
+    {
+        std::vector<int64_t> fill(tp.begin(), tp.end() - 1);
+        for (int32_t r = 0; r < N; r++)
+            for (int64_t k = rp[r]; k < rp[r + 1]; k++) {
+                tr[fill[ci[k]]] = r;                               // ascending r per column
+                g.after[k] = ++fill[ci[k]];
+            }
+    }
+    // symmetric pattern <=> CSR(A) == CSR(A^T) (both have ascending columns)
+    g.symmetric = rp == tp && ci == tr;
+    return CBM_OK;
 }
 
-const char* cbm_host_version(void) { return "cbm4gnn_amd host builder 0.1"; }
-
-void cbm_format_free(cbm_format* f) {
-    if (!f) return;
-    std::free(f->rowptr); std::free(f->idx); std::free(f->parent); std::free(f->order);
-    std::free(f->level_off); std::free(f->mst_row); std::free(f->mst_col);
-    std::memset(f, 0, sizeof(*f));
-}
-
-int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
-                      int32_t* sched_out) {
-    if (!rowptr || !sched_out) return CBM_ERR_NULL;
-    if (n < 0) return CBM_ERR_SHAPE;
-    try {
-        // counting sort by gather rounds (64 entries each), longest first, stable
-        std::vector<int32_t> rounds(n);
-        int32_t max_rounds = 0;
-        for (int32_t r = 0; r < n; r++) {
-            const int32_t len = rowptr[r + 1] - rowptr[r];
-            if (len < 0) return CBM_ERR_SHAPE;
-            rounds[r] = (len + 63) / 64;
-            max_rounds = std::max(max_rounds, rounds[r]);
-        }
-        std::vector<int64_t> first(max_rounds + 2, 0);
-        for (int32_t r = 0; r < n; r++) first[max_rounds - rounds[r] + 1]++;
-        for (int32_t b = 0; b <= max_rounds; b++) first[b + 1] += first[b];
-        for (int32_t r = 0; r < n; r++) {
-            int32_t* o = sched_out + 4 * first[max_rounds - rounds[r]]++;
-            const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
-            o[0] = rowptr[r]; o[1] = rowptr[r + 1]; o[2] = r;
-            std::memcpy(&o[3], &scale, sizeof(float));
-        }
-        return CBM_OK;
-    } catch (const std::bad_alloc&) {
-        return CBM_ERR_ALLOC;
+// Candidate edges of the distance graph (reference rule, cbm_extensions.cpp:75-103) from the
+// admissible pairs of one row i, in the reference's emission order: the edge from the virtual
+// root, then for every j > i ascending the edges j -> i and i -> j.
+//   pair (i, j>i) with s shared columns: h = nnz_i + nnz_j - 2s;
+//   j -> i admitted iff h < nnz_i - alpha  <=>  2s > nnz_j + alpha
+//   i -> j admitted iff h < nnz_j - alpha  <=>  2s > nnz_i + alpha
+inline void emit_row(const Graph& g, int32_t alpha, int32_t i, std::vector<std::pair<int32_t, int32_t>>& adm,
+                     std::vector<CandEdge>& o) {
+    const int32_t ni = g.nnz[i];
+    o.push_back({g.N, i, ni});
+    std::sort(adm.begin(), adm.end());
+    for (auto& js : adm) {
+        const int32_t j = js.first, nj = g.nnz[j];
+        const int32_t h = ni + nj - 2 * js.second;
+        if (h < ni - alpha) o.push_back({j, i, h});
+        if (h < nj - alpha) o.push_back({i, j, h});
     }
 }
 
-int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t alpha,
-                   int32_t threads, cbm_format* out) {
-    if (!out) return CBM_ERR_NULL;
-    std::memset(out, 0, sizeof(*out));
-    if ((!row || !col) && E > 0) return CBM_ERR_NULL;
-    if (N <= 0 || E < 0 || N >= (1 << 30)) return CBM_ERR_SHAPE;
-    if (threads <= 0) threads = omp_get_max_threads();
-    double t_mark = omp_get_wtime();
-    auto lap = [&](int slot) { const double t = omp_get_wtime(); g_last_timings[slot] = t - t_mark; t_mark = t; };
-    try {
-        // ---- COO -> CSR(A) with sorted unique columns, and its transpose -----------------------
-        std::vector<int64_t> rp(N + 1, 0);
-        for (int64_t k = 0; k < E; k++) {
-            if (row[k] < 0 || row[k] >= N || col[k] < 0 || col[k] >= N) return CBM_ERR_SHAPE;
-            rp[row[k] + 1]++;
-        }
-        for (int32_t r = 0; r < N; r++) rp[r + 1] += rp[r];
-        std::vector<int32_t> ci(E);
-        {
-            std::vector<int64_t> fill(rp.begin(), rp.end() - 1);
-            for (int64_t k = 0; k < E; k++) ci[fill[row[k]]++] = col[k];
-        }
-        std::vector<int32_t> nnz(N);
-#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
-        for (int32_t r = 0; r < N; r++) {
-            auto b = ci.begin() + rp[r], e = ci.begin() + rp[r + 1];
-            std::sort(b, e);
-            nnz[r] = (int32_t)(std::unique(b, e) - b);
-        }
-        {   // compact duplicates away
-            int64_t w = 0;
-            for (int32_t r = 0; r < N; r++) {
-                const int64_t b = rp[r];
-                rp[r] = w;
-                if (w != b) std::memmove(&ci[w], &ci[b], sizeof(int32_t) * (size_t)nnz[r]);
-                w += nnz[r];
-            }
-            rp[N] = w;
-            ci.resize(w);
-        }
-        const int64_t nnzA = rp[N];
-        std::vector<int64_t> tp(N + 1, 0);
-        for (int64_t k = 0; k < nnzA; k++) tp[ci[k] + 1]++;
-        for (int32_t c = 0; c < N; c++) tp[c + 1] += tp[c];
-        std::vector<int32_t> tr(nnzA);
-        {
-            std::vector<int64_t> fill(tp.begin(), tp.end() - 1);
-            for (int32_t r = 0; r < N; r++)
-                for (int64_t k = rp[r]; k < rp[r + 1]; k++) tr[fill[ci[k]]++] = r;   // ascending r per column
-        }
+inline int concat_chunks(std::vector<std::vector<CandEdge>>& chunk_out, std::vector<CandEdge>& cand) {
+    size_t tot = 0;
+    for (auto& o : chunk_out) tot += o.size();
+    if (tot >= (size_t)INT32_MAX) return CBM_ERR_SHAPE;
+    cand.reserve(tot);
+    for (auto& o : chunk_out) { cand.insert(cand.end(), o.begin(), o.end()); std::vector<CandEdge>().swap(o); }
+    return CBM_OK;
+}
 
-        // symmetric pattern <=> CSR(A) == CSR(A^T) (both have ascending columns)
-        const bool symmetric = rp == tp && ci == tr;
-        lap(0);
-        // ---- candidate edges (reference rule, cpp:75-103), streamed and pruned ------------------
-        // pair (i, j>i) with s shared columns: h = nnz_i + nnz_j - 2s;
-        //   j -> i admitted iff h < nnz_i - alpha  <=>  2s > nnz_j + alpha
-        //   i -> j admitted iff h < nnz_j - alpha  <=>  2s > nnz_i + alpha
-        const int32_t CH = 64;
-        const int32_t n_chunks = (N + CH - 1) / CH;
-        std::vector<std::vector<CandEdge>> chunk_out(n_chunks);
+// Row intersections on the host: |row_i ^ row_j| streamed row by row with a per-thread sparse
+// accumulator, only admissible pairs kept.
+int candidates_host(const Graph& g, int32_t alpha, int threads, std::vector<CandEdge>& cand) {
+    const int32_t N = g.N;
+    const int32_t CH = 64;
+    const int32_t n_chunks = (N + CH - 1) / CH;
+    std::vector<std::vector<CandEdge>> chunk_out(n_chunks);
 #pragma omp parallel num_threads(threads)
-        {
-            std::vector<int32_t> cnt(N, 0), touched;
-            std::vector<std::pair<int32_t, int32_t>> adm;
-            touched.reserve(1024);
+    {
+        std::vector<int32_t> cnt(N, 0), touched;
+        std::vector<std::pair<int32_t, int32_t>> adm;
+        touched.reserve(1024);
 #pragma omp for schedule(dynamic, 1)
-            for (int32_t ch = 0; ch < n_chunks; ch++) {
-                std::vector<CandEdge>& o = chunk_out[ch];
-                const int32_t i_end = std::min(N, (ch + 1) * CH);
-                for (int32_t i = ch * CH; i < i_end; i++) {
-                    const int32_t ni = nnz[i];
-                    o.push_back({N, i, ni});
-                    touched.clear();
-                    for (int64_t k = rp[i]; k < rp[i + 1]; k++) {
-                        const int32_t c = ci[k];
-                        const int32_t* lo = tr.data() + tp[c];
-                        const int32_t* hi = tr.data() + tp[c + 1];
-                        for (const int32_t* q = std::upper_bound(lo, hi, i); q < hi; ++q) {
-                            const int32_t j = *q;
-                            if (cnt[j]++ == 0) touched.push_back(j);
-                        }
-                    }
-                    adm.clear();
-                    for (int32_t j : touched) {
-                        const int32_t s = cnt[j];
-                        cnt[j] = 0;
-                        if (2 * s > std::min(ni, nnz[j]) + alpha) adm.push_back({j, s});
-                    }
-                    std::sort(adm.begin(), adm.end());
-                    for (auto& js : adm) {
-                        const int32_t j = js.first, nj = nnz[j];
-                        const int32_t h = ni + nj - 2 * js.second;
-                        if (h < ni - alpha) o.push_back({j, i, h});
-                        if (h < nj - alpha) o.push_back({i, j, h});
+        for (int32_t ch = 0; ch < n_chunks; ch++) {
+            std::vector<CandEdge>& o = chunk_out[ch];
+            const int32_t i_end = std::min(N, (ch + 1) * CH);
+            for (int32_t i = ch * CH; i < i_end; i++) {
+                const int32_t ni = g.nnz[i];
+                touched.clear();
+                for (int64_t k = g.rp[i]; k < g.rp[i + 1]; k++) {
+                    const int32_t* q = g.tr.data() + g.after[k];
+                    const int32_t* hi = g.tr.data() + g.tp[g.ci[k] + 1];
+                    for (; q < hi; ++q) {
+                        const int32_t j = *q;
+                        if (cnt[j]++ == 0) touched.push_back(j);
                     }
                 }
+                adm.clear();
+                for (int32_t j : touched) {
+                    const int32_t s = cnt[j];
+                    cnt[j] = 0;
+                    if (2 * s > std::min(ni, g.nnz[j]) + alpha) adm.push_back({j, s});
+                }
+                emit_row(g, alpha, i, adm, o);
             }
         }
-        std::vector<CandEdge> cand;
-        {
-            size_t tot = 0;
-            for (auto& o : chunk_out) tot += o.size();
-            cand.reserve(tot);
-            for (auto& o : chunk_out) { cand.insert(cand.end(), o.begin(), o.end()); std::vector<CandEdge>().swap(o); }
-        }
-        if (cand.size() >= (size_t)INT32_MAX) return CBM_ERR_SHAPE;
+    }
+    return concat_chunks(chunk_out, cand);
+}
 
-        lap(1);
+// The same candidate list from row intersections computed elsewhere (on the GPU): pairs (i, j, s)
+// with i < j and s = |row_i ^ row_j|, in any order, holding at least every admissible pair.
+int candidates_from_pairs(const Graph& g, int32_t alpha, const cbm_pair* pairs, int64_t n_pairs, int threads,
+                          std::vector<CandEdge>& cand) {
+    const int32_t N = g.N;
+    std::vector<int64_t> first(N + 1, 0);
+    for (int64_t p = 0; p < n_pairs; p++) {
+        const cbm_pair& q = pairs[p];
+        if (q.i < 0 || q.j <= q.i || q.j >= N || q.s <= 0 || q.s > std::min(g.nnz[q.i], g.nnz[q.j])) return CBM_ERR_SHAPE;
+        first[q.i + 1]++;
+    }
+    for (int32_t i = 0; i < N; i++) first[i + 1] += first[i];
+    std::vector<std::pair<int32_t, int32_t>> by_row(n_pairs);
+    {
+        std::vector<int64_t> fill(first.begin(), first.end() - 1);
+        for (int64_t p = 0; p < n_pairs; p++) by_row[fill[pairs[p].i]++] = {pairs[p].j, pairs[p].s};
+    }
+    const int32_t CH = 64;
+    const int32_t n_chunks = (N + CH - 1) / CH;
+    std::vector<std::vector<CandEdge>> chunk_out(n_chunks);
+    bool duplicate = false;
+#pragma omp parallel num_threads(threads)
+    {
+        std::vector<std::pair<int32_t, int32_t>> adm;
+#pragma omp for schedule(dynamic, 1)
+        for (int32_t ch = 0; ch < n_chunks; ch++) {
+            const int32_t i_end = std::min(N, (ch + 1) * CH);
+            for (int32_t i = ch * CH; i < i_end; i++) {
+                adm.clear();
+                for (int64_t p = first[i]; p < first[i + 1]; p++)
+                    if (2 * by_row[p].second > std::min(g.nnz[i], g.nnz[by_row[p].first]) + alpha) adm.push_back(by_row[p]);
+                emit_row(g, alpha, i, adm, chunk_out[ch]);              // sorts adm by j
+                for (size_t a = 1; a < adm.size(); a++)
+                    if (adm[a].first == adm[a - 1].first) {
+#pragma omp atomic write
+                        duplicate = true;
+                    }
+            }
+        }
+    }
+    if (duplicate) return CBM_ERR_SHAPE;
+    return concat_chunks(chunk_out, cand);
+}
+
+// seconds spent by the last build of this thread in: CSR + transpose, candidate edges,
+// arborescence, tree arrays + deltas
+thread_local double g_last_timings[4] = {0, 0, 0, 0};
+
+// Arborescence, tree arrays, signed deltas.
+int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, cbm_format* out, double t_mark) {
+    const int32_t N = g.N;
+    const std::vector<int64_t>& rp = g.rp; const std::vector<int32_t>& ci = g.ci; const std::vector<int32_t>& nnz = g.nnz;
+    const int64_t nnzA = g.nnzA;
+    const bool symmetric = g.symmetric;
+    auto lap = [&](int slot) { const double t = omp_get_wtime(); g_last_timings[slot] = t - t_mark; t_mark = t; };
+    {
         // ---- arborescence ----------------------------------------------------------------------
         std::vector<int32_t> par;
         int64_t weight;
@@ -491,10 +521,126 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N,
         out->order = dup_array(order); out->level_off = dup_array(level_off);
         out->mst_row = dup_array(mst_row); out->mst_col = dup_array(mst_col);
         return CBM_OK;
+    }
+}
+
+}  // namespace
+
+struct cbm_builder {
+    Graph g;
+    int threads = 1;
+};
+
+extern "C" {
+
+void cbm_build_host_timings(double* out4) {
+    if (out4) for (int i = 0; i < 4; i++) out4[i] = g_last_timings[i];
+}
+
+const char* cbm_host_version(void) { return "cbm4gnn_amd host builder 0.1"; }
+
+void cbm_format_free(cbm_format* f) {
+    if (!f) return;
+    std::free(f->rowptr); std::free(f->idx); std::free(f->parent); std::free(f->order);
+    std::free(f->level_off); std::free(f->mst_row); std::free(f->mst_col);
+    std::memset(f, 0, sizeof(*f));
+}
+
+int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
+                      int32_t* sched_out) {
+    if (!rowptr || !sched_out) return CBM_ERR_NULL;
+    if (n < 0) return CBM_ERR_SHAPE;
+    try {
+        // counting sort by gather rounds (64 entries each), longest first, stable
+        std::vector<int32_t> rounds(n);
+        int32_t max_rounds = 0;
+        for (int32_t r = 0; r < n; r++) {
+            const int32_t len = rowptr[r + 1] - rowptr[r];
+            if (len < 0) return CBM_ERR_SHAPE;
+            rounds[r] = (len + 63) / 64;
+            max_rounds = std::max(max_rounds, rounds[r]);
+        }
+        std::vector<int64_t> first(max_rounds + 2, 0);
+        for (int32_t r = 0; r < n; r++) first[max_rounds - rounds[r] + 1]++;
+        for (int32_t b = 0; b <= max_rounds; b++) first[b + 1] += first[b];
+        for (int32_t r = 0; r < n; r++) {
+            int32_t* o = sched_out + 4 * first[max_rounds - rounds[r]]++;
+            const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
+            o[0] = rowptr[r]; o[1] = rowptr[r + 1]; o[2] = r;
+            std::memcpy(&o[3], &scale, sizeof(float));
+        }
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        return CBM_ERR_ALLOC;
+    }
+}
+
+int cbm_builder_create(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t threads,
+                       cbm_builder** out) {
+    if (!out) return CBM_ERR_NULL;
+    *out = nullptr;
+    if ((!row || !col) && E > 0) return CBM_ERR_NULL;
+    if (N <= 0 || E < 0 || N >= (1 << 30)) return CBM_ERR_SHAPE;
+    if (threads <= 0) threads = omp_get_max_threads();
+    const double t0 = omp_get_wtime();
+    cbm_builder* b = nullptr;
+    try {
+        b = new cbm_builder();
+        b->threads = threads;
+        if (int rc = build_graph(row, col, E, N, threads, b->g)) { delete b; return rc; }
+    } catch (const std::bad_alloc&) {
+        delete b;
+        return CBM_ERR_ALLOC;
+    }
+    g_last_timings[0] = omp_get_wtime() - t0;
+    g_last_timings[1] = g_last_timings[2] = g_last_timings[3] = 0;
+    *out = b;
+    return CBM_OK;
+}
+
+int cbm_builder_arrays(const cbm_builder* b, const int64_t** rowptr, const int32_t** col, const int64_t** colptr_t,
+                       const int32_t** row_t, const int64_t** after, const int32_t** row_nnz, int64_t* nnz) {
+    if (!b) return CBM_ERR_NULL;
+    if (rowptr) *rowptr = b->g.rp.data();
+    if (col) *col = b->g.ci.data();
+    if (colptr_t) *colptr_t = b->g.tp.data();
+    if (row_t) *row_t = b->g.tr.data();
+    if (after) *after = b->g.after.data();
+    if (row_nnz) *row_nnz = b->g.nnz.data();
+    if (nnz) *nnz = b->g.nnzA;
+    return CBM_OK;
+}
+
+int cbm_builder_finish(cbm_builder* b, int32_t alpha, const cbm_pair* pairs, int64_t n_pairs, cbm_format* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if (!b || (n_pairs > 0 && !pairs)) return CBM_ERR_NULL;
+    const double t0 = omp_get_wtime();
+    try {
+        std::vector<CandEdge> cand;
+        const int rc = n_pairs < 0 ? candidates_host(b->g, alpha, b->threads, cand)
+                                   : candidates_from_pairs(b->g, alpha, pairs, n_pairs, b->threads, cand);
+        if (rc) return rc;
+        const double t1 = omp_get_wtime();
+        g_last_timings[1] = t1 - t0;
+        return finish_format(b->g, cand, b->threads, out, t1);
     } catch (const std::bad_alloc&) {
         cbm_format_free(out);
         return CBM_ERR_ALLOC;
     }
+}
+
+void cbm_builder_free(cbm_builder* b) { delete b; }
+
+int cbm_build_host(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t alpha,
+                   int32_t threads, cbm_format* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    cbm_builder* b = nullptr;
+    if (int rc = cbm_builder_create(row, col, E, N, threads, &b)) return rc;
+    const int rc = cbm_builder_finish(b, alpha, nullptr, -1, out);
+    cbm_builder_free(b);
+    return rc;
 }
 
 }  // extern "C"

@@ -571,6 +571,109 @@ inline Tiling pick_tiling(int d, int64_t ld_a, int64_t ld_b, const void* pa, con
 // SpMM kernel choice: 0 = automatic, 1 = always one wave per row, 2 = slabs whenever the shape allows
 int g_spmm_kernel = 0;
 
+// ---------------------------------------------------------------------------------------------
+// (3) Row intersections for the builder: all pairs (i, j > i) of rows of A with
+// 2 |row_i ^ row_j| > min(nnz_i, nnz_j) + alpha, the pairs the distance graph can admit
+// (cbm_extensions.cpp:75-103; the reference gets |row_i ^ row_j| from mkl_sparse_syrk).
+//
+// One workgroup owns a private array of n counters and takes rows from a shared ticket.  For a
+// row i it walks, for every column c of the row, the rows j > i of that column (one wavefront per
+// column, lanes along the column: coalesced) three times, with a barrier in between:
+//   1. increment counter j;
+//   2. read counter j; where it passes the admission test, swap it with 0 -- exactly one thread
+//      per distinct j gets the count and appends (i, j, s);
+//   3. store 0 to counter j, so that the array is clean for the next row.
+// The increments and swaps are workgroup-scope atomics (they execute in the XCD's L2, never in
+// the L1), the reads and the clearing stores go to the L2 as well; only the ticket and the output
+// cursor are device-scope.  The L2's atomic units bound the kernel: reading before swapping and
+// clearing with stores instead of swapping every counter took it from 0.78 s to 0.61 s on
+// 132 534 rows x 620 entries (25 G increments).
+// ---------------------------------------------------------------------------------------------
+constexpr int kIsectWaves = 16;
+constexpr int kIsectUnroll = 4;
+
+__global__ __launch_bounds__(kWave * kIsectWaves) void row_intersections(
+    const int64_t* __restrict__ rowptr, const int32_t* __restrict__ col, const int64_t* __restrict__ colptr_t,
+    const int32_t* __restrict__ row_t, const int64_t* __restrict__ after, const int32_t* __restrict__ row_nnz,
+    int n, int alpha, uint32_t* __restrict__ counters, uint32_t* __restrict__ ticket, cbm_pair* __restrict__ pairs,
+    unsigned long long capacity, unsigned long long* __restrict__ n_pairs) {
+    __shared__ int s_row;
+    uint32_t* __restrict__ cnt = counters + (size_t)blockIdx.x * n;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    for (;;) {
+        if (threadIdx.x == 0) s_row = (int)atomicAdd(ticket, 1u);
+        __syncthreads();
+        const int i = s_row;
+        if (i >= n) return;                                  // every thread of the workgroup sees the same ticket
+        const int64_t b = rowptr[i], e = rowptr[i + 1];
+        const int ni = row_nnz[i];
+        // kIsectUnroll list entries per lane and step: the loads of a step, then its atomics, are in
+        // flight together (positions past the end of the list are clamped to its last entry and
+        // masked out afterwards)
+        for (int64_t k = b + wave; k < e; k += kIsectWaves) {
+            const int64_t hi = colptr_t[col[k] + 1];
+            for (int64_t t0 = after[k]; t0 < hi; t0 += kWave * kIsectUnroll) {
+                int j[kIsectUnroll];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++) j[u] = row_t[min(t0 + u * kWave + lane, hi - 1)];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++)
+                    if (t0 + u * kWave + lane < hi)
+                        __hip_atomic_fetch_add(&cnt[j[u]], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        __syncthreads();
+        for (int64_t k = b + wave; k < e; k += kIsectWaves) {
+            const int64_t hi = colptr_t[col[k] + 1];
+            for (int64_t t0 = after[k]; t0 < hi; t0 += kWave * kIsectUnroll) {   // whole wavefront iterates together (ballot below)
+                int j[kIsectUnroll], sh[kIsectUnroll], nj[kIsectUnroll];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++) j[u] = row_t[min(t0 + u * kWave + lane, hi - 1)];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++) {
+                    // a read at the L2 (the counters are only ever touched there), then the claim
+                    // by exchange for the few that pass; everything is zeroed by plain stores below
+                    sh[u] = (int)__hip_atomic_load(&cnt[j[u]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    nj[u] = row_nnz[j[u]];
+                }
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++) {
+                    bool keep = t0 + u * kWave + lane < hi && 2 * sh[u] > min(ni, nj[u]) + alpha;
+                    if (keep) {
+                        sh[u] = (int)__hip_atomic_exchange(&cnt[j[u]], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        keep = sh[u] > 0;
+                    }
+                    const unsigned long long mask = __ballot(keep);
+                    if (mask) {
+                        unsigned long long base = 0;
+                        const int leader = __ffsll((long long)mask) - 1;
+                        if (lane == leader) base = atomicAdd(n_pairs, (unsigned long long)__popcll(mask));
+                        base = __shfl(base, leader, kWave);
+                        if (keep) {
+                            const unsigned long long at = base + __popcll(mask & ((1ull << lane) - 1ull));
+                            if (at < capacity) pairs[at] = cbm_pair{i, j[u], sh[u]};
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        for (int64_t k = b + wave; k < e; k += kIsectWaves) {
+            const int64_t hi = colptr_t[col[k] + 1];
+            for (int64_t t0 = after[k]; t0 < hi; t0 += kWave * kIsectUnroll) {
+                int j[kIsectUnroll];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++) j[u] = row_t[min(t0 + u * kWave + lane, hi - 1)];
+#pragma unroll
+                for (int u = 0; u < kIsectUnroll; u++)
+                    __hip_atomic_store(&cnt[j[u]], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();                                     // counters are zero again; s_row may be overwritten
+    }
+}
+
 // How a multiply of feature width d runs.
 struct SlabPlan {
     int lpe = 0;            // lanes per delta entry: 8 -> 128-byte slabs, 16 -> 256-byte slabs, 0 -> one wave per row
@@ -873,6 +976,31 @@ int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t 
 int64_t cbm_relayout_floats(int32_t n, int32_t d) {
     if (n <= 0 || d <= 0) return 0;
     return (int64_t)n * padded_slab_count(d) * 32;
+}
+
+int cbm_row_intersections_groups(int32_t n) {
+    if (n <= 0) return 0;
+    // 16 workgroups per XCD (measured on 132 534 rows x 620 entries: 1.32 s with 40 workgroups,
+    // 0.78 s with 128, no better with 256 or 512: the L2's atomic units are the limit), fewer when
+    // the private counter arrays would together exceed 2 GB, at least one per XCD
+    const int64_t fit = ((int64_t)2 << 30) / ((int64_t)n * 4) / kXcds;
+    const int g = fit < 1 ? 1 : (fit > 16 ? 16 : (int)fit);
+    return g * kXcds;
+}
+
+int cbm_row_intersections(const int64_t* rowptr, const int32_t* col, const int64_t* colptr_t, const int32_t* row_t,
+                          const int64_t* after, const int32_t* row_nnz, int32_t n, int32_t alpha, uint32_t* counters,
+                          int32_t groups, uint32_t* ticket, cbm_pair* pairs, int64_t capacity,
+                          unsigned long long* n_pairs, void* stream) {
+    if (n < 0 || capacity < 0 || groups < 0) return CBM_ERR_SHAPE;
+    if (n == 0) return CBM_OK;
+    if (!rowptr || !col || !colptr_t || !row_t || !after || !row_nnz || !counters || !ticket || !n_pairs) return CBM_ERR_NULL;
+    if (capacity > 0 && !pairs) return CBM_ERR_NULL;
+    if (groups < 1) return CBM_ERR_SHAPE;
+    hipLaunchKernelGGL(row_intersections, dim3((unsigned)groups), dim3(kWave * kIsectWaves), 0,
+                       static_cast<hipStream_t>(stream), rowptr, col, colptr_t, row_t, after, row_nnz, n, alpha,
+                       counters, ticket, pairs, (unsigned long long)capacity, n_pairs);
+    return check_launch();
 }
 
 int cbm_set_spmm_occupancy(int waves_per_simd) {

@@ -86,6 +86,30 @@ const char* cbm_host_version(void);
 int cbm_build_host(const int32_t* row, const int32_t* col, int64_t n_edges, int32_t n, int32_t alpha,
                    int32_t threads, cbm_format* out);
 
+/* The same build in stages, so that the row intersections -- the dominant cost for large graphs
+ * -- can be computed elsewhere (cbm_row_intersections on the GPU) and handed back:
+ *   cbm_builder_create   CSR of the input with sorted unique columns, and its transpose
+ *   cbm_builder_arrays   HOST views of those arrays (valid until cbm_builder_free):
+ *                          rowptr[n+1], col[nnz]           rows of A
+ *                          colptr_t[n+1], row_t[nnz]       columns of A (row ids ascending)
+ *                          after[nnz]                      per entry (r, c) of A: first position in
+ *                                                          row_t of a row id > r inside column c
+ *                          row_nnz[n]                      entries per row
+ *   cbm_builder_finish   candidate edges, arborescence, deltas.  pairs = (i, j, s) with i < j and
+ *                        s = |row_i ^ row_j| in any order, holding at least every pair with
+ *                        2 s > min(nnz_i, nnz_j) + alpha; n_pairs < 0 computes them on the host.
+ * cbm_build_host is create + finish(n_pairs = -1) + free.  Replaces the mkl_sparse_syrk step of
+ * cbm_init_v1_/_v2_ (cbm_extensions.cpp:46-65) as a separable stage. */
+typedef struct cbm_builder cbm_builder;
+struct cbm_pair { int32_t i, j, s; };
+int cbm_builder_create(const int32_t* row, const int32_t* col, int64_t n_edges, int32_t n, int32_t threads,
+                       cbm_builder** out);
+int cbm_builder_arrays(const cbm_builder* b, const int64_t** rowptr, const int32_t** col, const int64_t** colptr_t,
+                       const int32_t** row_t, const int64_t** after, const int32_t** row_nnz, int64_t* nnz);
+int cbm_builder_finish(cbm_builder* b, int32_t alpha, const struct cbm_pair* pairs, int64_t n_pairs,
+                       struct cbm_format* out);
+void cbm_builder_free(cbm_builder* b);
+
 void cbm_format_free(cbm_format* f);
 
 /* Seconds the calling thread's last cbm_build_host spent in its four phases: CSR + transpose,
@@ -191,6 +215,20 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int6
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
                         const float* X_dev, float* Y_dev, float* workspace_dev, int32_t n, int32_t d,
                         int64_t ldx, int64_t ldy, int32_t flags, void* stream);
+
+/* Row intersections for the builder on the GPU: appends to pairs[] every (i, j > i, s) with
+ * s = |row_i ^ row_j| and 2 s > min(nnz_i, nnz_j) + alpha, in no particular order, and adds their
+ * number to *n_pairs (which may exceed capacity: then only the first `capacity` were stored and the
+ * call must be repeated with a larger buffer).  The six input arrays are device copies of
+ * cbm_builder_arrays(); counters = groups * n uint32 and ticket = 1 uint32 and n_pairs = 1 uint64,
+ * all zero on entry (the counters are zero again on exit); groups = number of workgroups, e.g.
+ * cbm_row_intersections_groups(n).  Feed the result to cbm_builder_finish.
+ * Replaces mkl_sparse_syrk + the admission scan of cbm_init_v1_/_v2_ (cbm_extensions.cpp:46-103). */
+int cbm_row_intersections_groups(int32_t n);
+int cbm_row_intersections(const int64_t* rowptr_dev, const int32_t* col_dev, const int64_t* colptr_t_dev,
+                          const int32_t* row_t_dev, const int64_t* after_dev, const int32_t* row_nnz_dev, int32_t n,
+                          int32_t alpha, uint32_t* counters_dev, int32_t groups, uint32_t* ticket_dev,
+                          struct cbm_pair* pairs_dev, int64_t capacity, unsigned long long* n_pairs_dev, void* stream);
 
 /* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */

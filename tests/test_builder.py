@@ -208,3 +208,89 @@ def test_graphs_with_empty_rows_single_node_and_self_loop_only(orc):
     assert orc.check_format(ei.numpy(), 5, mat.rowptr.numpy(), _u32(mat.idx), mat.mst_row.numpy(), mat.mst_col.numpy())
     one = cbm_matrix(torch.tensor([[0], [0]], dtype=torch.int32), None, alpha=0, normalized=True)
     assert one.num_rows == 1 and one.nnz == 1 and one.n_levels == 1 and float(one.col_multiplier[0]) == 1.0
+
+
+def _staged_build(ei, n, alpha, pairs):
+    """cbm_builder_create -> (arrays) -> cbm_builder_finish; returns (status, format arrays, host arrays)."""
+    host = _lib.host_lib()
+    row = np.ascontiguousarray(ei[0], np.int32); col = np.ascontiguousarray(ei[1], np.int32)
+    handle = C.c_void_p()
+    assert host.cbm_builder_create(row.ctypes.data_as(C.c_void_p), col.ctypes.data_as(C.c_void_p), ei.shape[1], n, 2,
+                                   C.byref(handle)) == 0
+    try:
+        ptrs = [C.c_void_p() for _ in range(6)]
+        nnz = C.c_int64()
+        assert host.cbm_builder_arrays(handle, *[C.byref(p) for p in ptrs], C.byref(nnz)) == 0
+        take = lambda p, count, ct: np.ctypeslib.as_array(C.cast(p, C.POINTER(ct)), shape=(max(count, 1),))[:count].copy()
+        arrays = dict(rowptr=take(ptrs[0], n + 1, C.c_int64), col=take(ptrs[1], nnz.value, C.c_int32),
+                      colptr_t=take(ptrs[2], n + 1, C.c_int64), row_t=take(ptrs[3], nnz.value, C.c_int32),
+                      after=take(ptrs[4], nnz.value, C.c_int64), row_nnz=take(ptrs[5], n, C.c_int32))
+        fmt = _lib.CbmFormat()
+        if pairs is None:
+            rc = host.cbm_builder_finish(handle, alpha, None, -1, C.byref(fmt))
+        else:
+            p = np.ascontiguousarray(pairs, np.int32).reshape(-1, 3)
+            rc = host.cbm_builder_finish(handle, alpha, p.ctypes.data_as(C.c_void_p) if len(p) else None, len(p), C.byref(fmt))
+        out = None
+        if rc == 0:
+            g = lambda ptr, count: np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].copy()
+            out = dict(nnz=int(fmt.nnz), n_candidates=int(fmt.n_candidates), rowptr=g(fmt.rowptr, n + 1),
+                       idx=g(fmt.idx, int(fmt.nnz)), parent=g(fmt.parent, n), order=g(fmt.order, n),
+                       level_off=g(fmt.level_off, fmt.n_levels + 1))
+        host.cbm_format_free(C.byref(fmt))
+        return rc, out, arrays
+    finally:
+        host.cbm_builder_free(handle)
+
+
+def _all_pairs(ei, n):
+    """(i, j > i, |row_i ^ row_j|) for every pair of rows that share a column, by dense arithmetic."""
+    a = np.zeros((n, n), np.int64)
+    a[ei[0], ei[1]] = 1
+    s = a @ a.T
+    i, j = np.nonzero(np.triu(s, 1))
+    return np.stack([i, j, s[i, j]], 1).astype(np.int32)
+
+
+@pytest.mark.parametrize("alpha", [0, 2, 5])
+def test_staged_build_from_pairs_equals_one_call_build(alpha):
+    n = 90
+    ei = graphs.add_self_loops(graphs.sbm(n, 6, 0.6, 0.05, seed=alpha), n)
+    ref = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha)
+    pairs = _all_pairs(ei, n)
+    rng = np.random.default_rng(alpha)
+    for given in (None, pairs, pairs[rng.permutation(len(pairs))]):      # host intersections / any order of pairs
+        rc, out, arrays = _staged_build(ei, n, alpha, given)
+        assert rc == 0
+        assert out["nnz"] == ref.nnz and out["n_candidates"] == ref.n_candidates
+        assert np.array_equal(out["rowptr"], ref.rowptr.numpy()) and np.array_equal(out["idx"], _u32(ref.idx))
+        assert np.array_equal(out["parent"], ref.parent.numpy()) and np.array_equal(out["order"], ref.order.numpy())
+        assert np.array_equal(out["level_off"], ref.level_off.numpy())
+    # only the admissible pairs are needed
+    nz = arrays["row_nnz"]
+    adm = pairs[2 * pairs[:, 2] > np.minimum(nz[pairs[:, 0]], nz[pairs[:, 1]]) + alpha]
+    rc, out, _ = _staged_build(ei, n, alpha, adm)
+    assert rc == 0 and np.array_equal(out["idx"], _u32(ref.idx)) and np.array_equal(out["parent"], ref.parent.numpy())
+    # the arrays handed to the GPU kernel: after[k] = first position in row_t of a row id > r within column col[k]
+    rp, col, tp, rt, after = (arrays[k] for k in ("rowptr", "col", "colptr_t", "row_t", "after"))
+    for r in range(n):
+        for k in range(rp[r], rp[r + 1]):
+            seg = rt[tp[col[k]]:tp[col[k] + 1]]
+            assert after[k] == tp[col[k]] + np.searchsorted(seg, r, side="right") and seg[after[k] - tp[col[k]] - 1] == r
+
+
+def test_staged_build_rejects_bad_pairs():
+    n = 40
+    ei = graphs.add_self_loops(graphs.erdos_renyi(n, 0.4, 1), n)
+    pairs = _all_pairs(ei, n)
+    assert _staged_build(ei, n, 0, pairs)[0] == 0
+    for bad in ([5, 5, 1], [7, 3, 1], [0, n, 1], [-1, 2, 1], [0, 1, 0], [0, 1, 10_000]):
+        assert _staged_build(ei, n, 0, np.vstack([pairs, [bad]]))[0] == 3, bad
+    assert _staged_build(ei, n, 0, np.vstack([pairs, pairs[:1]]))[0] in (0, 3)     # a duplicate: refused if admissible
+    nz = np.bincount(ei[0], minlength=n)
+    adm = pairs[2 * pairs[:, 2] > np.minimum(nz[pairs[:, 0]], nz[pairs[:, 1]])]
+    if len(adm):
+        assert _staged_build(ei, n, 0, np.vstack([pairs, adm[:1]]))[0] == 3
+    host = _lib.host_lib()
+    assert host.cbm_builder_finish(None, 0, None, -1, C.byref(_lib.CbmFormat())) == 1
+    assert host.cbm_builder_create(None, None, 5, 4, 1, C.byref(C.c_void_p())) == 1

@@ -476,3 +476,25 @@ def test_launch_size_does_not_change_results(orc):
         assert lib.cbm_set_spmm_occupancy(0) == 0
     ref = oracle_product(orc, mat, ei, n, x.cpu().numpy(), True)
     assert np.array_equal(want.cpu().numpy(), ref)
+
+
+def test_gpu_row_intersections_build_the_same_format(monkeypatch):
+    """builder="gpu": cbm_row_intersections + cbm_builder_finish give exactly the arrays of the
+    all-host build, also when the first pair buffer is too small and a second pass is needed."""
+    from cbm4gnn_amd import cbm as cbm_mod
+    cases = [(graphs.add_self_loops(graphs.sbm(600, 6, 0.5, 0.02, seed=1), 600), 0),
+             (graphs.add_self_loops(graphs.erdos_renyi(300, 0.3, 2), 300), 3),
+             (graphs.workload("c2", scale=0.25).edge_index, 0),
+             (graphs.workload("c1").edge_index, 0),
+             (np.array([[0, 1, 2], [0, 1, 2]], np.int32), 0)]                       # self loops only: no pair at all
+    for tiny_buffer in (False, True):
+        if tiny_buffer:                                     # 8 pairs of room: the second, exactly sized pass runs
+            monkeypatch.setattr(cbm_mod, "_first_pair_capacity", lambda nnz: 8)
+        for k, (ei, alpha) in enumerate(cases):
+            say("gpu builder case", k, "tiny buffer", tiny_buffer)
+            a = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha)
+            b = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, builder="gpu")
+            assert a.n_candidates == b.n_candidates and a.nnz == b.nnz
+            for name in ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col"):
+                assert torch.equal(getattr(a, name), getattr(b, name)), (k, name)
+            assert "gpu_intersections" in b.build_seconds
