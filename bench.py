@@ -265,7 +265,7 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--builder", choices=("host", "gpu"), default="host",
+    ap.add_argument("--builder", choices=("auto", "host", "gpu"), default="auto",
                     help="where the format builder computes its row intersections (same format either way)")
     ap.add_argument("--probe", action="store_true",
                     help="counter run: 3 multiplies and 3 plain device copies of X (known size, for scaling "
@@ -374,7 +374,7 @@ def main():
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, alpha, d)) if args.scale == 1.0 else None,
                      "algorithmic_bytes": b_spmm, "avg_launch_ms": spmm_ms},
-        "host_s": {"generate": t_gen, "build_format": t_build, "builder": args.builder, "build_phases": mat.build_seconds},
+        "host_s": {"generate": t_gen, "build_format": t_build, "builder": mat.builder, "build_phases": mat.build_seconds},
     }
     if not args.no_cpu:
         cpu, y_cpu = cpu_baseline(w, mat, x.numpy())

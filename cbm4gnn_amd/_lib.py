@@ -61,8 +61,8 @@ HIP_SYMBOLS = {
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "csr_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
-    "cbm_row_intersections_groups": (C.c_int, [_I32]),
-    "cbm_row_intersections": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _P, _I32, _P, _P, _I64, _P, _P]),
+    "cbm_row_intersections_groups": (C.c_int, []),
+    "cbm_row_intersections": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _P, _I64, _P, _P]),
 }
 
 _host = None

@@ -149,6 +149,9 @@ def tree_levels(mst_row: np.ndarray, mst_col: np.ndarray):
     return parent.astype(np.int32), order.astype(np.int32), level_off.astype(np.int32)
 
 
+_GPU_BUILDER_MIN_EDGES = 2_000_000     # builder="auto": below this the host intersections are as fast as upload + kernel + download
+
+
 def _first_pair_capacity(nnz):
     """Room for admissible pairs in the first pass of the GPU row intersections (12 B each); they
     rarely outnumber the entries of the matrix, and a second, exactly sized pass runs if they do."""
@@ -185,8 +188,8 @@ def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
         row_t = up(ptrs[3], nnz.value, C.c_int32, np.int32)
         after = up(ptrs[4], nnz.value, C.c_int64, np.int64)
         row_nnz = up(ptrs[5], n, C.c_int32, np.int32)
-        groups = int(hip.cbm_row_intersections_groups(n))
-        counters = torch.zeros(groups * n, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            groups = int(hip.cbm_row_intersections_groups())
         capacity = _first_pair_capacity(nnz.value)
         while True:
             ticket = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -194,7 +197,7 @@ def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
             pairs = torch.empty((capacity, 3), dtype=torch.int32, device=dev)
             with torch.cuda.device(dev):
                 rc = hip.cbm_row_intersections(_ptr(rowptr), _ptr(col), _ptr(colptr_t), _ptr(row_t), _ptr(after),
-                                               _ptr(row_nnz), n, alpha, _ptr(counters), groups, _ptr(ticket), _ptr(pairs),
+                                               _ptr(row_nnz), n, alpha, groups, _ptr(ticket), _ptr(pairs),
                                                capacity, _ptr(count), _stream(dev))
             if rc:
                 return rc, 0.0
@@ -214,7 +217,7 @@ def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
 class cbm_matrix:
 
     def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
-                 deltas_format="csr", threads=0, builder="host"):
+                 deltas_format="csr", threads=0, builder="auto"):
         ei = torch.as_tensor(edge_index)
         if ei.dim() != 2 or ei.size(0) != 2:
             raise ValueError("Edge index should have shape (2, num_edges)")
@@ -233,9 +236,13 @@ class cbm_matrix:
         self.deltas_format = deltas_format if deltas_format in ("csr", "coo") else "csr"
 
         # builder: "host" = everything on the CPU; "gpu" = the row intersections (the dominant cost
-        # for large graphs) on the GPU, the rest on the CPU.  Both give the same format.
-        if builder not in ("host", "gpu"):
-            raise ValueError('builder must be "host" or "gpu"')
+        # for large graphs) on the GPU, the rest on the CPU; "auto" = "gpu" when a HIP device is
+        # there and the matrix is large enough to repay the transfers.  All give the same format.
+        if builder not in ("auto", "host", "gpu"):
+            raise ValueError('builder must be "auto", "host" or "gpu"')
+        if builder == "auto":
+            builder = "gpu" if (torch.cuda.is_available() and ei_cpu.size(1) >= _GPU_BUILDER_MIN_EDGES) else "host"
+        self.builder = builder
         fmt = _lib.CbmFormat()
         if builder == "gpu":
             rc, t_pairs = _build_with_gpu_intersections(ei_cpu, n, self.alpha, int(threads), fmt)
@@ -324,6 +331,7 @@ class cbm_matrix:
         if not ok:
             raise ValueError(f"{path} does not hold a consistent CBM format")
         self.build_seconds = None
+        self.builder = None                                 # loaded, not built
         self._deltas, self._dev, self._transposed = None, {}, None
         self.stream_coefficients = True
         self.relayout = True

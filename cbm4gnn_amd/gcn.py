@@ -23,7 +23,7 @@ from .cbm import CBMMatmul, cbm_matrix, csr_spmm, schedule_rows
 __all__ = ["CBMGCNLayer", "CSRGCNLayer", "TwoLayerGCN", "build_operator", "csr_operator", "CSRMatmul"]
 
 
-def build_operator(edge_index, alpha: int = 2, normalized: bool = True, builder: str = "host") -> cbm_matrix:
+def build_operator(edge_index, alpha: int = 2, normalized: bool = True, builder: str = "auto") -> cbm_matrix:
     """``cbm_matrix`` of the TRANSPOSED edge list, as the reference's layers build it
     (``cbm_message_passing.py:48-49``; default alpha = 2, ``:8``)."""
     ei = torch.as_tensor(edge_index)

@@ -220,15 +220,15 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int6
  * s = |row_i ^ row_j| and 2 s > min(nnz_i, nnz_j) + alpha, in no particular order, and adds their
  * number to *n_pairs (which may exceed capacity: then only the first `capacity` were stored and the
  * call must be repeated with a larger buffer).  The six input arrays are device copies of
- * cbm_builder_arrays(); counters = groups * n uint32 and ticket = 1 uint32 and n_pairs = 1 uint64,
- * all zero on entry (the counters are zero again on exit); groups = number of workgroups, e.g.
- * cbm_row_intersections_groups(n).  Feed the result to cbm_builder_finish.
+ * cbm_builder_arrays(); ticket = 1 uint32 and n_pairs = 1 uint64, both zero on entry; groups =
+ * number of workgroups, e.g. cbm_row_intersections_groups() (one per CU).  No scratch memory:
+ * the counters live in LDS.  Feed the result to cbm_builder_finish.
  * Replaces mkl_sparse_syrk + the admission scan of cbm_init_v1_/_v2_ (cbm_extensions.cpp:46-103). */
-int cbm_row_intersections_groups(int32_t n);
+int cbm_row_intersections_groups(void);
 int cbm_row_intersections(const int64_t* rowptr_dev, const int32_t* col_dev, const int64_t* colptr_t_dev,
                           const int32_t* row_t_dev, const int64_t* after_dev, const int32_t* row_nnz_dev, int32_t n,
-                          int32_t alpha, uint32_t* counters_dev, int32_t groups, uint32_t* ticket_dev,
-                          struct cbm_pair* pairs_dev, int64_t capacity, unsigned long long* n_pairs_dev, void* stream);
+                          int32_t alpha, int32_t groups, uint32_t* ticket_dev, struct cbm_pair* pairs_dev,
+                          int64_t capacity, unsigned long long* n_pairs_dev, void* stream);
 
 /* Plain CSR SpMM  Y = A * X  (val == NULL means all ones): the hand-written GPU baseline.
  * Replaces seq_/omp_s_spmm_csr_int32_ (cbm_extensions.cpp:790-843, :1707-1755). */
