@@ -257,22 +257,61 @@ struct Graph {
     std::vector<int64_t> after;          // per entry k = (r, c) of A: first position in tr of a row id > r inside column c
 };
 
+// Stable parallel bucketing (a counting sort): item t of `count` goes to bucket key(t) in
+// [0, n_buckets); offsets[] (n_buckets + 1) is computed, place(t, position) stores the item.
+// Items keep their order inside a bucket: the threads take consecutive chunks of the items and
+// count their chunk per bucket; a prefix over (bucket, chunk) gives every chunk its own range.
+// One chunk when threads x buckets counters would be too many or the input is small.
+template <class Key, class Place>
+void bucket_stable(int64_t count, int32_t n_buckets, std::vector<int64_t>& offsets, int threads, Key key, Place place) {
+    int chunks = threads;
+    if ((int64_t)chunks * n_buckets > ((int64_t)1 << 28) || count < (int64_t)1 << 16) chunks = 1;
+    std::vector<int64_t> start((size_t)chunks * n_buckets);
+    const int64_t per = (count + chunks - 1) / chunks;
+#pragma omp parallel for schedule(static, 1) num_threads(chunks)
+    for (int c = 0; c < chunks; c++) {
+        int64_t* mine = start.data() + (size_t)c * n_buckets;
+        std::fill(mine, mine + n_buckets, 0);
+        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
+        for (int64_t t = lo; t < hi; t++) mine[key(t)]++;
+    }
+    offsets.assign((size_t)n_buckets + 1, 0);
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (int32_t b = 0; b < n_buckets; b++) {
+        int64_t size = 0;
+        for (int c = 0; c < chunks; c++) size += start[(size_t)c * n_buckets + b];
+        offsets[b + 1] = size;
+    }
+    for (int32_t b = 0; b < n_buckets; b++) offsets[b + 1] += offsets[b];
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (int32_t b = 0; b < n_buckets; b++) {
+        int64_t at = offsets[b];
+        for (int c = 0; c < chunks; c++) {
+            int64_t& slot = start[(size_t)c * n_buckets + b];
+            const int64_t size = slot;
+            slot = at;
+            at += size;
+        }
+    }
+#pragma omp parallel for schedule(static, 1) num_threads(chunks)
+    for (int c = 0; c < chunks; c++) {
+        int64_t* mine = start.data() + (size_t)c * n_buckets;
+        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
+        for (int64_t t = lo; t < hi; t++) place(t, mine[key(t)]++);
+    }
+}
+
 // COO -> CSR(A) with sorted unique columns, and its transpose.
 int build_graph(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int threads, Graph& g) {
     g.N = N;
     std::vector<int64_t>& rp = g.rp; std::vector<int32_t>& ci = g.ci; std::vector<int32_t>& nnz = g.nnz;
     std::vector<int64_t>& tp = g.tp; std::vector<int32_t>& tr = g.tr;
-    rp.assign(N + 1, 0);
-    for (int64_t k = 0; k < E; k++) {
-        if (row[k] < 0 || row[k] >= N || col[k] < 0 || col[k] >= N) return CBM_ERR_SHAPE;
-        rp[row[k] + 1]++;
-    }
-    for (int32_t r = 0; r < N; r++) rp[r + 1] += rp[r];
+    bool bad = false;
+#pragma omp parallel for schedule(static) num_threads(threads) reduction(|| : bad)
+    for (int64_t k = 0; k < E; k++) bad = bad || row[k] < 0 || row[k] >= N || col[k] < 0 || col[k] >= N;
+    if (bad) return CBM_ERR_SHAPE;
     ci.resize(E);
-    {
-        std::vector<int64_t> fill(rp.begin(), rp.end() - 1);
-        for (int64_t k = 0; k < E; k++) ci[fill[row[k]]++] = col[k];
-    }
+    bucket_stable(E, N, rp, threads, [&](int64_t k) { return row[k]; }, [&](int64_t k, int64_t at) { ci[at] = col[k]; });
     nnz.resize(N);
 #pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
     for (int32_t r = 0; r < N; r++) {
@@ -292,19 +331,16 @@ int build_graph(const int32_t* row, const int32_t* col, int64_t E, int32_t N, in
         ci.resize(w);
     }
     g.nnzA = rp[N];
-    tp.assign(N + 1, 0);
-    for (int64_t k = 0; k < g.nnzA; k++) tp[ci[k] + 1]++;
-    for (int32_t c = 0; c < N; c++) tp[c + 1] += tp[c];
+    // transpose: entry k = (r, c) goes to column c; entries arrive in ascending r, so every column
+    // of A^T lists its rows in ascending order and after[k] is the position behind the entry
+    std::vector<int32_t> row_of(g.nnzA);
+#pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
+    for (int32_t r = 0; r < N; r++)
+        for (int64_t k = rp[r]; k < rp[r + 1]; k++) row_of[k] = r;
     tr.resize(g.nnzA);
     g.after.resize(g.nnzA);
-    {
-        std::vector<int64_t> fill(tp.begin(), tp.end() - 1);
-        for (int32_t r = 0; r < N; r++)
-            for (int64_t k = rp[r]; k < rp[r + 1]; k++) {
-                tr[fill[ci[k]]] = r;                               // ascending r per column
-                g.after[k] = ++fill[ci[k]];
-            }
-    }
+    bucket_stable(g.nnzA, N, tp, threads, [&](int64_t k) { return ci[k]; },
+                  [&](int64_t k, int64_t at) { tr[at] = row_of[k]; g.after[k] = at + 1; });
     // symmetric pattern <=> CSR(A) == CSR(A^T) (both have ascending columns)
     g.symmetric = rp == tp && ci == tr;
     return CBM_OK;
