@@ -498,3 +498,46 @@ def test_gpu_row_intersections_build_the_same_format(monkeypatch):
             for name in ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col"):
                 assert torch.equal(getattr(a, name), getattr(b, name)), (k, name)
             assert "gpu_intersections" in b.build_seconds
+
+
+def test_reference_message_passing_call_pattern():
+    """The way the reference's layers drive the matrix (gnns/message_passing/cbm_message_passing.py:16-60,
+    tests/test_message_passing.py:53-98 restated with seeds): cbm_matrix of the TRANSPOSED int32 edge
+    list with unit values, alpha = 2, built once; one cached output buffer on x's device, overwritten
+    by every call; the result is the scatter-add of source features into target rows."""
+    for seed in range(3):
+        ei = torch.from_numpy(graphs.erdos_renyi(25, 0.75, seed)).long()
+        x = torch.randint(0, 10, (25, 10), generator=torch.Generator().manual_seed(seed)).float().cuda()
+        native = torch.zeros(25, 10, device="cuda").index_add_(0, ei[1].cuda(), x[ei[0].cuda()])   # out[target] += x[source]
+        ei_t = torch.stack([ei[1], ei[0]], dim=0).to(torch.int32)
+        say("message passing pattern", seed)
+        a_t = cbm_matrix(ei_t, torch.ones(ei.size(1), dtype=x.dtype), normalized=False, alpha=2)
+        out = torch.empty((int(ei.max()) + 1, x.size(1)), dtype=x.dtype, device=x.device)
+        for call in (a_t.seq_mkl_csr_spmm_update, a_t.omp_mkl_csr_spmm_update):
+            out.fill_(float("nan"))
+            assert call(x, out) is None
+            torch.testing.assert_close(out, native, atol=1e-4, rtol=1e-4)
+            assert torch.equal(out, native)                  # integer features: exact
+        # two hops through the same cached buffer, as stacked layers of equal width do
+        a_t.omp_mkl_csr_spmm_update(x, out)
+        hop2 = torch.empty_like(out)
+        a_t.omp_mkl_csr_spmm_update(out, hop2)
+        want2 = torch.zeros(25, 10, device="cuda").index_add_(0, ei[1].cuda(), native[ei[0].cuda()])
+        assert torch.equal(hop2, want2)
+        # matmul-returning variants (CBM*TorchCSR* layers)
+        torch.testing.assert_close(a_t.seq_torch_csr_matmul(x), native, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(a_t.omp_torch_csr_matmul(x), native, atol=1e-4, rtol=1e-4)
+        # normalised flavour: GCN weights deg^-1/2[target] * deg^-1/2[source] on the self-looped graph
+        # (gnns/utility.py:25-43), fused into the matrix by normalized=True
+        n = 25
+        loops = torch.arange(n).repeat(2, 1)
+        ei_l = torch.cat([ei[:, ei[0] != ei[1]], loops], dim=1)
+        deg = torch.zeros(n).index_add_(0, ei_l[1], torch.ones(ei_l.size(1)))
+        w = (deg.pow(-0.5)[ei_l[0]] * deg.pow(-0.5)[ei_l[1]]).cuda()
+        native_n = torch.zeros(n, 10, device="cuda").index_add_(0, ei_l[1].cuda(), x[ei_l[0].cuda()] * w[:, None])
+        a_n = cbm_matrix(torch.stack([ei_l[1], ei_l[0]]).to(torch.int32), torch.ones(ei_l.size(1)), normalized=True, alpha=2)
+        out_n = torch.empty_like(out)
+        for call in (a_n.seq_mkl_csr_fused_spmm_update, a_n.omp_mkl_csr_fused_spmm_update):
+            out_n.fill_(float("nan"))
+            call(x, out_n)
+            torch.testing.assert_close(out_n, native_n, atol=1e-4, rtol=1e-4)
