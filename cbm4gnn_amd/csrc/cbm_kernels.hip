@@ -473,7 +473,7 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_narrow_levels(
 // fetched kChainDepth levels ahead.  The 64 row ids (and their m) of a stretch come in with one
 // coalesced load and are broadcast with v_readlane.  Arithmetic per level is exactly that of
 // propagate_row.
-constexpr int kChainDepth = 32;
+constexpr int kChainDepth = 64;
 constexpr int kMinChain = 4;               // shorter runs of single-row levels stay with the other kernels
 
 template <bool NORM>
