@@ -352,6 +352,18 @@ def test_c_abi_status_codes_on_device_calls():
     assert lib.cbm_spmm_update_f32(p(rp), p(idx), 0, None, None, p(par), None, p(order), p(rp), lo, 1, p(x), p(x), None, n, d, d, d, 0, None) == 3
     torch.cuda.synchronize()
     assert (y == 0).all()
+    # row intersections: (rowptr, col, colptr_t, row_t, after, row_nnz, n, alpha, groups, ticket, pairs, capacity, n_pairs, stream)
+    i64 = torch.zeros(n + 1, dtype=torch.int64, device="cuda"); i32 = torch.zeros(n, dtype=torch.int32, device="cuda")
+    tick = torch.zeros(1, dtype=torch.int32, device="cuda"); cnt = torch.zeros(1, dtype=torch.int64, device="cuda")
+    ri = lambda *a: lib.cbm_row_intersections(*a)
+    assert lib.cbm_row_intersections_groups() >= 8
+    assert ri(None, p(i32), p(i64), p(i32), p(i64), p(i32), n, 0, 8, p(tick), None, 0, p(cnt), None) == 1
+    assert ri(p(i64), p(i32), p(i64), p(i32), p(i64), p(i32), n, 0, 0, p(tick), None, 0, p(cnt), None) == 3      # no workgroups
+    assert ri(p(i64), p(i32), p(i64), p(i32), p(i64), p(i32), n, 0, 8, p(tick), None, 4, p(cnt), None) == 1      # room but no buffer
+    assert ri(p(i64), p(i32), p(i64), p(i32), p(i64), p(i32), 0, 0, 8, p(tick), None, 0, p(cnt), None) == 0      # nothing to do
+    assert ri(p(i64), p(i32), p(i64), p(i32), p(i64), p(i32), n, 0, 8, p(tick), None, 0, p(cnt), None) == 0      # n empty rows: no pair
+    torch.cuda.synchronize()
+    assert int(cnt) == 0 and int(tick) >= n
 
 
 def test_two_layer_gcn_forward_backward_matches_dense(orc):
