@@ -36,6 +36,50 @@ namespace {
 
 struct CandEdge { int32_t u, v, w; };
 
+// Stable parallel bucketing (a counting sort): item t of `count` goes to bucket key(t) in
+// [0, n_buckets); offsets[] (n_buckets + 1) is computed, place(t, position) stores the item.
+// Items keep their order inside a bucket: the threads take consecutive chunks of the items and
+// count their chunk per bucket; a prefix over (bucket, chunk) gives every chunk its own range.
+// One chunk when threads x buckets counters would be too many or the input is small.
+template <class Key, class Place>
+void bucket_stable(int64_t count, int32_t n_buckets, std::vector<int64_t>& offsets, int threads, Key key, Place place) {
+    int chunks = threads;
+    if ((int64_t)chunks * n_buckets > ((int64_t)1 << 28) || count < (int64_t)1 << 16) chunks = 1;
+    std::vector<int64_t> start((size_t)chunks * n_buckets);
+    const int64_t per = (count + chunks - 1) / chunks;
+#pragma omp parallel for schedule(static, 1) num_threads(chunks)
+    for (int c = 0; c < chunks; c++) {
+        int64_t* mine = start.data() + (size_t)c * n_buckets;
+        std::fill(mine, mine + n_buckets, 0);
+        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
+        for (int64_t t = lo; t < hi; t++) mine[key(t)]++;
+    }
+    offsets.assign((size_t)n_buckets + 1, 0);
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (int32_t b = 0; b < n_buckets; b++) {
+        int64_t size = 0;
+        for (int c = 0; c < chunks; c++) size += start[(size_t)c * n_buckets + b];
+        offsets[b + 1] = size;
+    }
+    for (int32_t b = 0; b < n_buckets; b++) offsets[b + 1] += offsets[b];
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (int32_t b = 0; b < n_buckets; b++) {
+        int64_t at = offsets[b];
+        for (int c = 0; c < chunks; c++) {
+            int64_t& slot = start[(size_t)c * n_buckets + b];
+            const int64_t size = slot;
+            slot = at;
+            at += size;
+        }
+    }
+#pragma omp parallel for schedule(static, 1) num_threads(chunks)
+    for (int c = 0; c < chunks; c++) {
+        int64_t* mine = start.data() + (size_t)c * n_buckets;
+        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
+        for (int64_t t = lo; t < hi; t++) place(t, mine[key(t)]++);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Minimum spanning arborescence (Tarjan 1977 / Camerini-Fratta-Maffioli 1979 expansion).
 //
@@ -58,14 +102,9 @@ public:
         const int64_t m = (int64_t)edges_.size();
         // runs: edges grouped by head, each group sorted by (weight, id); weight and tail are
         // copied next to the id so that walking a run never touches edges_
-        run_beg_.assign(n_ + 1, 0);
-        for (int64_t e = 0; e < m; e++) run_beg_[edges_[e].v + 1]++;
-        for (int32_t v = 0; v < n_; v++) run_beg_[v + 1] += run_beg_[v];
         run_id_.resize(m); run_w_.resize(m); run_tail_.resize(m);
-        {
-            std::vector<int64_t> fill(run_beg_.begin(), run_beg_.end() - 1);
-            for (int64_t e = 0; e < m; e++) run_id_[fill[edges_[e].v]++] = (int32_t)e;
-        }
+        bucket_stable(m, n_, run_beg_, threads_, [&](int64_t e) { return edges_[e].v; },
+                      [&](int64_t e, int64_t at) { run_id_[at] = (int32_t)e; });
 #pragma omp parallel for schedule(dynamic, 64) num_threads(threads_)
         for (int32_t v = 0; v < n_; v++) {
             const int64_t b = run_beg_[v], e = run_beg_[v + 1];
@@ -257,50 +296,6 @@ struct Graph {
     std::vector<int64_t> after;          // per entry k = (r, c) of A: first position in tr of a row id > r inside column c
 };
 
-// Stable parallel bucketing (a counting sort): item t of `count` goes to bucket key(t) in
-// [0, n_buckets); offsets[] (n_buckets + 1) is computed, place(t, position) stores the item.
-// Items keep their order inside a bucket: the threads take consecutive chunks of the items and
-// count their chunk per bucket; a prefix over (bucket, chunk) gives every chunk its own range.
-// One chunk when threads x buckets counters would be too many or the input is small.
-template <class Key, class Place>
-void bucket_stable(int64_t count, int32_t n_buckets, std::vector<int64_t>& offsets, int threads, Key key, Place place) {
-    int chunks = threads;
-    if ((int64_t)chunks * n_buckets > ((int64_t)1 << 28) || count < (int64_t)1 << 16) chunks = 1;
-    std::vector<int64_t> start((size_t)chunks * n_buckets);
-    const int64_t per = (count + chunks - 1) / chunks;
-#pragma omp parallel for schedule(static, 1) num_threads(chunks)
-    for (int c = 0; c < chunks; c++) {
-        int64_t* mine = start.data() + (size_t)c * n_buckets;
-        std::fill(mine, mine + n_buckets, 0);
-        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
-        for (int64_t t = lo; t < hi; t++) mine[key(t)]++;
-    }
-    offsets.assign((size_t)n_buckets + 1, 0);
-#pragma omp parallel for schedule(static) num_threads(threads)
-    for (int32_t b = 0; b < n_buckets; b++) {
-        int64_t size = 0;
-        for (int c = 0; c < chunks; c++) size += start[(size_t)c * n_buckets + b];
-        offsets[b + 1] = size;
-    }
-    for (int32_t b = 0; b < n_buckets; b++) offsets[b + 1] += offsets[b];
-#pragma omp parallel for schedule(static) num_threads(threads)
-    for (int32_t b = 0; b < n_buckets; b++) {
-        int64_t at = offsets[b];
-        for (int c = 0; c < chunks; c++) {
-            int64_t& slot = start[(size_t)c * n_buckets + b];
-            const int64_t size = slot;
-            slot = at;
-            at += size;
-        }
-    }
-#pragma omp parallel for schedule(static, 1) num_threads(chunks)
-    for (int c = 0; c < chunks; c++) {
-        int64_t* mine = start.data() + (size_t)c * n_buckets;
-        const int64_t lo = std::min(count, c * per), hi = std::min(count, lo + per);
-        for (int64_t t = lo; t < hi; t++) place(t, mine[key(t)]++);
-    }
-}
-
 // COO -> CSR(A) with sorted unique columns, and its transpose.
 int build_graph(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int threads, Graph& g) {
     g.N = N;
@@ -419,18 +414,17 @@ int candidates_host(const Graph& g, int32_t alpha, int threads, std::vector<Cand
 int candidates_from_pairs(const Graph& g, int32_t alpha, const cbm_pair* pairs, int64_t n_pairs, int threads,
                           std::vector<CandEdge>& cand) {
     const int32_t N = g.N;
-    std::vector<int64_t> first(N + 1, 0);
+    bool bad = false;
+#pragma omp parallel for schedule(static) num_threads(threads) reduction(|| : bad)
     for (int64_t p = 0; p < n_pairs; p++) {
         const cbm_pair& q = pairs[p];
-        if (q.i < 0 || q.j <= q.i || q.j >= N || q.s <= 0 || q.s > std::min(g.nnz[q.i], g.nnz[q.j])) return CBM_ERR_SHAPE;
-        first[q.i + 1]++;
+        bad = bad || q.i < 0 || q.j <= q.i || q.j >= N || q.s <= 0 || q.s > std::min(g.nnz[q.i], g.nnz[q.j]);
     }
-    for (int32_t i = 0; i < N; i++) first[i + 1] += first[i];
+    if (bad) return CBM_ERR_SHAPE;
+    std::vector<int64_t> first;
     std::vector<std::pair<int32_t, int32_t>> by_row(n_pairs);
-    {
-        std::vector<int64_t> fill(first.begin(), first.end() - 1);
-        for (int64_t p = 0; p < n_pairs; p++) by_row[fill[pairs[p].i]++] = {pairs[p].j, pairs[p].s};
-    }
+    bucket_stable(n_pairs, N, first, threads, [&](int64_t p) { return pairs[p].i; },
+                  [&](int64_t p, int64_t at) { by_row[at] = {pairs[p].j, pairs[p].s}; });
     const int32_t CH = 64;
     const int32_t n_chunks = (N + CH - 1) / CH;
     std::vector<std::vector<CandEdge>> chunk_out(n_chunks);
