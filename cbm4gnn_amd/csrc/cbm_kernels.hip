@@ -579,17 +579,37 @@ int g_spmm_kernel = 0;
 // One workgroup (16 wavefronts) per CU keeps `tile` 32-bit counters in LDS and takes rows from a
 // shared ticket.  The candidate rows j are cut into tiles of `tile` consecutive ids; for every
 // tile that can hold a j > i the workgroup walks, for every column c of row i, the rows j > i of
-// that column (one wavefront per column, lanes along the column: coalesced, lists re-read from L2
-// once per tile) twice with a barrier in between:
+// that column (one wavefront per column, lanes along the column: coalesced; only the part of
+// the sorted list that can hold ids of the tile, found by sampling the list with the 64 lanes)
+// twice with a barrier in between:
 //   1. increment counter j - tile start (LDS atomic);
 //   2. swap the counter with 0 -- exactly one thread per distinct j gets the count, decides
 //      admission and appends (i, j, s); the counters are clean for the next tile.
 // Only the ticket and the output cursor are device-scope atomics.  Measured on 132 534 rows x
-// 620 entries (25 G increments): 0.24 s; the same walks with the counters in device memory
-// (workgroup-scope atomics executed by the L2) took 0.61-0.78 s; 16 host threads take 3.4 s.
+// 620 entries (25 G increments): 0.19 s (0.24 s when every tile re-read the whole lists); the
+// same walks with the counters in device memory (workgroup-scope atomics executed by the L2)
+// took 0.61-0.78 s; 16 host threads take 3.4 s.  What is left is the chain of dependent loads
+// per (column, tile): column id -> list bounds -> samples -> list part.
 // ---------------------------------------------------------------------------------------------
 constexpr int kIsectWaves = 16;
-constexpr int kIsectUnroll = 4;
+constexpr int kIsectUnroll = 2;
+
+// Part [beg, fin) of an ascending list of `len` row ids that can hold ids of the tile
+// [lo_j, lo_j + tile): the 64 lanes sample the list at equal steps and two ballots bracket the
+// tile's first and last element to within one step (ids outside the tile that fall into the
+// bracket are filtered by the caller).  Wave-uniform result.
+__device__ __forceinline__ void tile_range(const int32_t* __restrict__ lst, int len, int lo_j, int tile, int lane,
+                                           int& beg, int& fin) {
+    beg = 0; fin = 0;
+    if (len <= 0) return;
+    const int step = (len + kWave - 1) / kWave;
+    const int at = lane * step;
+    const int id = lst[min(at, len - 1)];
+    const int below = __popcll(__ballot(at < len && id < lo_j));           // samples before the tile
+    const int upto = __popcll(__ballot(at < len && id - lo_j < tile));      // samples before the tile's end
+    beg = max(below - 1, 0) * step;
+    fin = min(upto * step, len);
+}
 
 __global__ __launch_bounds__(kWave * kIsectWaves) void row_intersections(
     const int64_t* __restrict__ rowptr, const int32_t* __restrict__ col, const int64_t* __restrict__ colptr_t,
@@ -612,28 +632,32 @@ __global__ __launch_bounds__(kWave * kIsectWaves) void row_intersections(
         for (int lo_j = ((i + 1) / tile) * tile; lo_j < n; lo_j += tile) {
             if (lo_j != ((i + 1) / tile) * tile) __syncthreads();          // previous tile's swaps are done
             for (int64_t k = b + wave; k < e; k += kIsectWaves) {
-                const int64_t hi = colptr_t[col[k] + 1];
-                for (int64_t t0 = after[k]; t0 < hi; t0 += kWave * kIsectUnroll) {
+                const int32_t* __restrict__ lst = row_t + after[k];
+                int beg, fin;
+                tile_range(lst, (int)(colptr_t[col[k] + 1] - after[k]), lo_j, tile, lane, beg, fin);
+                for (int t0 = beg; t0 < fin; t0 += kWave * kIsectUnroll) {
                     int j[kIsectUnroll];
 #pragma unroll
-                    for (int u = 0; u < kIsectUnroll; u++) j[u] = row_t[min(t0 + u * kWave + lane, hi - 1)];
+                    for (int u = 0; u < kIsectUnroll; u++) j[u] = lst[min(t0 + u * kWave + lane, fin - 1)];
 #pragma unroll
                     for (int u = 0; u < kIsectUnroll; u++)
-                        if (t0 + u * kWave + lane < hi && (unsigned)(j[u] - lo_j) < (unsigned)tile)
+                        if (t0 + u * kWave + lane < fin && (unsigned)(j[u] - lo_j) < (unsigned)tile)
                             atomicAdd(&lds_cnt[j[u] - lo_j], 1u);
                 }
             }
             __syncthreads();
             for (int64_t k = b + wave; k < e; k += kIsectWaves) {
-                const int64_t hi = colptr_t[col[k] + 1];
-                for (int64_t t0 = after[k]; t0 < hi; t0 += kWave * kIsectUnroll) {   // whole wavefront iterates together (ballot below)
+                const int32_t* __restrict__ lst = row_t + after[k];
+                int beg, fin;
+                tile_range(lst, (int)(colptr_t[col[k] + 1] - after[k]), lo_j, tile, lane, beg, fin);
+                for (int t0 = beg; t0 < fin; t0 += kWave * kIsectUnroll) {   // whole wavefront iterates together (ballot below)
                     int j[kIsectUnroll];
 #pragma unroll
-                    for (int u = 0; u < kIsectUnroll; u++) j[u] = row_t[min(t0 + u * kWave + lane, hi - 1)];
+                    for (int u = 0; u < kIsectUnroll; u++) j[u] = lst[min(t0 + u * kWave + lane, fin - 1)];
 #pragma unroll
                     for (int u = 0; u < kIsectUnroll; u++) {
                         int sh = 0;
-                        if (t0 + u * kWave + lane < hi && (unsigned)(j[u] - lo_j) < (unsigned)tile)
+                        if (t0 + u * kWave + lane < fin && (unsigned)(j[u] - lo_j) < (unsigned)tile)
                             sh = (int)atomicExch(&lds_cnt[j[u] - lo_j], 0u);
                         // 2 s > min(n_i, n_j) + alpha; n_j is only fetched where n_i alone does not decide
                         bool keep = sh > 0;
