@@ -631,10 +631,15 @@ __global__ __launch_bounds__(kWave * kIsectWaves) void row_intersections(
         const int ni = row_nnz[i];
         for (int lo_j = ((i + 1) / tile) * tile; lo_j < n; lo_j += tile) {
             if (lo_j != ((i + 1) / tile) * tile) __syncthreads();          // previous tile's swaps are done
+            // the bounds of the wave's next list are fetched while the current one is walked
+            int64_t nx_a = 0, nx_hi = 0;
+            if (b + wave < e) { nx_a = after[b + wave]; nx_hi = colptr_t[col[b + wave] + 1]; }
             for (int64_t k = b + wave; k < e; k += kIsectWaves) {
-                const int32_t* __restrict__ lst = row_t + after[k];
+                const int32_t* __restrict__ lst = row_t + nx_a;
+                const int len = (int)(nx_hi - nx_a);
+                if (k + kIsectWaves < e) { nx_a = after[k + kIsectWaves]; nx_hi = colptr_t[col[k + kIsectWaves] + 1]; }
                 int beg, fin;
-                tile_range(lst, (int)(colptr_t[col[k] + 1] - after[k]), lo_j, tile, lane, beg, fin);
+                tile_range(lst, len, lo_j, tile, lane, beg, fin);
                 for (int t0 = beg; t0 < fin; t0 += kWave * kIsectUnroll) {
                     int j[kIsectUnroll];
 #pragma unroll
@@ -646,10 +651,13 @@ __global__ __launch_bounds__(kWave * kIsectWaves) void row_intersections(
                 }
             }
             __syncthreads();
+            if (b + wave < e) { nx_a = after[b + wave]; nx_hi = colptr_t[col[b + wave] + 1]; }
             for (int64_t k = b + wave; k < e; k += kIsectWaves) {
-                const int32_t* __restrict__ lst = row_t + after[k];
+                const int32_t* __restrict__ lst = row_t + nx_a;
+                const int len = (int)(nx_hi - nx_a);
+                if (k + kIsectWaves < e) { nx_a = after[k + kIsectWaves]; nx_hi = colptr_t[col[k + kIsectWaves] + 1]; }
                 int beg, fin;
-                tile_range(lst, (int)(colptr_t[col[k] + 1] - after[k]), lo_j, tile, lane, beg, fin);
+                tile_range(lst, len, lo_j, tile, lane, beg, fin);
                 for (int t0 = beg; t0 < fin; t0 += kWave * kIsectUnroll) {   // whole wavefront iterates together (ballot below)
                     int j[kIsectUnroll];
 #pragma unroll
