@@ -152,8 +152,11 @@ int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X
 
 /* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 use for this shape when
  * given one: the size of the slab-major copy of X (n rows x 128-byte slabs, the slab count
- * rounded up for odd widths).  The workspace stays optional: without it, widths that are a
- * multiple of 32 gather from the row-major X and all others take one wavefront per row. */
+ * rounded up for odd widths), or 0 where the copy would buy nothing: d = 32, 64, 128 or 256 with
+ * 128-byte-aligned rows whose stride ldx is an ODD number of 128-byte lines (e.g. ldx = d + 32),
+ * which spreads the lines of a slab over all L2 channels by itself.  The workspace stays
+ * optional: without it, widths that are a multiple of 32 gather from the row-major X and all
+ * others take one wavefront per row. */
 int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev);
 
 /* coef[k] = +-m[column of entry k] for the packed entries idx[0 .. nnz): the delta VALUES of the

@@ -553,3 +553,28 @@ def test_reference_message_passing_call_pattern():
             out_n.fill_(float("nan"))
             call(x, out_n)
             torch.testing.assert_close(out_n, native_n, atol=1e-4, rtol=1e-4)
+
+
+def test_alias_free_row_stride_needs_no_copy(orc):
+    """X whose row stride is an odd number of 128-byte lines is gathered in place: the library asks
+    for no workspace, and the result is bit-identical to the one through the slab-major copy."""
+    lib = _lib.hip_lib()
+    n, d = 700, 256
+    ei = graphs.add_self_loops(graphs.sbm(n, 7, 0.3, 0.01, seed=9), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+    assert mat.nnz >= 24 * n
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(9)).cuda()
+    xp = torch.zeros((n, d + 32), device="cuda")[:, :d]
+    xp.copy_(x)
+    assert xp.stride(0) == 288 and xp.data_ptr() % 128 == 0
+    y = torch.empty_like(x)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    assert lib.cbm_spmm_workspace_floats(n, d, 256, 256, p(x), p(y)) == n * d
+    assert lib.cbm_spmm_workspace_floats(n, d, 288, 256, p(xp), p(y)) == 0
+    assert lib.cbm_spmm_workspace_floats(n, d, 320, 256, p(xp), p(y)) == n * d      # 10 lines per row: even again
+    say("alias-free stride")
+    want = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, want)
+    got = torch.full_like(x, float("nan")); mat.omp_mkl_csr_fused_spmm_update(xp, got)
+    assert torch.equal(got, want)
+    ref = oracle_product(orc, mat, ei, n, x.cpu().numpy(), True, groups=8)
+    assert np.array_equal(got.cpu().numpy(), ref)
