@@ -21,6 +21,7 @@ Additions that the reference lacks: ``matmul`` / ``CBMMatmul`` with a correct au
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import warnings
 from collections import deque
@@ -30,7 +31,16 @@ import torch
 
 from . import _lib
 
-warnings.filterwarnings("ignore", message="Sparse CSR tensor support is in beta state", category=UserWarning)
+
+
+@contextlib.contextmanager
+def _quiet_sparse_csr():
+    """torch announces on first use that sparse CSR support is in beta; the reference's ``deltas``
+    attribute is such a tensor, so the notice is suppressed around its construction only."""
+    with warnings.catch_warnings():
+        warnings.filterwarnings("ignore", message="Sparse CSR tensor support is in beta state", category=UserWarning)
+        yield
+
 
 __all__ = ["cbm_matrix", "CBMMatmul", "csr_spmm", "tree_levels", "schedule_rows", "relayout_slabs"]
 
@@ -353,7 +363,8 @@ class cbm_matrix:
             if self.col_multiplier is not None:
                 val = val * self.col_multiplier[col]
             n = self.num_rows
-            csr = torch.sparse_csr_tensor(self.rowptr.to(torch.int64), col, val, size=(n, n))
+            with _quiet_sparse_csr():
+                csr = torch.sparse_csr_tensor(self.rowptr.to(torch.int64), col, val, size=(n, n))
             self._deltas = csr if self.deltas_format == "csr" else csr.to_sparse_coo().coalesce()
         return self._deltas
 
@@ -365,7 +376,8 @@ class cbm_matrix:
 
     def to_sparse_csr_tensor(self, row, col, val, data_type=torch.float32):
         """COO triplets -> torch CSR tensor (``cbm.py:132-141``)."""
-        return self.to_sparse_coo_tensor(row, col, val, data_type).to_sparse_csr()
+        with _quiet_sparse_csr():
+            return self.to_sparse_coo_tensor(row, col, val, data_type).to_sparse_csr()
 
     def compression_ratio(self):
         """Element-count ratio CSR(A) / CBM, ``benchmark/utility.py:45-64``."""
