@@ -32,7 +32,6 @@ import torch
 from . import _lib
 
 
-
 @contextlib.contextmanager
 def _quiet_sparse_csr():
     """torch announces on first use that sparse CSR support is in beta; the reference's ``deltas``
