@@ -40,11 +40,12 @@ struct CandEdge { int32_t u, v, w; };
 // [0, n_buckets); offsets[] (n_buckets + 1) is computed, place(t, position) stores the item.
 // Items keep their order inside a bucket: the threads take consecutive chunks of the items and
 // count their chunk per bucket; a prefix over (bucket, chunk) gives every chunk its own range.
-// One chunk when threads x buckets counters would be too many or the input is small.
+// Fewer chunks than threads when threads x buckets counters would be too many; one for small inputs.
 template <class Key, class Place>
 void bucket_stable(int64_t count, int32_t n_buckets, std::vector<int64_t>& offsets, int threads, Key key, Place place) {
-    int chunks = threads;
-    if ((int64_t)chunks * n_buckets > ((int64_t)1 << 28) || count < (int64_t)1 << 16) chunks = 1;
+    // at most 2^26 counters (512 MB) in all
+    int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(threads, ((int64_t)1 << 26) / std::max(n_buckets, 1)));
+    if (count < (int64_t)1 << 16) chunks = 1;
     std::vector<int64_t> start((size_t)chunks * n_buckets);
     const int64_t per = (count + chunks - 1) / chunks;
 #pragma omp parallel for schedule(static, 1) num_threads(chunks)
