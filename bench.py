@@ -227,7 +227,7 @@ def alpha_sweep_bench(args):
     alphas = [args.alpha] if args.alpha is not None else list(w.alphas)
     for alpha in alphas:
         t0 = time.perf_counter()
-        mat = cbm_matrix(ei, None, alpha=alpha, normalized=w.normalized, builder=args.builder)
+        mat = cbm_matrix(ei, None, alpha=alpha, normalized=w.normalized, builder=args.builder, max_levels=args.max_levels)
         t_build = time.perf_counter() - t0
         mat.to(xd.device)
         step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
@@ -265,6 +265,8 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--max-levels", type=int, default=None,
+                    help="depth limit of the arborescence (default: none, as the reference)")
     ap.add_argument("--builder", choices=("auto", "host", "gpu"), default="auto",
                     help="where the format builder computes its row intersections (same format either way)")
     ap.add_argument("--probe", action="store_true",
@@ -298,7 +300,7 @@ def main():
     d = args.d or w.d
     t_gen = time.perf_counter() - t0
     t0 = time.perf_counter()
-    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder)
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder, max_levels=args.max_levels)
     t_build = time.perf_counter() - t0
     n, nnz, n_edges = w.n, mat.nnz, mat.nnz_a
     norm = int(w.normalized)

@@ -45,6 +45,7 @@ HOST_SYMBOLS = {
     "cbm_builder_arrays": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
                                      C.POINTER(_P), C.POINTER(_I64)]),
     "cbm_builder_finish": (C.c_int, [_P, _I32, _P, _I64, C.POINTER(CbmFormat)]),
+    "cbm_builder_set_max_levels": (C.c_int, [_P, _I32]),
     "cbm_builder_free": (None, [_P]),
 }
 HIP_SYMBOLS = {

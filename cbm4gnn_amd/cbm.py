@@ -167,18 +167,26 @@ def _first_pair_capacity(nnz):
     return max(1 << 16, int(nnz))
 
 
-def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
-    """Staged build (``cbm_builder_*``) with ``cbm_row_intersections`` on the current HIP device.
-    Returns (status, seconds spent on upload + kernel + download)."""
+def _build_staged(ei_cpu, n, alpha, threads, fmt, gpu, max_levels):
+    """Staged build (``cbm_builder_*``); with ``gpu`` the row intersections run on the current HIP
+    device (``cbm_row_intersections``).  Returns (status, seconds spent on upload + kernel +
+    download or None)."""
     import time
-    _require_gpu()
-    host, hip = _lib.host_lib(), _lib.hip_lib()
+    if gpu:
+        _require_gpu()
+    host, hip = _lib.host_lib(), _lib.hip_lib() if gpu else None
     handle = C.c_void_p()
     rc = host.cbm_builder_create(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()), ei_cpu.size(1), n, threads,
                                  C.byref(handle))
     if rc:
-        return rc, 0.0
+        return rc, None
     try:
+        if max_levels:
+            rc = host.cbm_builder_set_max_levels(handle, int(max_levels))
+            if rc:
+                return rc, None
+        if not gpu:
+            return host.cbm_builder_finish(handle, alpha, None, -1, C.byref(fmt)), None
         ptrs = [C.c_void_p() for _ in range(6)]
         nnz = C.c_int64()
         rc = host.cbm_builder_arrays(handle, *[C.byref(p) for p in ptrs], C.byref(nnz))
@@ -226,7 +234,7 @@ def _build_with_gpu_intersections(ei_cpu, n, alpha, threads, fmt):
 class cbm_matrix:
 
     def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
-                 deltas_format="csr", threads=0, builder="auto"):
+                 deltas_format="csr", threads=0, builder="auto", max_levels=None):
         ei = torch.as_tensor(edge_index)
         if ei.dim() != 2 or ei.size(0) != 2:
             raise ValueError("Edge index should have shape (2, num_edges)")
@@ -252,12 +260,13 @@ class cbm_matrix:
         if builder == "auto":
             builder = "gpu" if (torch.cuda.is_available() and ei_cpu.size(1) >= _GPU_BUILDER_MIN_EDGES) else "host"
         self.builder = builder
+        # max_levels: no tree level beyond this one (None = no limit, as the reference).  Rows that
+        # would land deeper hang off the root instead: more delta entries, fewer dependent launches.
+        if max_levels is not None and int(max_levels) < 1:
+            raise ValueError("max_levels must be >= 1 (1 = flat tree)")
+        self.max_levels = None if max_levels is None else int(max_levels)
         fmt = _lib.CbmFormat()
-        if builder == "gpu":
-            rc, t_pairs = _build_with_gpu_intersections(ei_cpu, n, self.alpha, int(threads), fmt)
-        else:
-            rc, t_pairs = _lib.host_lib().cbm_build_host(_ptr(ei_cpu[0].contiguous()), _ptr(ei_cpu[1].contiguous()),
-                                                         ei_cpu.size(1), n, self.alpha, int(threads), C.byref(fmt)), None
+        rc, t_pairs = _build_staged(ei_cpu, n, self.alpha, int(threads), fmt, builder == "gpu", self.max_levels)
         try:
             _lib.check(rc, "cbm_build_host")
             t4 = (C.c_double * 4)()
@@ -341,6 +350,7 @@ class cbm_matrix:
             raise ValueError(f"{path} does not hold a consistent CBM format")
         self.build_seconds = None
         self.builder = None                                 # loaded, not built
+        self.max_levels = None
         self._deltas, self._dev, self._transposed = None, {}, None
         self.stream_coefficients = True
         self.relayout = True

@@ -458,7 +458,8 @@ int candidates_from_pairs(const Graph& g, int32_t alpha, const cbm_pair* pairs, 
 thread_local double g_last_timings[4] = {0, 0, 0, 0};
 
 // Arborescence, tree arrays, signed deltas.
-int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, cbm_format* out, double t_mark) {
+int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, int32_t max_levels, cbm_format* out,
+                  double t_mark) {
     const int32_t N = g.N;
     const std::vector<int64_t>& rp = g.rp; const std::vector<int32_t>& ci = g.ci; const std::vector<int32_t>& nnz = g.nnz;
     const int64_t nnzA = g.nnzA;
@@ -478,12 +479,35 @@ int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, cbm_
 
         lap(2);
         // ---- tree arrays: children ascending per parent; levels by BFS --------------------------
-        std::vector<int32_t> mst_row(N + 2, 0), mst_col(N);
-        for (int32_t v = 0; v < N; v++) mst_row[par[v] + 1]++;
-        for (int32_t u = 0; u <= N; u++) mst_row[u + 1] += mst_row[u];
-        {
+        std::vector<int32_t> mst_row, mst_col(N);
+        auto children_of = [&]() {
+            mst_row.assign(N + 2, 0);
+            for (int32_t v = 0; v < N; v++) mst_row[par[v] + 1]++;
+            for (int32_t u = 0; u <= N; u++) mst_row[u + 1] += mst_row[u];
             std::vector<int32_t> fill(mst_row.begin(), mst_row.end() - 1);
             for (int32_t v = 0; v < N; v++) mst_col[fill[par[v]]++] = v;
+        };
+        children_of();
+        bool cut_any = false;
+        if (max_levels > 0) {
+            // Depth limit: a row that would land on level max_levels is re-attached to the virtual
+            // root (its delta becomes the whole row) and its subtree moves up with it.  Every tree
+            // level costs the multiply a dependent launch, so a few extra delta entries can be the
+            // better deal; the result is still a valid format, only no longer of minimum weight.
+            std::vector<int32_t> lvl(N, 0), queue(N);
+            int32_t head = 0, tail = 0;
+            for (int32_t q = mst_row[N]; q < mst_row[N + 1]; q++) queue[tail++] = mst_col[q];
+            while (head < tail) {
+                const int32_t u = queue[head++];
+                for (int32_t q = mst_row[u]; q < mst_row[u + 1]; q++) {
+                    const int32_t c = mst_col[q];
+                    lvl[c] = lvl[u] + 1;
+                    if (lvl[c] >= max_levels) { par[c] = N; lvl[c] = 0; cut_any = true; }
+                    queue[tail++] = c;
+                }
+            }
+            if (tail != N) return CBM_ERR_INTERNAL;
+            if (cut_any) children_of();
         }
         std::vector<int32_t> level(N, -1), order(N), level_off;
         {
@@ -524,7 +548,7 @@ int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, cbm_
         }
         int64_t run = 0;
         for (int32_t v = 0; v < N; v++) { run += drp[v + 1]; if (run > INT32_MAX) return CBM_ERR_SHAPE; drp[v + 1] = (int32_t)run; }
-        if (run != weight) return CBM_ERR_INTERNAL;      // nnz(delta) must equal the arborescence weight
+        if (!cut_any && run != weight) return CBM_ERR_INTERNAL;      // nnz(delta) must equal the arborescence weight
         std::vector<uint32_t> idx(run);
 #pragma omp parallel for schedule(dynamic, 256) num_threads(threads)
         for (int32_t v = 0; v < N; v++) {
@@ -560,6 +584,7 @@ int finish_format(const Graph& g, std::vector<CandEdge>& cand, int threads, cbm_
 struct cbm_builder {
     Graph g;
     int threads = 1;
+    int32_t max_levels = 0;      // 0 = no limit
 };
 
 extern "C" {
@@ -654,11 +679,18 @@ int cbm_builder_finish(cbm_builder* b, int32_t alpha, const cbm_pair* pairs, int
         if (rc) return rc;
         const double t1 = omp_get_wtime();
         g_last_timings[1] = t1 - t0;
-        return finish_format(b->g, cand, b->threads, out, t1);
+        return finish_format(b->g, cand, b->threads, b->max_levels, out, t1);
     } catch (const std::bad_alloc&) {
         cbm_format_free(out);
         return CBM_ERR_ALLOC;
     }
+}
+
+int cbm_builder_set_max_levels(cbm_builder* b, int32_t max_levels) {
+    if (!b) return CBM_ERR_NULL;
+    if (max_levels < 0) return CBM_ERR_SHAPE;
+    b->max_levels = max_levels;
+    return CBM_OK;
 }
 
 void cbm_builder_free(cbm_builder* b) { delete b; }

@@ -98,6 +98,12 @@ int cbm_build_host(const int32_t* row, const int32_t* col, int64_t n_edges, int3
  *   cbm_builder_finish   candidate edges, arborescence, deltas.  pairs = (i, j, s) with i < j and
  *                        s = |row_i ^ row_j| in any order, holding at least every pair with
  *                        2 s > min(nnz_i, nnz_j) + alpha; n_pairs < 0 computes them on the host.
+ *   cbm_builder_set_max_levels   optional, before finish: no tree level beyond max_levels (0 = no
+ *                        limit, the default and what the reference does).  A row that would land
+ *                        deeper is re-attached to the virtual root together with its subtree:
+ *                        fewer dependent launches per multiply for a few more delta entries (nnz
+ *                        then exceeds msa_weight).  No reference counterpart; alpha is the
+ *                        reference's only knob for the same trade (cbm_extensions.cpp:75-103).
  * cbm_build_host is create + finish(n_pairs = -1) + free.  Replaces the mkl_sparse_syrk step of
  * cbm_init_v1_/_v2_ (cbm_extensions.cpp:46-65) as a separable stage. */
 typedef struct cbm_builder cbm_builder;
@@ -108,6 +114,7 @@ int cbm_builder_arrays(const cbm_builder* b, const int64_t** rowptr, const int32
                        const int32_t** row_t, const int64_t** after, const int32_t** row_nnz, int64_t* nnz);
 int cbm_builder_finish(cbm_builder* b, int32_t alpha, const struct cbm_pair* pairs, int64_t n_pairs,
                        struct cbm_format* out);
+int cbm_builder_set_max_levels(cbm_builder* b, int32_t max_levels);
 void cbm_builder_free(cbm_builder* b);
 
 void cbm_format_free(cbm_format* f);

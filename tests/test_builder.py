@@ -294,3 +294,23 @@ def test_staged_build_rejects_bad_pairs():
     host = _lib.host_lib()
     assert host.cbm_builder_finish(None, 0, None, -1, C.byref(_lib.CbmFormat())) == 1
     assert host.cbm_builder_create(None, None, 5, 4, 1, C.byref(C.c_void_p())) == 1
+
+
+@pytest.mark.parametrize("max_levels", [1, 2, 3, 6])
+def test_depth_limit_gives_a_valid_shallower_format(orc, max_levels):
+    w = _small_chain_workload()                               # 64-level chain below clique blocks
+    ei, n = w.edge_index, w.n
+    free = cbm_matrix(torch.from_numpy(ei), None, alpha=0)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, max_levels=max_levels)
+    assert free.n_levels > 6 and mat.n_levels == min(max_levels, free.n_levels)
+    assert mat.nnz >= free.nnz and mat.n_candidates == free.n_candidates
+    if max_levels == 1:
+        assert mat.nnz == mat.nnz_a and (mat.parent == -1).all()           # flat tree: delta = A
+    _assert_format_equals_derivation(orc, ei, n, mat)
+    assert orc.check_format(ei, n, mat.rowptr.numpy(), _u32(mat.idx), mat.mst_row.numpy(), mat.mst_col.numpy())
+    assert mat.check_format(torch.from_numpy(ei))
+    # rows above the limit keep the parent the arborescence gave them
+    keep = mat.parent.numpy() >= 0
+    assert np.array_equal(mat.parent.numpy()[keep], free.parent.numpy()[keep])
+    with pytest.raises(ValueError):
+        cbm_matrix(torch.from_numpy(ei), None, alpha=0, max_levels=0)

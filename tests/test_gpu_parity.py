@@ -578,3 +578,34 @@ def test_alias_free_row_stride_needs_no_copy(orc):
     assert torch.equal(got, want)
     ref = oracle_product(orc, mat, ei, n, x.cpu().numpy(), True, groups=8)
     assert np.array_equal(got.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+def test_depth_limited_trees_multiply_like_the_oracle(orc, normalized):
+    """max_levels re-attaches deep rows to the root: a different (heavier, shallower) but valid
+    format; the product is the same matrix, bit for bit against the oracle on the product's tree."""
+    ei = graphs.sbm_with_chain(n=1500, blocks=24, p_in=1.0, mean_deg=80.0, chain=64, base=48, seed=0)
+    n = 1500
+    if normalized:
+        ei = graphs.add_self_loops(ei, n)
+    x = np.random.default_rng(11).standard_normal((n, 96)).astype(np.float32)
+    dense = orc.dense_product(ei, n, x, normalized)
+    levels = []
+    for limit in (None, 8, 3, 1):
+        say("depth limit", limit, normalized)
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized, max_levels=limit)
+        levels.append(mat.n_levels)
+        got = gpu_product(mat, x, normalized)
+        assert np.array_equal(got, oracle_product(orc, mat, ei, n, x, normalized))
+        assert orc.max_rel_err(got, dense) <= TOL_CSR
+    assert levels[0] > 8 and levels[1:] == [8, 3, 1]
+
+
+def test_tuner_sweeps_depth_limits():
+    from cbm4gnn_amd.tuner import tune_alpha
+    w = graphs.workload("c2", scale=0.25)
+    say("tuner with depth limits")
+    best, rows = tune_alpha(w.edge_index, 64, alphas=(0, 10_000), normalized=True, iters=10, warmup=2, max_levels=(None, 3))
+    assert [(r["alpha"], r["max_levels"]) for r in rows] == [(0, None), (0, 3), (10_000, None), (10_000, 3)]
+    assert rows[1]["tree_levels"] <= 3 < rows[0]["tree_levels"] and rows[1]["nnz_delta"] >= rows[0]["nnz_delta"]
+    assert sum(r["best"] for r in rows) == 1 and next(r for r in rows if r["best"])["alpha"] == best
