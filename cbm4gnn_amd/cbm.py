@@ -615,7 +615,7 @@ class cbm_matrix:
             return self
         if self._transposed is None:
             ei = self._edge_index_cpu
-            t = cbm_matrix(torch.stack([ei[1], ei[0]]), None, alpha=self.alpha, normalized=False)
+            t = cbm_matrix(torch.stack([ei[1], ei[0]]), None, alpha=self.alpha, normalized=False, max_levels=self.max_levels)
             t.col_multiplier = self.col_multiplier      # diag(m) A^T diag(m): same vector both sides
             t.normalized = self.normalized
             t._transposed = self
