@@ -303,14 +303,20 @@ class cbm_matrix:
 
         self._deltas = None
         self._dev = {}
-        self.stream_coefficients = True     # False: gather m[col] in the kernel, 4 B/entry less device memory
+        self._stream_coefficients = True    # see the property
         self.relayout = True                # False: gather from the caller's row-major X, no n*d scratch per call
         self._transposed = None
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
 
     # ------------------------------------------------------------------ on-disk cache --------
     _SAVED_ARRAYS = ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col")
-    FORMAT_VERSION = 1
+    FORMAT_VERSION = 2                  # 2 adds the depth limit (max_levels); version 1 files load with none
+
+    @staticmethod
+    def _npz_path(path):
+        """``np.savez`` appends ``.npz`` to a name without it; ``save`` and ``load`` agree on that."""
+        path = str(path)
+        return path if path.endswith(".npz") else path + ".npz"
 
     def save(self, path):
         """Write the built format to ``path`` (NumPy ``.npz``, no pickled objects).  The reference
@@ -321,19 +327,21 @@ class cbm_matrix:
         if self._edge_index_cpu is not None:                      # needed to build the transposed operator
             arrays["edge_index"] = self._edge_index_cpu.numpy()
         meta = np.array([self.FORMAT_VERSION, self.num_rows, self.alpha, int(self.normalized), self.nnz, self.nnz_a,
-                         self.n_candidates, self.n_levels, int(self.is_symmetric)], np.int64)
-        np.savez(path, meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
+                         self.n_candidates, self.n_levels, int(self.is_symmetric), self.max_levels or 0], np.int64)
+        np.savez(self._npz_path(path), meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
 
     @classmethod
     def load(cls, path):
         """Inverse of ``save``; runs no builder.  Consistency of the arrays is checked."""
+        path = cls._npz_path(path)
         with np.load(path, allow_pickle=False) as z:
             meta = z["meta"].tolist()
-            if meta[0] != cls.FORMAT_VERSION:
+            if meta[0] not in (1, cls.FORMAT_VERSION):
                 raise ValueError(f"unsupported CBM file version {meta[0]}")
             self = cls.__new__(cls)
             (_, self.num_rows, self.alpha, normalized, self.nnz, self.nnz_a, self.n_candidates, self.n_levels,
-             symmetric) = meta
+             symmetric) = meta[:9]
+            self.max_levels = (meta[9] or None) if meta[0] >= 2 else None
             self.normalized, self.is_symmetric = bool(normalized), bool(symmetric)
             self.deltas_format = str(z["deltas_format"])
             for k in cls._SAVED_ARRAYS:
@@ -350,11 +358,33 @@ class cbm_matrix:
             raise ValueError(f"{path} does not hold a consistent CBM format")
         self.build_seconds = None
         self.builder = None                                 # loaded, not built
-        self.max_levels = None
         self._deltas, self._dev, self._transposed = None, {}, None
-        self.stream_coefficients = True
+        self._stream_coefficients = True
         self.relayout = True
         return self
+
+    # Settings the cached device arrays depend on: changing one drops the cache, so that a later
+    # multiply never runs on coefficients or schedules derived from the old value.
+    @property
+    def stream_coefficients(self):
+        """True (default): the SpMM streams ``+-m[col]`` per delta entry, expanded once per device;
+        False: it gathers ``m[col]`` in the kernel, 4 B per entry less device memory."""
+        return self._stream_coefficients
+
+    @stream_coefficients.setter
+    def stream_coefficients(self, value):
+        if bool(value) != self._stream_coefficients:
+            self._dev = {}
+        self._stream_coefficients = bool(value)
+
+    @property
+    def col_multiplier(self):
+        return self._col_multiplier
+
+    @col_multiplier.setter
+    def col_multiplier(self, value):
+        self._col_multiplier = value
+        self._dev, self._deltas = {}, None
 
     # ------------------------------------------------------------------ format views --------
     def columns(self):
@@ -548,10 +578,21 @@ class cbm_matrix:
         if yd is not y:
             y.copy_(yd)
 
+    def _plain_spmm_update(self, x, y):
+        """The reference's un-fused ``*_spmm_update``: delta SpMM, then the plain walk.  On a
+        matrix built with ``normalized=True`` the reference's delta values are ``+-m[col]``
+        (``cbm.py:56-66`` with the v2 builder, ``cbm_extensions.cpp:504-585``), so that call
+        returns ``A diag(m) X`` -- the right scaling only; the same here."""
+        if self.col_multiplier is None:
+            self._run_spmm_update(x, y, use_m=False)
+            return
+        self._run_spmm(x, y, use_m=True, scale_roots=False)
+        self._run_propagate(y, use_m=False)
+
     # ------------------------------------------------------------------ reference methods ---
     # "Sequential" methods (cbm.py:144-188)
     def seq_mkl_csr_spmm_update(self, x, y):
-        self._run_spmm_update(x, y, use_m=False)
+        self._plain_spmm_update(x, y)
 
     def seq_mkl_csr_spmm(self, x, y):
         self._run_spmm(x, y, use_m=self.col_multiplier is not None, scale_roots=False)
@@ -567,7 +608,7 @@ class cbm_matrix:
 
     # "Parallel" methods (cbm.py:191-249)
     def omp_mkl_csr_spmm_update(self, x, y):
-        self._run_spmm_update(x, y, use_m=False)
+        self._plain_spmm_update(x, y)
 
     def omp_mkl_csr_spmm(self, x, y):
         self._run_spmm(x, y, use_m=self.col_multiplier is not None, scale_roots=False)
@@ -581,7 +622,7 @@ class cbm_matrix:
     def omp_mkl_csr_spmm_update_v2(self, x, y):
         # the reference wrapper (cbm.py:219-228) names a native function that its extension
         # never exports; here it is the plain spmm + update
-        self._run_spmm_update(x, y, use_m=False)
+        self._plain_spmm_update(x, y)
 
     def omp_mkl_csr_fused_spmm_update(self, x, y):
         self._run_spmm_update(x, y, use_m=True)
@@ -624,7 +665,12 @@ class cbm_matrix:
 
 
 class CBMMatmul(torch.autograd.Function):
-    """y = A_hat x with backward g -> A_hat^T g, both through the HIP kernels."""
+    """y = A_hat x with backward g -> A_hat^T g, both through the HIP kernels.
+
+    ``fused=True``: ``diag(m) A diag(m) x`` (the fused normalised path).  ``fused=False``: the
+    reference's un-fused path, ``A x`` on a plain matrix and ``A diag(m) x`` on a normalised one
+    (its delta values carry the right scaling, ``cbm.py:255-265``); backward is then
+    ``diag(m) A^T g``."""
 
     @staticmethod
     def forward(ctx, x, mat, fused):
@@ -635,14 +681,20 @@ class CBMMatmul(torch.autograd.Function):
             raise RuntimeError("rhs tensor (NOT torch::kFloat32)")
         xd = xd.contiguous()
         y = torch.empty_like(xd)
-        mat._run_spmm_update(xd, y, use_m=fused)
+        if fused:
+            mat._run_spmm_update(xd, y, use_m=True)
+        else:
+            mat._plain_spmm_update(xd, y)
         return y
 
     @staticmethod
     def backward(ctx, g):
         g = g.contiguous()
         gx = torch.empty_like(g)
-        ctx.mat.transposed()._run_spmm_update(g, gx, use_m=ctx.fused)
+        mat = ctx.mat
+        mat.transposed()._run_spmm_update(g, gx, use_m=ctx.fused)
+        if not ctx.fused and mat.col_multiplier is not None:
+            gx.mul_(mat.col_multiplier.to(gx.device).unsqueeze(1))
         return gx, None, None
 
 

@@ -22,6 +22,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "../../include/cbm_hip.h"
@@ -568,8 +570,10 @@ inline Tiling pick_tiling(int d, int64_t ld_a, int64_t ld_b, const void* pa, con
     return t;
 }
 
-// SpMM kernel choice: 0 = automatic, 1 = always one wave per row, 2 = slabs whenever the shape allows
-int g_spmm_kernel = 0;
+// SpMM kernel choice: 0 = automatic, 1 = always one wave per row, 2 = slabs whenever the shape allows.
+// A process-wide tuning hook; atomic so that threads launching on their own streams may read it
+// while another thread sets it.
+std::atomic<int> g_spmm_kernel{0};
 
 // ---------------------------------------------------------------------------------------------
 // (3) Row intersections for the builder: all pairs (i, j > i) of rows of A with
@@ -716,7 +720,7 @@ inline int padded_slab_count(int d) {
 inline SlabPlan plan_slabs(int d, int64_t ldx, int64_t ldz, const void* X, const void* Z, bool have_workspace,
                            bool force_copy) {
     SlabPlan p;
-    if (g_spmm_kernel == 1 && !force_copy) return p;
+    if (g_spmm_kernel.load(std::memory_order_relaxed) == 1 && !force_copy) return p;
     const bool x_vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16);
     p.vec_out = d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16);
     SlabPlan direct;                                       // gather from the caller's row-major X
@@ -772,44 +776,70 @@ inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
 // fastest at 3-4 (3-8 % over 6-8), rows averaging 45 entries at 5-6 (4 costs 7 %, 3 costs 20 %),
 // rows averaging 13 entries at the register limit (6 costs 7 %); 256-byte slabs are fastest at
 // 3-4 on every graph tried.
-int g_spmm_occupancy = 0;                                  // 0 = automatic
+std::atomic<int> g_spmm_occupancy{0};                      // 0 = automatic
 inline int slab_waves_per_simd(int64_t nnz, int32_t n, int lpe) {
-    if (g_spmm_occupancy > 0) return g_spmm_occupancy;
+    const int fixed = g_spmm_occupancy.load(std::memory_order_relaxed);
+    if (fixed > 0) return fixed;
     if (lpe == 16) return 4;
     if (nnz >= (int64_t)128 * n) return 4;
     return nnz >= (int64_t)32 * n ? 6 : 8;                 // 8: every wavefront the registers allow
 }
 
-// Workgroups per XCD of the persistent slab kernel that are resident at once, and workgroups per
-// XCD that give one wavefront per SIMD.
+// Per-device launch facts of the persistent slab kernel, queried once per device (a process may
+// drive several devices from several threads): compute units, and for every instantiation the
+// workgroups per XCD that are resident at once.
+constexpr int kMaxDevices = 64;
+struct DeviceFacts {
+    int cus = 0;
+    int groups[2][2][3] = {};                              // [PACKED][lpe == 16][coefficient mode]
+};
+DeviceFacts g_facts[kMaxDevices];
+std::atomic<int> g_facts_ready[kMaxDevices];               // zero-initialised
+std::mutex g_facts_mutex;
+
 template <class K>
-int resident_groups_per_xcd(K kernel) {
-    int dev = 0, cus = 0, per_cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+int resident_groups_per_xcd(K kernel, int cus) {
+    int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kWave * kWavesPerBlock, 0) != hipSuccess) return 0;
     if (cus < kXcds || per_cu < 1) return 0;
     return (cus / kXcds) * per_cu;
 }
 
-// Resident workgroups per XCD of each slab kernel instantiation, queried once.
 template <bool PACKED>
-int slab_kernel_groups(int lpe, int coef_mode) {
-    static const int g[2][3] = {
-        {resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefStream, CBM_SLAB_ROUNDS>),
-         resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSign, CBM_SLAB_ROUNDS>),
-         resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>)},
-        {resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefStream, CBM_SLAB_ROUNDS>),
-         resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSign, CBM_SLAB_ROUNDS>),
-         resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>)}};
-    return g[lpe == 8 ? 0 : 1][coef_mode];
+void fill_groups(int (&g)[2][3], int cus) {
+    g[0][kCoefStream] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefStream, CBM_SLAB_ROUNDS>, cus);
+    g[0][kCoefSign] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSign, CBM_SLAB_ROUNDS>, cus);
+    g[0][kCoefSignM] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>, cus);
+    g[1][kCoefStream] = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefStream, CBM_SLAB_ROUNDS>, cus);
+    g[1][kCoefSign] = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSign, CBM_SLAB_ROUNDS>, cus);
+    g[1][kCoefSignM] = resident_groups_per_xcd(spmm_slab_per_xcd<16, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>, cus);
 }
 
-inline int groups_per_xcd_per_wave() {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    return cus / kXcds;
+// Facts of the CURRENT device, or nullptr if they cannot be had.
+const DeviceFacts* device_facts() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    if (!g_facts_ready[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_facts_mutex);
+        if (!g_facts_ready[dev].load(std::memory_order_relaxed)) {
+            DeviceFacts f;
+            if (hipDeviceGetAttribute(&f.cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return nullptr;
+            fill_groups<false>(f.groups[0], f.cus);
+            fill_groups<true>(f.groups[1], f.cus);
+            g_facts[dev] = f;
+            g_facts_ready[dev].store(1, std::memory_order_release);
+        }
+    }
+    return &g_facts[dev];
+}
+
+// Byte ranges [a, a + bytes_a) and [b, b + bytes_b) share at least one byte.
+inline bool ranges_overlap(const void* a, int64_t bytes_a, const void* b, int64_t bytes_b) {
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return bytes_a > 0 && bytes_b > 0 && pa < pb + (uintptr_t)bytes_b && pb < pa + (uintptr_t)bytes_a;
+}
+inline int64_t matrix_bytes(int32_t n, int32_t d, int64_t ld) {
+    return n > 0 && d > 0 ? ((int64_t)(n - 1) * ld + d) * 4 : 0;
 }
 
 inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s) {
@@ -833,9 +863,17 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
     if (sched && !aligned(sched, 16)) return CBM_ERR_SHAPE;
-    if (X == Z) return CBM_ERR_SHAPE;                    // rows of X are gathered while rows of Z are written
+    // rows of X are gathered while rows of Z are written: the two must not share a byte
+    if (X == Z || ranges_overlap(X, matrix_bytes(n, d, ldx), Z, matrix_bytes(n, d, ldz))) return CBM_ERR_SHAPE;
     const bool ready = (flags & CBM_SPMM_WORKSPACE_READY) != 0;
-    const bool have_ws = workspace && aligned(workspace, 16) && workspace != Z && workspace != X;
+    if (workspace) {                                      // the slab-major copy must be disjoint from X and Z
+        if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
+        const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+        if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
+            ranges_overlap(workspace, ws_bytes, Z, matrix_bytes(n, d, ldz)))
+            return CBM_ERR_SHAPE;
+    }
+    const bool have_ws = workspace != nullptr;
     if (ready && !have_ws) return CBM_ERR_NULL;
     if (n == 0 || d == 0) return CBM_OK;
     const int4* sc = reinterpret_cast<const int4*>(sched);
@@ -850,8 +888,9 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
             Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
         }
         const int coef_mode = val ? kCoefStream : (m ? kCoefSignM : kCoefSign);
-        static const int per_wave = groups_per_xcd_per_wave();
-        int G = slab_kernel_groups<PACKED>(lpe, coef_mode);
+        const DeviceFacts* facts = device_facts();
+        const int per_wave = facts ? facts->cus / kXcds : 0;
+        int G = facts ? facts->groups[PACKED ? 1 : 0][lpe == 8 ? 0 : 1][coef_mode] : 0;
         if (G > 0) {
             const int cap = per_wave * slab_waves_per_simd(nnz, n, lpe);
             if (cap > 0 && G > cap) G = cap;

@@ -111,7 +111,18 @@ def test_symmetry_flag_and_transpose():
     assert not c.is_symmetric
     t = c.transposed()
     assert t is not c and t.transposed() is c
-    assert torch.equal(t.deltas.to_dense(), c.deltas.to_dense().t()) or t.nnz <= 4
+    # the transposed object is the CBM of A^T: its rows rebuild to the transposed adjacency
+    assert t.check_format(torch.stack([ei[1], ei[0]]))
+    with pytest.raises(ValueError):
+        t.check_format(ei)                                  # and not to A itself (A is not symmetric)
+    assert t.nnz_a == c.nnz_a == 4 and t.num_rows == c.num_rows
+    # a larger directed graph, where the deltas really compress: same checks
+    rng = np.random.default_rng(4)
+    base = rng.integers(0, 40, (2, 300)).astype(np.int32)
+    big = torch.from_numpy(np.unique(np.concatenate([base, np.stack([np.arange(40), np.arange(40)]).astype(np.int32)], 1), axis=1))
+    cb = cbm_matrix(big, None, alpha=0)
+    tb = cb.transposed()
+    assert not cb.is_symmetric and tb.check_format(torch.stack([big[1], big[0]]))
     und = cbm_matrix(torch.from_numpy(graphs.erdos_renyi(10, 0.5, 1)), None)
     assert und.is_symmetric and und.transposed() is und
 
@@ -135,6 +146,14 @@ def test_save_and_load_round_trip(tmp_path):
         assert b.check_format(edge_index)
         if not b.is_symmetric:
             assert torch.equal(b.transposed().rowptr, a.transposed().rowptr)
+    # a path without the extension names the same file in save and load; the depth limit survives
+    deep = cbm_matrix(ei, None, alpha=0, max_levels=2)
+    bare = str(tmp_path / "no_extension")
+    deep.save(bare)
+    again = cbm_matrix.load(bare)
+    assert again.max_levels == 2 and again.n_levels <= 2 and torch.equal(again.idx, deep.idx)
+    assert cbm_matrix.load(bare + ".npz").max_levels == 2
+    assert cbm_matrix.load(path).max_levels is None
     bad = dict(np.load(path))
     bad["order"] = bad["order"][:-1]
     np.savez(str(tmp_path / "bad.npz"), **bad)

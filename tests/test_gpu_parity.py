@@ -609,3 +609,116 @@ def test_tuner_sweeps_depth_limits():
     assert [(r["alpha"], r["max_levels"]) for r in rows] == [(0, None), (0, 3), (10_000, None), (10_000, 3)]
     assert rows[1]["tree_levels"] <= 3 < rows[0]["tree_levels"] and rows[1]["nnz_delta"] >= rows[0]["nnz_delta"]
     assert sum(r["best"] for r in rows) == 1 and next(r for r in rows if r["best"])["alpha"] == best
+
+
+def test_plain_methods_on_a_normalised_matrix_apply_the_right_scaling_only(orc):
+    """The reference's delta values on a ``normalized=True`` matrix are +-m[col] (cbm.py:56-66 with
+    the v2 builder), so its un-fused calls (``*_spmm_update``, ``*_torch_csr_matmul``) return
+    A diag(m) X, and ``*_csr_spmm`` followed by ``*_csr_update`` is the same thing in two steps.
+    Oracle: SpMM with values +-m[col], then the plain walk."""
+    n, d = 800, 96
+    ei = graphs.add_self_loops(graphs.sbm(n, 10, 0.3, 0.01, seed=21), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+    assert mat.n_levels >= 2
+    x = np.random.default_rng(21).standard_normal((n, d)).astype(np.float32)
+    m = orc.col_multiplier(ei, n)
+    col, sign = mat.columns()
+    val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
+    z = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=mat_groups(mat, d))
+    want = orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z.copy())
+    a = orc.dense_adjacency(ei, n).astype(np.float64)
+    dense = a @ (m.astype(np.float64)[:, None] * x.astype(np.float64))
+    assert orc.max_rel_err(want, dense) <= TOL_CBM
+    xd = torch.from_numpy(x).cuda()
+    say("plain methods on a normalised matrix")
+    for name in ("seq_mkl_csr_spmm_update", "omp_mkl_csr_spmm_update", "omp_mkl_csr_spmm_update_v2"):
+        yd = torch.full_like(xd, float("nan"))
+        getattr(mat, name)(xd, yd)
+        assert np.array_equal(yd.cpu().numpy(), want), name
+    two = torch.full_like(xd, float("nan"))
+    mat.omp_mkl_csr_spmm(xd, two)
+    assert np.array_equal(two.cpu().numpy(), z)
+    mat.omp_mkl_csr_update(two)
+    assert np.array_equal(two.cpu().numpy(), want)
+    # deltas @ x (the torch route of cbm.py:255-265) + update agrees to rounding
+    mixed = (mat.deltas.to(xd.device) @ xd).contiguous()
+    mat.seq_mkl_csr_update(mixed)
+    assert orc.max_rel_err(mixed.cpu().numpy(), want) <= 1e-5
+    # the matmul-returning twins, and their gradient diag(m) A^T g
+    xg = xd.clone().requires_grad_(True)
+    y = mat.omp_torch_csr_matmul(xg)
+    assert np.array_equal(y.detach().cpu().numpy(), want)
+    g = torch.randn((n, d), generator=torch.Generator().manual_seed(3)).cuda()
+    (y * g).sum().backward()
+    want_g = m.astype(np.float64)[:, None] * (a.T @ g.cpu().numpy().astype(np.float64))
+    assert orc.max_rel_err(xg.grad.cpu().numpy(), want_g) <= TOL_CBM
+    # and the fused calls still give diag(m) A diag(m) X
+    yf = torch.empty_like(xd); mat.omp_mkl_csr_fused_spmm_update(xd, yf)
+    assert orc.max_rel_err(yf.cpu().numpy(), orc.dense_product(ei, n, x, True)) <= TOL_CBM
+
+
+def test_changing_a_cached_setting_takes_effect():
+    """``stream_coefficients`` and ``col_multiplier`` feed device arrays that are cached per device;
+    changing either after a multiply must not leave the old arrays in use."""
+    n, d = 500, 64
+    ei = graphs.add_self_loops(graphs.sbm(n, 5, 0.3, 0.01, seed=8), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(8)).cuda()
+    say("cached settings")
+    y1 = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, y1)
+    assert mat._device_arrays(x.device)["coef"] is not None
+    mat.stream_coefficients = False
+    y2 = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, y2)
+    assert mat._device_arrays(x.device)["coef"] is None and torch.equal(y1, y2)
+    mat.col_multiplier = mat.col_multiplier * 2.0           # diag(2m) A diag(2m) = 4 x the product, exactly
+    y3 = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, y3)
+    assert torch.equal(y3, 4.0 * y1)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_a_loaded_format_multiplies_like_the_built_one(tmp_path, symmetric):
+    """save() -> load() -> multiply and backward: bit-equal to the freshly built matrix, including
+    the depth limit and (directed graphs) the transposed operator of the backward pass."""
+    n, d = 900, 72
+    ei = graphs.add_self_loops(graphs.sbm(n, 9, 0.3, 0.01, seed=31), n)
+    if not symmetric:                                       # drop a third of the directed edges
+        keep = (np.random.default_rng(31).random(ei.shape[1]) > 0.33) | (ei[0] == ei[1])
+        ei = np.ascontiguousarray(ei[:, keep])
+    built = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True, max_levels=3)
+    assert built.is_symmetric == symmetric and 2 <= built.n_levels <= 3
+    path = str(tmp_path / "fmt")
+    built.save(path)
+    loaded = cbm_matrix.load(path)
+    assert loaded.max_levels == 3
+    say("loaded format", symmetric)
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(31)).cuda()
+    g = torch.randn((n, d), generator=torch.Generator().manual_seed(32)).cuda()
+    out = []
+    for mat in (built, loaded):
+        y = torch.full_like(x, float("nan")); mat.omp_mkl_csr_fused_spmm_update(x, y)
+        yp = torch.full_like(x, float("nan")); mat.omp_mkl_csr_spmm_update(x, yp)
+        xg = x.clone().requires_grad_(True)
+        (mat.matmul(xg) * g).sum().backward()
+        out.append((y, yp, xg.grad))
+    for a, b in zip(*out):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+    if not symmetric:
+        t_built, t_loaded = built.transposed(), loaded.transposed()
+        assert t_loaded.max_levels == 3
+        for name in ("rowptr", "idx", "parent", "order", "level_off"):
+            assert torch.equal(getattr(t_built, name), getattr(t_loaded, name)), name
+
+
+def test_gpu_built_format_counts_equal_the_oracle_build(orc):
+    """builder="gpu" on the 4,096-node SBM and the duplication graph at a quarter of its size: the
+    number of candidate edges and the weight of the arborescence (delta non-zeros) equal those of
+    the oracle's own build (its own candidate scan, its own Chu-Liu/Edmonds)."""
+    for name, scale, alpha in (("c1", 1.0, 0), ("c2", 0.25, 0), ("c2", 0.25, 8)):
+        w = graphs.workload(name, scale=scale)
+        say("gpu build vs oracle build", name, scale, alpha)
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, builder="gpu")
+        fmt = orc.build_format(w.edge_index, w.n, alpha)
+        assert mat.n_candidates == fmt["n_candidates"]
+        assert mat.nnz == fmt["nnz"] == int(fmt["d_row"].shape[0])
+        assert orc.check_format(w.edge_index, w.n, mat.rowptr.numpy(), mat.idx.numpy().view(np.uint32),
+                                mat.mst_row.numpy(), mat.mst_col.numpy())

@@ -261,3 +261,44 @@ def test_compression_ratio_formula(orc):
     # benchmark/utility.py:45-64 in element counts
     assert orc.compression_ratio(10, 40, 40) == pytest.approx((11 + 80) / (11 + 80 + 12 + 10))
     assert orc.compression_ratio(10, 40, 10) > 1.0
+
+
+def test_grouped_csr_spmm_order_is_pinned(orc):
+    """``csr_spmm(groups=g)``: entry k of a row goes to partial sum k mod g (each an in-order FMA
+    chain) and the g sums are added pairwise as a balanced tree.  Pinned by integer features
+    (exact for every order), by real features against the in-order sum, and by a row whose fp32
+    result differs between the orders in a way worked out by hand."""
+    rng = np.random.default_rng(3)
+    n, d = 257, 19
+    ei = graphs.add_self_loops(graphs.erdos_renyi(n, 0.3, 17), n)
+    rp, ci = _csr(ei, n)
+    a = np.zeros((n, n))
+    a[ei[0], ei[1]] = 1.0
+    xi = rng.integers(0, 10, (n, d)).astype(np.float32)
+    xr = rng.standard_normal((n, d)).astype(np.float32)
+    val = rng.standard_normal(ci.shape[0]).astype(np.float32)
+    av = np.zeros((n, n)); av[ei[0][np.lexsort((ei[1], ei[0]))], ci] = val
+    in_order = orc.csr_spmm(rp, ci, val, xr)
+    for g in (2, 4, 8, 16, 32, 64):
+        assert np.array_equal(orc.csr_spmm(rp, ci, None, xi, groups=g).astype(np.float64), a @ xi.astype(np.float64))
+        got = orc.csr_spmm(rp, ci, val, xr, threads=2, groups=g)
+        assert orc.max_rel_err(got, in_order) <= 1e-6
+        assert orc.max_rel_err(got, av @ xr.astype(np.float64)) <= 1e-6
+        assert not np.array_equal(got, in_order)            # it IS another order
+    assert np.array_equal(orc.csr_spmm(rp, ci, val, xr, groups=1), in_order)
+    # one row (1e8, 1, -1e8, 1) times a column of ones, fp32:
+    #   in order          ((1e8 + 1) - 1e8) + 1 = (1e8 - 1e8) + 1           = 1
+    #   2 partial sums    (1e8 - 1e8) + (1 + 1)                             = 2
+    #   4 partial sums    (1e8 + 1) + (-1e8 + 1) = 1e8 + -1e8               = 0
+    #   8 partial sums    ((1e8 + 1) + (-1e8 + 1)) + ((0 + 0) + (0 + 0))    = 0
+    rp1 = np.array([0, 4], np.int32); c1 = np.array([0, 1, 2, 3], np.int32)
+    v1 = np.array([1e8, 1.0, -1e8, 1.0], np.float32)
+    ones = np.ones((4, 1), np.float32)
+    # the matrix is 1 x 4: the oracle takes the row count from crow
+    assert [float(orc.csr_spmm(rp1, c1, v1, ones, groups=g)[0, 0]) for g in (1, 2, 4, 8)] == [1.0, 2.0, 0.0, 0.0]
+    # six entries in 4 partial sums: sums 0 and 1 get two entries each, in order
+    #   p0 = 1e8 + 3 (= 1e8, 3 is below half an ulp of 8), p1 = 1 + 5 = 6, p2 = -1e8, p3 = 1
+    #   tree: (p0 + p1) + (p2 + p3) = (1e8 + 6 -> 1e8 + 8) + (-1e8 + 1 -> -1e8) = 8
+    rp2 = np.array([0, 6], np.int32); c2 = np.arange(6, dtype=np.int32)
+    v2 = np.array([1e8, 1.0, -1e8, 1.0, 3.0, 5.0], np.float32)
+    assert float(orc.csr_spmm(rp2, c2, v2, np.ones((6, 1), np.float32), groups=4)[0, 0]) == 8.0
