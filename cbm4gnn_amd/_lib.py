@@ -14,6 +14,8 @@ from .build import HIP_LIB, HOST_LIB
 CBM_OK = 0
 CBM_PROP_SCALE_ROOTS = 1
 CBM_SPMM_WORKSPACE_READY = 1
+CBM_ERR_SCRATCH = 7
+CBM_STATIC_SCRATCH_FLOATS = 32 * 1024 * 1024
 
 
 class CbmLibraryError(RuntimeError):
@@ -61,6 +63,7 @@ HIP_SYMBOLS = {
     "cbm_relayout_slabs_f32": (C.c_int, [_P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "csr_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_row_intersections_groups": (C.c_int, []),
     "cbm_row_intersections": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _P, _I64, _P, _P]),

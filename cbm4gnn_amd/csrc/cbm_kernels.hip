@@ -995,6 +995,40 @@ int validate_levels(const int32_t* lo, int32_t n_levels, int32_t n) {
     return CBM_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Static scratch of cbm_spmm_update_static_f32, the entry point that allocates nothing: the
+// slab-major copy of X lives in this array instead of a workspace the caller brings.  Every
+// device the library runs on holds its own copy of the array (CBM_STATIC_SCRATCH_FLOATS floats)
+// at its own address until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and copies get the per-device address looked up below.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[CBM_STATIC_SCRATCH_FLOATS];
+
+float* g_scratch_ptr[kMaxDevices];                         // device address of `scratch`, per device
+std::atomic<int> g_scratch_ready[kMaxDevices];             // zero-initialised
+std::mutex g_scratch_mutex;
+
+// Address of the CURRENT device's copy of `scratch`, looked up once per device.
+int static_scratch(float** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return CBM_ERR_LAUNCH;
+    if (dev < 0 || dev >= kMaxDevices) return CBM_ERR_UNSUPPORTED;
+    if (!g_scratch_ready[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ready[dev].load(std::memory_order_relaxed)) {
+            void* ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+                (void)hipGetLastError();
+                return CBM_ERR_LAUNCH;
+            }
+            g_scratch_ptr[dev] = static_cast<float*>(ptr);
+            g_scratch_ready[dev].store(1, std::memory_order_release);
+        }
+    }
+    *out = g_scratch_ptr[dev];
+    return CBM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1010,6 +1044,7 @@ const char* cbm_status_string(int status) {
         case CBM_ERR_LAUNCH: return "HIP launch failed";
         case CBM_ERR_INTERNAL: return "internal invariant failed";
         case CBM_ERR_UNSUPPORTED: return "not implemented in this build";
+        case CBM_ERR_SCRATCH: return "shape needs more scratch than the static array holds (CBM_STATIC_SCRATCH_FLOATS)";
         default: return "unknown status";
     }
 }
@@ -1135,6 +1170,24 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
     // children of the root were scaled by the SpMM epilogue already
     return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,
                              flags & ~CBM_PROP_SCALE_ROOTS, stream);
+}
+
+int cbm_spmm_update_static_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m,
+                               const float* coef, const int32_t* parent, const int32_t* row_sched,
+                               const int32_t* order, const int32_t* level_off_dev, const int32_t* level_off_host,
+                               int32_t n_levels, const float* X, float* Y, int32_t n, int32_t d, int64_t ldx,
+                               int64_t ldy, int32_t flags, void* stream) {
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (int rc = check_matrix(n, d, ldy)) return rc;
+    const int64_t need = cbm_spmm_workspace_floats(n, d, ldx, ldy, X, Y);
+    if (need > (int64_t)CBM_STATIC_SCRATCH_FLOATS) return CBM_ERR_SCRATCH;
+    float* ws = nullptr;                                  // need == 0: this shape gathers from X in place
+    if (need > 0)
+        if (int rc = static_scratch(&ws)) return rc;
+    // relayout_slabs overwrites every float of the copy it makes (padding columns included), so
+    // nothing of the previous call's contents has to be cleared.
+    return cbm_spmm_update_f32(rowptr, idx, nnz, m, coef, parent, row_sched, order, level_off_dev, level_off_host,
+                               n_levels, X, Y, ws, n, d, ldx, ldy, flags, stream);
 }
 
 }  // extern "C"

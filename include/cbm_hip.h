@@ -33,8 +33,13 @@ enum {
     CBM_ERR_SHAPE = 3,       /* size / stride / index out of the supported range   */
     CBM_ERR_LAUNCH = 4,      /* the HIP runtime rejected a launch                  */
     CBM_ERR_INTERNAL = 5,    /* an internal invariant failed                       */
-    CBM_ERR_UNSUPPORTED = 6  /* valid request this build does not implement        */
+    CBM_ERR_UNSUPPORTED = 6, /* valid request this build does not implement        */
+    CBM_ERR_SCRATCH = 7      /* the shape needs more scratch than the static array of
+                                cbm_spmm_update_static_f32 holds                     */
 };
+
+/* Floats of the per-device static scratch array of cbm_spmm_update_static_f32 (128 MiB). */
+#define CBM_STATIC_SCRATCH_FLOATS (32 * 1024 * 1024)
 
 /* flags of cbm_spmm_f32 / csr_spmm_f32 */
 enum {
@@ -225,6 +230,24 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int6
                         const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
                         const float* X_dev, float* Y_dev, float* workspace_dev, int32_t n, int32_t d,
                         int64_t ldx, int64_t ldy, int32_t flags, void* stream);
+
+/* cbm_spmm_update_f32 for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring the
+ * workspace of the slab-major copy of X either.  No counterpart in the reference.  Same arguments
+ * minus the workspace, same result bit for bit as cbm_spmm_update_f32 with a workspace of
+ * cbm_spmm_workspace_floats() floats: the copy goes to a static device array of
+ * CBM_STATIC_SCRATCH_FLOATS floats (128 MiB) that every device the library runs on holds until the
+ * process ends.  A shape whose copy needs more (n * 32 * ceil(d / 32) floats, slab count rounded up
+ * to 1, 2, 4 or 8 below 8) is rejected with CBM_ERR_SCRATCH and nothing is enqueued.  The call
+ * allocates and frees nothing, on host or device.  All calls on one device share that device's
+ * array: calls that may overlap in time on one device (different streams, different threads)
+ * race on it; serialise them.  The array keeps the previous call's contents; every float the
+ * gather reads is rewritten by the copy first. */
+int cbm_spmm_update_static_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz, const float* m_dev,
+                               const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
+                               const int32_t* order_dev, const int32_t* level_off_dev,
+                               const int32_t* level_off_host, int32_t n_levels, const float* X_dev, float* Y_dev,
+                               int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream);
 
 /* Row intersections for the builder on the GPU: appends to pairs[] every (i, j > i, s) with
  * s = |row_i ^ row_j| and 2 s > min(nnz_i, nnz_j) + alpha, in no particular order, and adds their
