@@ -7,17 +7,27 @@ A "step" is one CBM multiply  Y = A_hat X  (delta SpMM + tree propagation throug
 on fixed device buffers; the format is built once, outside the timed region, as in the
 reference's protocol (``benchmark/parallel/benchmark_spmm_cpu.py:119-151``: 50 timed calls on
 fixed x, y).  Default workload: the 100k-node Chung-Lu + cliques graph, GCN-normalised, alpha=16,
-feature width 256.  Prints ONE JSON line.
+feature width 256.  Prints ONE JSON line.  The default run also carries, in the same line,
 
-The ``cpu_baseline`` leg times the reference-style CPU path on the host cores of the same box:
-MKL ``mkl_sparse_s_mm`` (reached through torch's libtorch_cpu.so, handle re-created per call
-like the reference) followed by the OpenMP tree walk of the CPU oracle.
+  * ``gcn_epoch``        the 2-layer GCN forward + backward epoch on the 233k-node SBM (c4), with
+                         CBM aggregation and with the hand-written GPU CSR layers;
+  * ``other_workloads``  one compact row each for the duplication graph (c2, alpha 0 and 8), the
+                         4,096-node SBM (c1) and the dense-community graph with the deep chain (c5);
+  * ``cpu_baseline``     the reference-style CPU path on the host cores of the same box, all
+                         threads and one thread (``benchmark/sequential/benchmark_spmm_cpu.py:1-11``):
+                         MKL ``mkl_sparse_s_mm`` (reached through torch's libtorch_cpu.so, handle
+                         re-created per call like the reference) + the OpenMP tree walk of the oracle.
+
+``--only-multiply`` skips the two extra sections; ``--gcn`` and ``--sweep`` run one of them alone.
 """
 from __future__ import annotations
 
 import argparse
+import glob
+import hashlib
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -27,12 +37,39 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+KERNEL_SOURCE = os.path.join(ROOT, "cbm4gnn_amd", "csrc", "cbm_kernels.hip")
 
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `bench.py --probe` scaled by a plain copy of known size (FETCH_SIZE x 2.00, WRITE_SIZE
-# x 1.00 on this part); keyed by (workload, alpha, d).  Counters cannot be read from inside this
-# process, so a configuration that was not profiled reports null.
-MEASURED_TRAFFIC_BYTES = {("c3", 16, 256): 2.32e9 + 0.1024e9}
+
+def kernel_source_hash():
+    with open(KERNEL_SOURCE, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def measured_traffic(workload, alpha, d):
+    """HBM-side bytes per launch of the dominant kernel from the counter summaries under
+    ``profiles/``.  Counters cannot be read from inside this process; a summary records them as
+
+        traffic-record: workload=c3 alpha=16 d=256 kernel=<instantiation> fetch_bytes=.. write_bytes=.. kernels_sha256=..
+
+    where ``kernels_sha256`` is the hash of the kernel source the counters were taken on.  A record
+    taken on another version of the kernels is reported as stale and contributes no number."""
+    want = {"workload": workload, "alpha": str(alpha), "d": str(d)}
+    stale = None
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        with open(path) as f:
+            for line in f:
+                if "traffic-record:" not in line:
+                    continue
+                rec = dict(kv.split("=", 1) for kv in re.findall(r"\S+=\S+", line.split("traffic-record:", 1)[1]))
+                if any(rec.get(k) != v for k, v in want.items()):
+                    continue
+                src = {"file": os.path.relpath(path, ROOT), "kernel": rec.get("kernel"),
+                       "kernels_sha256": rec.get("kernels_sha256")}
+                if rec.get("kernels_sha256") != kernel_source_hash():
+                    stale = src
+                    continue
+                return float(rec["fetch_bytes"]) + float(rec["write_bytes"]), src, False
+    return None, stale, stale is not None
 
 
 def algorithmic_bytes(n, nnz, d, norm, tree_edges, levels, n_edges_a):
@@ -43,8 +80,13 @@ def algorithmic_bytes(n, nnz, d, norm, tree_edges, levels, n_edges_a):
     return b_spmm, b_prop, b_csr
 
 
+def compulsory_bytes(n, nnz, d):
+    """Lower bound: X read once, Y written once, every index once, three words per row."""
+    return 4 * d * 2 * n + 4 * (nnz + 3 * n)
+
+
 def time_gpu(fn, steps, warmup, torch):
-    """(mean ms per step over the bracketed loop, median ms of per-call events)."""
+    """(wall ms per step, ms per step over the event-bracketed loop, median ms of per-call events)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -62,13 +104,40 @@ def time_gpu(fn, steps, warmup, torch):
     return wall_ms, span_ms, statistics.median(per_call)
 
 
-def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
-    """Reference-style CPU CBM and CPU CSR multiplies on this host (MKL SpMM + OpenMP walk)."""
+def csr_of(edge_index, n, m=None):
+    """(rowptr int32, col int32, val fp32 or None, order) of the CSR of a COO list, NumPy."""
     import numpy as np
+    ei = edge_index
+    order = np.lexsort((ei[1], ei[0]))
+    rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int32)
+    col = np.ascontiguousarray(ei[1][order].astype(np.int32))
+    val = None
+    if m is not None:
+        val = (m[ei[0][order]] * m[col]).astype(np.float32)
+    return rp, col, val
+
+
+def cpu_rows_fp64(rp, col, val, x, rows):
+    """Rows ``rows`` of ``A_hat X`` in fp64 straight from the CSR arrays (SciPy): an anchor that
+    shares no code with the kernels, cheap enough for every workload."""
+    import numpy as np
+    import scipy.sparse as sp
+    cnt = (rp[rows + 1] - rp[rows]).astype(np.int64)
+    take = np.repeat(rp[rows].astype(np.int64), cnt) + (np.arange(int(cnt.sum())) - np.repeat(np.cumsum(cnt) - cnt, cnt))
+    sub = sp.csr_matrix((np.ones(take.shape[0]) if val is None else val[take].astype(np.float64), col[take],
+                         np.concatenate([[0], np.cumsum(cnt)])), shape=(rows.shape[0], x.shape[0]))
+    return sub @ x.astype(np.float64)
+
+
+def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
+    """Reference-style CPU CBM and CPU CSR multiplies on this host (MKL SpMM + OpenMP walk), with
+    all threads and with one thread."""
+    import numpy as np
+    import torch
     from oracle import cbm_oracle as orc
 
     n, d = x.shape
-    threads = orc.max_threads()
+    all_threads = orc.max_threads()
     ei = w.edge_index
     m = orc.col_multiplier(ei, n) if w.normalized else None
     col, sign = mat.columns()
@@ -77,63 +146,139 @@ def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
     rp = mat.rowptr.numpy()
     rb, re = np.ascontiguousarray(rp[:-1]), np.ascontiguousarray(rp[1:])
     mst_row, mst_col = mat.mst_row.numpy(), mat.mst_col.numpy()
-    order = np.lexsort((ei[1], ei[0]))
-    arp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int32)
+    arp, acol, aval = csr_of(ei, n, m)
+    if aval is None:
+        aval = np.ones(acol.shape[0], np.float32)
     arb, are = np.ascontiguousarray(arp[:-1]), np.ascontiguousarray(arp[1:])
-    acol = np.ascontiguousarray(ei[1][order].astype(np.int32))
-    aval = ((m[ei[0][order]] * m[acol]) if m is not None else np.ones(acol.shape[0])).astype(np.float32)
     y = np.empty((n, d), np.float32)
     use_mkl = orc.mkl() is not None
 
-    def spmm(b, e, c, v):
-        if use_mkl:
-            orc.mkl_csr_spmm(b, e, c, v, x, y)
-        else:
-            y[:] = orc.csr_spmm(np.concatenate([b, e[-1:]]), c, v, x, threads)
+    def legs(threads, budget, iters):
+        def spmm(b, e, c, v):
+            if use_mkl:
+                orc.mkl_csr_spmm(b, e, c, v, x, y)
+            else:
+                y[:] = orc.csr_spmm(np.concatenate([b, e[-1:]]), c, v, x, threads)
 
-    def cbm_call():
-        spmm(rb, re, col, val)
-        if m is None:
-            orc.update_plain(mst_row, mst_col, y, threads)
-        else:
-            orc.update_fused(mst_row, mst_col, m, y, threads)
+        def cbm_call():
+            spmm(rb, re, col, val)
+            if m is None:
+                orc.update_plain(mst_row, mst_col, y, threads)
+            else:
+                orc.update_fused(mst_row, mst_col, m, y, threads)
 
-    def csr_call():
-        spmm(arb, are, acol, aval)
+        def csr_call():
+            spmm(arb, are, acol, aval)
 
-    def run(fn):
-        fn()                                              # 1 warm-up, as the reference
-        ts = []
-        t_end = time.perf_counter() + budget_s / 2
-        while len(ts) < max_iters and time.perf_counter() < t_end:
-            t = time.perf_counter(); fn(); ts.append((time.perf_counter() - t) * 1e3)
-        return ts
+        def run(fn):
+            fn()                                              # 1 warm-up, as the reference
+            ts = []
+            t_end = time.perf_counter() + budget / 2
+            while len(ts) < iters and (not ts or time.perf_counter() < t_end):
+                t = time.perf_counter(); fn(); ts.append((time.perf_counter() - t) * 1e3)
+            return ts
 
-    t_cbm = run(cbm_call)
-    y_cbm = y.copy()
-    t_csr = run(csr_call)
+        t_cbm = run(cbm_call)
+        y_cbm = y.copy()
+        t_csr = run(csr_call)
+        return t_cbm, t_csr, y_cbm
+
+    t_cbm, t_csr, y_cbm = legs(all_threads, budget_s, max_iters)
+    torch.set_num_threads(1)                                  # OpenMP and MKL: the "sequential" protocol
+    try:
+        t_cbm1, t_csr1, _ = legs(1, budget_s / 2, 10)
+    finally:
+        torch.set_num_threads(all_threads)
     return {
         "cbm_ms_mean": statistics.mean(t_cbm), "cbm_ms_median": statistics.median(t_cbm),
         "csr_ms_mean": statistics.mean(t_csr), "csr_ms_median": statistics.median(t_csr),
-        "iters": [len(t_cbm), len(t_csr)], "threads": threads,
+        "cbm_ms_1t": statistics.mean(t_cbm1), "csr_ms_1t": statistics.mean(t_csr1),
+        "iters": [len(t_cbm), len(t_csr)], "iters_1t": [len(t_cbm1), len(t_csr1)], "threads": all_threads,
         "spmm": "mkl_sparse_s_mm via libtorch_cpu.so" if use_mkl else "hand OpenMP CSR SpMM (non-MKL stand-in)",
     }, y_cbm
 
 
-def gcn_epoch_bench(args):
-    """2-layer GCN forward + backward (cross-entropy) with CBM aggregation; prints one JSON line.
-    Model and protocol follow benchmark/parallel/benchmark_gcn_cpu.py:70-103 (3 warm-up + 10 timed
-    passes, one cbm_matrix shared by both layers), plus the backward pass the reference lacks."""
+def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=512):
+    """Build the format of workload ``w`` and time the CBM multiply and the GPU CSR baseline on the
+    same X.  Returns (row dict, handles for the caller that wants more)."""
     import numpy as np
-    import torch
+
+    from cbm4gnn_amd.cbm import _wants_workspace, cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
+
+    t0 = time.perf_counter()
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder,
+                     max_levels=args.max_levels)
+    t_build = time.perf_counter() - t0
+    n, nnz, n_edges = w.n, mat.nnz, mat.nnz_a
+    norm = int(w.normalized)
+    tree_edges = n - int(mat.level_off[1])
+    x = w.features(0, d)
+    xd = x.cuda()
+    yd = torch.empty_like(xd)
+    mat.to(xd.device)
+    step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
+    wall_ms, span_ms, med_ms = time_gpu(step, args.steps, args.warmup, torch)
+
+    # hand-written GPU CSR baseline on A_hat (explicit values when normalised), same row scheduling
+    m_np = mat.col_multiplier.numpy() if w.normalized else None
+    rp, col, val = csr_of(w.edge_index, n, m_np)
+    rp_d, col_d = torch.from_numpy(rp).cuda(), torch.from_numpy(col).cuda()
+    val_d = None if val is None else torch.from_numpy(val).cuda()
+    ycsr = torch.empty_like(xd)
+    csr_sched = schedule_rows(torch.from_numpy(rp)).to(xd.device)
+    _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp_d, col_d, val_d, xd, ycsr, csr_sched), args.steps, args.warmup, torch)
+    step()
+    torch.cuda.synchronize()
+    err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
+    # anchor that shares no code with the kernels: a sample of rows in fp64 from the edge list
+    rows = np.sort(np.random.default_rng(0).choice(n, size=min(sample_rows, n), replace=False))
+    want = cpu_rows_fp64(rp, col, val, x.numpy(), rows)
+    got = yd[torch.from_numpy(rows).cuda()].cpu().numpy().astype(np.float64)
+    err_vs_cpu_rows = float(np.abs(got - want).max() / np.abs(want).max())
+
+    b_spmm, b_prop, b_csr = algorithmic_bytes(n, nnz, d, norm, tree_edges, mat.n_levels, n_edges)
+    row = {
+        "workload": w.name, "alpha": alpha, "d": d, "nodes": n, "nnz_A": n_edges, "nnz_delta": nnz,
+        "compression_ratio": mat.compression_ratio(), "tree_levels": mat.n_levels, "tree_edges": tree_edges,
+        "cbm_ms": span_ms, "cbm_ms_median": med_ms, "gpu_csr_ms": csr_ms, "speedup_vs_gpu_csr": csr_ms / span_ms,
+        "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
+        "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
+        "max_rel_err_vs_gpu_csr": err_vs_csr, "max_rel_err_vs_cpu_fp64_rows": err_vs_cpu_rows,
+        "cpu_rows_checked": int(rows.shape[0]), "build_s": t_build,
+    }
+    extra = {"mat": mat, "x": x, "xd": xd, "yd": yd, "wall_ms": wall_ms, "span_ms": span_ms, "med_ms": med_ms,
+             "csr_ms": csr_ms, "b": (b_spmm, b_prop, b_csr), "t_build": t_build, "tree_edges": tree_edges}
+    if split_kernels:
+        # the dominant kernel alone (delta SpMM gather), same launch as inside the step; where the step
+        # first copies X slab-major, that copy is made once here and timed on its own
+        zd = torch.empty_like(xd)
+        ws = relayout_slabs(xd) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
+        relayout_ms = 0.0
+        if ws is not None:
+            _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd), args.steps, args.warmup, torch)
+        spmm_only = lambda: mat._run_spmm(xd, zd, use_m=w.normalized, scale_roots=w.normalized, workspace=ws,
+                                          workspace_ready=ws is not None)
+        _, spmm_ms, _ = time_gpu(spmm_only, args.steps, args.warmup, torch)
+        prop_ms = 0.0
+        if tree_edges:
+            _, prop_ms, _ = time_gpu(lambda: mat._run_propagate(zd, use_m=w.normalized), args.steps, args.warmup, torch)
+        extra.update(relayout_ms=relayout_ms, spmm_ms=spmm_ms, prop_ms=prop_ms, slab=ws is not None or d % 32 == 0)
+    return row, extra
+
+
+def gcn_epoch(args, torch, workload="c4"):
+    """2-layer GCN forward + backward (cross-entropy) with CBM aggregation.  Model and protocol
+    follow benchmark/parallel/benchmark_gcn_cpu.py:70-103 (warm-up + timed passes, one cbm_matrix
+    shared by both layers), plus the backward pass the reference lacks."""
+    import numpy as np
 
     from cbm4gnn_amd import graphs
     from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
 
     t0 = time.perf_counter()
-    w = graphs.workload(args.workload if args.workload != "c3" else "c4", scale=args.scale)
+    w = graphs.workload(workload, scale=args.scale)
     t_gen = time.perf_counter() - t0
-    alpha = args.alpha if args.alpha is not None else w.alphas[-1]
+    alpha = args.alpha if (args.alpha is not None and args.gcn) else w.alphas[-1]
     hidden, classes = 128, 41
     ei = torch.from_numpy(w.edge_index)
     t0 = time.perf_counter()
@@ -145,14 +290,18 @@ def gcn_epoch_bench(args):
     g = torch.Generator().manual_seed(0)
     x = torch.randn((n, w.d), generator=g).to(dev)
     labels = torch.randint(0, classes, (n,), generator=g).to(dev)
-    torch.manual_seed(0)
-    model = TwoLayerGCN(CBMGCNLayer(w.d, hidden, op), CBMGCNLayer(hidden, classes, op)).to(dev)
     m = op.col_multiplier
     vals = m[ei[0].long()] * m[ei[1].long()]
     fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, vals, dev)       # rows = targets, as the CBM operator
     bwd = fwd if op.is_symmetric else csr_operator(ei, n, vals, dev)
-    torch.manual_seed(0)
-    base = TwoLayerGCN(CSRGCNLayer(w.d, hidden, fwd, bwd), CSRGCNLayer(hidden, classes, fwd, bwd)).to(dev)
+
+    def make(kind):
+        torch.manual_seed(0)
+        if kind == "csr":
+            return TwoLayerGCN(CSRGCNLayer(w.d, hidden, fwd, bwd), CSRGCNLayer(hidden, classes, fwd, bwd)).to(dev)
+        fused = kind == "cbm_fused"
+        return TwoLayerGCN(CBMGCNLayer(w.d, hidden, op, fused=fused, relu=fused),
+                           CBMGCNLayer(hidden, classes, op, fused=fused), relu_between=not fused).to(dev)
 
     def epoch(net):
         net.zero_grad(set_to_none=True)
@@ -170,31 +319,47 @@ def gcn_epoch_bench(args):
             loss = epoch(net)
         b.record()
         torch.cuda.synchronize()
-        return a.elapsed_time(b) / args.steps, float(loss)
+        return a.elapsed_time(b) / args.steps, float(loss.detach())
 
-    ms_cbm, loss_cbm = run(model)
-    ms_csr, loss_csr = run(base)
+    nets = {k: make(k) for k in ("cbm_fused", "cbm_unfused", "csr")}
+    res = {k: run(v) for k, v in nets.items()}
     # aggregation alone: the 4 multiplies of an epoch (d = hidden and d = classes, forward and backward)
     agg = 0.0
+    per_width = {}
     for dd in (hidden, classes):
         h = torch.randn((n, dd), device=dev)
         o = torch.empty_like(h)
         _, t, _ = time_gpu(lambda: op._run_spmm_update(h, o, use_m=True), args.steps, args.warmup, torch)
+        per_width[str(dd)] = t
         agg += 2 * t
-    grad_err = max(float((p.grad - q.grad).abs().max() / q.grad.abs().max())
-                   for p, q in zip(model.parameters(), base.parameters()))
-    print(json.dumps({
-        "metric": "2-layer GCN epoch ms (forward + backward, CBM aggregation)", "value": ms_cbm, "unit": "ms",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_cbm, "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{w.name}: {w.note}", "nodes": n, "nnz_A": op.nnz_a, "nnz_delta": op.nnz,
-                   "alpha": alpha, "in": w.d, "hidden": hidden, "classes": classes, "tree_levels": op.n_levels,
-                   "scale": args.scale},
-        "compression_ratio": op.compression_ratio(), "gcn_epoch_ms_gpu_csr": ms_csr, "speedup_vs_gpu_csr": ms_csr / ms_cbm,
-        "aggregation_ms_per_epoch": agg, "aggregation_share": agg / ms_cbm,
-        "loss": loss_cbm, "loss_gpu_csr": loss_csr, "max_rel_weight_grad_diff_vs_gpu_csr": grad_err,
+    base = nets["csr"]
+    grad_err = {k: max(float((p.grad - q.grad).abs().max() / q.grad.abs().max())
+                       for p, q in zip(nets[k].parameters(), base.parameters())) for k in ("cbm_fused", "cbm_unfused")}
+    ms = res["cbm_fused"][0]
+    return {
+        "workload": f"{w.name}: {w.note}", "nodes": n, "nnz_A": op.nnz_a, "nnz_delta": op.nnz, "alpha": alpha,
+        "in": w.d, "hidden": hidden, "classes": classes, "tree_levels": op.n_levels, "scale": args.scale,
+        "steps": args.steps, "warmup": args.warmup,
+        "gcn_epoch_ms": ms, "gcn_epoch_ms_unfused_layers": res["cbm_unfused"][0], "gcn_epoch_ms_gpu_csr": res["csr"][0],
+        "speedup_vs_gpu_csr": res["csr"][0] / ms, "compression_ratio": op.compression_ratio(),
+        "aggregation_ms_per_epoch": agg, "aggregation_share": agg / ms, "multiply_ms_by_width": per_width,
+        "loss": res["cbm_fused"][1], "loss_unfused_layers": res["cbm_unfused"][1], "loss_gpu_csr": res["csr"][1],
+        "max_rel_weight_grad_diff_vs_gpu_csr": grad_err,
         "host_s": {"generate": t_gen, "build_format": t_build, "build_phases": op.build_seconds},
-    }))
+    }
+
+
+def gcn_epoch_bench(args):
+    import torch
+    r = gcn_epoch(args, torch, args.workload if args.workload != "c3" else "c4")
+    print(json.dumps({
+        "metric": "2-layer GCN epoch ms (forward + backward, CBM aggregation)", "value": r["gcn_epoch_ms"], "unit": "ms",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["gcn_epoch_ms"],
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {k: r[k] for k in ("workload", "nodes", "nnz_A", "nnz_delta", "alpha", "in", "hidden", "classes",
+                                     "tree_levels", "scale")},
+        **{k: v for k, v in r.items() if k not in ("workload", "nodes", "nnz_A", "nnz_delta", "alpha", "in", "hidden",
+                                                   "classes", "tree_levels", "scale", "steps", "warmup")}}))
 
 
 def alpha_sweep_bench(args):
@@ -213,13 +378,10 @@ def alpha_sweep_bench(args):
     ei = torch.from_numpy(w.edge_index)
     xd = w.features(0, d).cuda()
     yd = torch.empty_like(xd)
-    order = np.lexsort((w.edge_index[1], w.edge_index[0]))
-    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(w.edge_index[0], minlength=n))]).astype(np.int32)).cuda()
-    col = torch.from_numpy(w.edge_index[1][order].astype(np.int32)).cuda()
-    val = None
-    if w.normalized:
-        m = torch.bincount(ei[0].long(), minlength=n).float().pow(-0.5)
-        val = (m[torch.from_numpy(w.edge_index[0][order].astype(np.int64))] * m[torch.from_numpy(w.edge_index[1][order].astype(np.int64))]).cuda()
+    m_np = torch.bincount(ei[0].long(), minlength=n).float().pow(-0.5).numpy() if w.normalized else None
+    rp_np, col_np, val_np = csr_of(w.edge_index, n, m_np)
+    rp, col = torch.from_numpy(rp_np).cuda(), torch.from_numpy(col_np).cuda()
+    val = None if val_np is None else torch.from_numpy(val_np).cuda()
     ycsr = torch.empty_like(xd)
     sched = schedule_rows(rp).to(xd.device)
     _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp, col, val, xd, ycsr, sched), args.steps, args.warmup, torch)
@@ -237,10 +399,11 @@ def alpha_sweep_bench(args):
         tree_edges = n - int(mat.level_off[1])
         b_spmm, b_prop, b_csr = algorithmic_bytes(n, mat.nnz, d, int(w.normalized), tree_edges, mat.n_levels, mat.nnz_a)
         step(); torch.cuda.synchronize()
+        widths = np.diff(mat.level_off.numpy())
         rows.append({"alpha": alpha, "compression_ratio": mat.compression_ratio(), "nnz_delta": mat.nnz,
                      "tree_levels": mat.n_levels, "tree_edges": tree_edges,
-                     "level_widths": {"first": np.diff(mat.level_off.numpy())[:12].tolist(),
-                                      "histogram": {int(k): int(v) for k, v in zip(*np.unique(np.diff(mat.level_off.numpy()), return_counts=True))} if mat.n_levels <= 64 or True else None},
+                     "level_widths": {"first": widths[:12].tolist(),
+                                      "histogram": {int(k): int(v) for k, v in zip(*np.unique(widths, return_counts=True))}},
                      "cbm_ms": ms, "delta_spmm_ms": spmm_ms,
                      "propagate_ms": ms - spmm_ms, "cbm_GBps": (b_spmm + b_prop) / ms / 1e6,
                      "speedup_vs_gpu_csr": csr_ms / ms, "build_s": t_build, "build_phases": mat.build_seconds,
@@ -265,6 +428,8 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--only-multiply", action="store_true",
+                    help="skip the gcn_epoch and other_workloads sections of the default run")
     ap.add_argument("--max-levels", type=int, default=None,
                     help="depth limit of the arborescence (default: none, as the reference)")
     ap.add_argument("--builder", choices=("auto", "host", "gpu"), default="auto",
@@ -280,113 +445,108 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); "
                  "run with --gpus 1")
-    if args.gcn or args.sweep:
-        import torch
-        if not torch.cuda.is_available():
-            sys.exit("bench.py needs a HIP device")
-        return gcn_epoch_bench(args) if args.gcn else alpha_sweep_bench(args)
-
     import numpy as np
     import torch
 
-    from cbm4gnn_amd import graphs
-    from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
-
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device")
+    if args.gcn or args.sweep:
+        return gcn_epoch_bench(args) if args.gcn else alpha_sweep_bench(args)
+
+    from cbm4gnn_amd import graphs
+
     t0 = time.perf_counter()
     w = graphs.workload(args.workload, scale=args.scale)
     alpha = args.alpha if args.alpha is not None else w.alphas[-1]
     d = args.d or w.d
     t_gen = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder, max_levels=args.max_levels)
-    t_build = time.perf_counter() - t0
-    n, nnz, n_edges = w.n, mat.nnz, mat.nnz_a
-    norm = int(w.normalized)
-    tree_edges = n - int(mat.level_off[1])
-    x = w.features(0, d)
-    xd = x.cuda()
-    yd = torch.empty_like(xd)
-    mat.to(xd.device)
-
-    step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
     if args.probe:
+        from cbm4gnn_amd.cbm import cbm_matrix
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized,
+                         builder=args.builder, max_levels=args.max_levels)
+        xd = w.features(0, d).cuda()
+        yd = torch.empty_like(xd)
+        step = (lambda: mat.omp_mkl_csr_fused_spmm_update(xd, yd)) if w.normalized else (lambda: mat.omp_mkl_csr_spmm_update(xd, yd))
         for _ in range(3):
             step()
         torch.cuda.synchronize()
         for _ in range(3):
             yd.copy_(xd)                                   # reads and writes n*d*4 bytes each
         torch.cuda.synchronize()
-        print(f"probe: 3 multiplies, then 3 device copies of {xd.numel() * 4} bytes (read) + the same written")
+        print(f"probe: 3 multiplies, then 3 device copies of {xd.numel() * 4} bytes (read) + the same written; "
+              f"kernels_sha256={kernel_source_hash()}")
         return
-    wall_ms, span_ms, med_ms = time_gpu(step, args.steps, args.warmup, torch)
 
-    # the dominant kernel alone (delta SpMM gather), same launch as inside the step; where the step
-    # first copies X slab-major, that copy is made once here and timed on its own
-    zd = torch.empty_like(xd)
-    from cbm4gnn_amd.cbm import _wants_workspace
-    ws = relayout_slabs(xd) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
-    relayout_ms = 0.0
-    if ws is not None:
-        _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd), args.steps, args.warmup, torch)
-    spmm_only = lambda: mat._run_spmm(xd, zd, use_m=w.normalized, scale_roots=w.normalized, workspace=ws,
-                                      workspace_ready=ws is not None)
-    _, spmm_ms, _ = time_gpu(spmm_only, args.steps, args.warmup, torch)
-    prop_ms = 0.0
-    if tree_edges:
-        prop_only = lambda: mat._run_propagate(zd, use_m=w.normalized)
-        _, prop_ms, _ = time_gpu(prop_only, args.steps, args.warmup, torch)
-
-    # hand-written GPU CSR baseline on A_hat (explicit values when normalised)
-    ei = w.edge_index
-    order = np.lexsort((ei[1], ei[0]))
-    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int32)).cuda()
-    col = torch.from_numpy(ei[1][order].astype(np.int32)).cuda()
-    val = None
-    if w.normalized:
-        m = mat.col_multiplier
-        val = (m[torch.from_numpy(ei[0][order].astype(np.int64))] * m[torch.from_numpy(ei[1][order].astype(np.int64))]).cuda()
-    ycsr = torch.empty_like(xd)
-    csr_sched = schedule_rows(rp).to(xd.device)          # the baseline gets the same row scheduling
-    _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp, col, val, xd, ycsr, csr_sched), args.steps, args.warmup, torch)
-    step()
-    torch.cuda.synchronize()
-    err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
-
-    b_spmm, b_prop, b_csr = algorithmic_bytes(n, nnz, d, norm, tree_edges, mat.n_levels, n_edges)
+    row, ex = measure_multiply(w, alpha, d, args, torch, split_kernels=True)
+    mat = ex["mat"]
+    n, nnz, n_edges = w.n, mat.nnz, mat.nnz_a
+    b_spmm, b_prop, b_csr = ex["b"]
+    span_ms, spmm_ms = ex["span_ms"], ex["spmm_ms"]
     achieved = b_spmm / (spmm_ms * 1e-3) / 1e9
+    traffic, traffic_src, traffic_stale = (measured_traffic(w.name, alpha, d) if args.scale == 1.0 else (None, None, False))
+    b_min = compulsory_bytes(n, nnz, d)
+    note = ""
+    if w.name == "c2":
+        note = (" [deviation: the stated duplication process yields 1.82 M undirected edges at N = 12 000, "
+                "not the ~240 k of the configuration text]")
     out = {
         "metric": "CBM SpMM ms at d=%d" % d,
         "value": span_ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": span_ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{w.name}: {w.note}", "nodes": n, "nnz_A": n_edges, "nnz_delta": nnz, "d": d,
+        "config": {"workload": f"{w.name}: {w.note}{note}", "nodes": n, "nnz_A": n_edges, "nnz_delta": nnz, "d": d,
                    "alpha": alpha, "normalized": bool(w.normalized), "tree_levels": mat.n_levels,
-                   "tree_edges": tree_edges, "scale": args.scale},
-        "ms_per_step_wall": wall_ms, "ms_per_step_median": med_ms,
+                   "tree_edges": ex["tree_edges"], "scale": args.scale},
+        "ms_per_step_wall": ex["wall_ms"], "ms_per_step_median": ex["med_ms"],
         "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
         "cbm_frac_of_8TBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
         "compression_ratio": mat.compression_ratio(),
-        "kernel_ms": {"relayout_slabs": relayout_ms, "delta_spmm": spmm_ms, "propagate": prop_ms},
-        "gpu_csr_ms": csr_ms, "gpu_csr_GBps": b_csr / (csr_ms * 1e-3) / 1e9, "speedup_vs_gpu_csr": csr_ms / span_ms,
-        "max_rel_err_vs_gpu_csr": err_vs_csr,
-        "roofline": {"bound": "hbm", "kernel": "spmm_slab_per_xcd" if (ws is not None or d % 32 == 0) else "spmm_wave_per_row", "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, alpha, d)) if args.scale == 1.0 else None,
-                     "algorithmic_bytes": b_spmm, "avg_launch_ms": spmm_ms},
-        "host_s": {"generate": t_gen, "build_format": t_build, "builder": mat.builder, "build_phases": mat.build_seconds},
+        "kernel_ms": {"relayout_slabs": ex["relayout_ms"], "delta_spmm": spmm_ms, "propagate": ex["prop_ms"]},
+        "gpu_csr_ms": ex["csr_ms"], "gpu_csr_GBps": b_csr / (ex["csr_ms"] * 1e-3) / 1e9,
+        "speedup_vs_gpu_csr": ex["csr_ms"] / span_ms,
+        "max_rel_err_vs_gpu_csr": row["max_rel_err_vs_gpu_csr"],
+        "max_rel_err_vs_cpu_fp64_rows": row["max_rel_err_vs_cpu_fp64_rows"],
+        # frac: algorithmic (gather-model, no reuse assumed) bytes over launch time -- it exceeds 1 where
+        # X rows are re-used out of L2 / the memory-side cache.  frac_traffic: counter-measured HBM-side
+        # bytes over the same launch time (what the memory system really moved).  frac_compulsory: the
+        # lower bound (X once, Y once, indices once) over the same time.
+        "roofline": {"bound": "hbm", "kernel": "spmm_slab_per_xcd" if ex["slab"] else "spmm_wave_per_row",
+                     "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": traffic,
+                     "frac_traffic": (traffic / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS) if traffic else None,
+                     "frac_compulsory": b_min / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic_source": traffic_src, "traffic_stale": traffic_stale,
+                     "kernels_sha256": kernel_source_hash(),
+                     "algorithmic_bytes": b_spmm, "compulsory_bytes": b_min, "avg_launch_ms": spmm_ms},
+        "host_s": {"generate": t_gen, "build_format": ex["t_build"], "builder": mat.builder, "build_phases": mat.build_seconds},
     }
     if not args.no_cpu:
-        cpu, y_cpu = cpu_baseline(w, mat, x.numpy())
+        cpu, y_cpu = cpu_baseline(w, mat, ex["x"].numpy())
         out["cpu_baseline"] = {
             "value": cpu["cbm_ms_mean"], "unit": "ms", "cores": cpu["threads"], "kind": "port",
-            "sample": f"{cpu['iters'][0]} full multiplies of the same workload after 1 warm-up ({cpu['spmm']} + OpenMP tree walk)",
+            "sample": f"{cpu['iters'][0]} full multiplies of the same workload after 1 warm-up ({cpu['spmm']} + OpenMP tree walk); "
+                      f"1-thread legs: {cpu['iters_1t'][0]} multiplies",
             "cbm_ms_median": cpu["cbm_ms_median"], "csr_ms_mean": cpu["csr_ms_mean"], "csr_ms_median": cpu["csr_ms_median"],
+            "cbm_ms_1t": cpu["cbm_ms_1t"], "csr_ms_1t": cpu["csr_ms_1t"],
         }
-        got = yd.cpu().numpy()
+        got = ex["yd"].cpu().numpy()
         out["max_rel_err_vs_cpu_cbm"] = float(np.abs(got - y_cpu).max() / np.abs(y_cpu).max())
+    if not args.only_multiply and args.workload == "c3" and args.scale == 1.0:
+        del ex, mat
+        torch.cuda.empty_cache()
+        others = []
+        short = argparse.Namespace(**{**vars(args), "steps": min(args.steps, 20), "warmup": min(args.warmup, 3)})
+        for name, alphas in (("c1", (0,)), ("c2", (0, 8)), ("c5", (0,))):
+            wk = graphs.workload(name)
+            for a in alphas:
+                r, e = measure_multiply(wk, a, wk.d, short, torch)
+                del e
+                others.append(r)
+            del wk
+            torch.cuda.empty_cache()
+        out["other_workloads"] = others
+        out["gcn_epoch"] = gcn_epoch(short, torch, "c4")
     print(json.dumps(out))
 
 

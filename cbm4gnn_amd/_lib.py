@@ -14,6 +14,9 @@ from .build import HIP_LIB, HOST_LIB
 CBM_OK = 0
 CBM_PROP_SCALE_ROOTS = 1
 CBM_SPMM_WORKSPACE_READY = 1
+CBM_SPMM_RELU = 2
+CBM_UPDATE_RELU = 2
+CBM_UPDATE_WORKSPACE_READY = 4
 CBM_ERR_SCRATCH = 7
 CBM_STATIC_SCRATCH_FLOATS = 32 * 1024 * 1024
 
@@ -61,6 +64,7 @@ HIP_SYMBOLS = {
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),
     "cbm_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_relayout_slabs_f32": (C.c_int, [_P, _P, _I32, _I32, _I64, _P]),
+    "cbm_relayout_slabs_masked_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),

@@ -551,7 +551,11 @@ class cbm_matrix:
         if back:
             y.copy_(yd)
 
-    def _run_spmm_update(self, x, y, use_m, flags=0):
+    def _run_spmm_update(self, x, y, use_m, flags=0, workspace=None, workspace_ready=False, relu=False):
+        """``y = A_hat x`` (``cbm_spmm_update_f32``).  ``workspace``: device scratch for the slab-major
+        copy of ``x`` (default: one from torch's caching allocator when the shape repays the copy);
+        ``workspace_ready``: it already holds that copy (``relayout_slabs``), ``x`` is not read;
+        ``relu``: ``y = max(A_hat x, 0)``."""
         n = self.num_rows
         _check_f32_matrix(x, "rhs", n)
         _check_f32_matrix(y, "dst", n)
@@ -567,7 +571,11 @@ class cbm_matrix:
         if yd.data_ptr() == xd.data_ptr():
             raise ValueError("dst must not alias rhs")
         st = self._device_arrays(xd.device)
-        ws = _workspace(xd, yd, self.nnz) if self.relayout else None
+        ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
+        if workspace_ready:
+            flags |= _lib.CBM_UPDATE_WORKSPACE_READY
+        if relu:
+            flags |= _lib.CBM_UPDATE_RELU
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
@@ -698,16 +706,27 @@ class CBMMatmul(torch.autograd.Function):
         return gx, None, None
 
 
-def relayout_slabs(x):
+def relayout_slabs(x, mask=None, out=None):
     """Slab-major copy of ``x`` for ``cbm_spmm_f32(..., CBM_SPMM_WORKSPACE_READY)`` (None for an
-    empty matrix)."""
+    empty matrix).  With ``mask`` (same shape) the copy holds ``x`` where ``mask > 0`` and zero
+    elsewhere (``cbm_relayout_slabs_masked_f32``: a ReLU gradient folded into the copy).  ``out``:
+    a float32 device tensor of at least ``cbm_relayout_floats(n, d)`` elements to reuse."""
     n, d = x.shape
     floats = _lib.hip_lib().cbm_relayout_floats(n, d)
     if floats <= 0:
         return None
-    ws = torch.empty(floats, dtype=torch.float32, device=x.device)
+    if out is not None and (out.numel() < floats or out.device != x.device or out.dtype != torch.float32):
+        raise ValueError("out is too small, on another device or not float32")
+    ws = out if out is not None else torch.empty(floats, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        rc = _lib.hip_lib().cbm_relayout_slabs_f32(_ptr(x), _ptr(ws), n, d, _ld(x), _stream(x.device))
+        if mask is None:
+            rc = _lib.hip_lib().cbm_relayout_slabs_f32(_ptr(x), _ptr(ws), n, d, _ld(x), _stream(x.device))
+        else:
+            _check_f32_matrix(mask, "mask", n)
+            if mask.size(1) != d or mask.device != x.device:
+                raise ValueError("mask must have the shape and device of x")
+            rc = _lib.hip_lib().cbm_relayout_slabs_masked_f32(_ptr(x), _ptr(mask), _ptr(ws), n, d, _ld(x), _ld(mask),
+                                                              _stream(x.device))
     _lib.check(rc, "cbm_relayout_slabs_f32")
     return ws
 

@@ -102,7 +102,7 @@ template <int VEC, int CH, bool PACKED, bool FULL>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
     const int32_t* __restrict__ rowptr, const uint32_t* __restrict__ idx, const float* __restrict__ val,
     const float* __restrict__ m, const int32_t* __restrict__ parent, const int4* __restrict__ sched,
-    const float* __restrict__ X, float* __restrict__ Z, int n, int d, int64_t ldx, int64_t ldz) {
+    const float* __restrict__ X, float* __restrict__ Z, int n, int d, int64_t ldx, int64_t ldz, int relu) {
     constexpr int U = (CH == 1) ? CBM_UNROLL_CH1 : (CH == 2 ? CBM_UNROLL_CH1 / 2 : CBM_UNROLL_CH1 / 4);   // X-row loads in flight per wave
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -187,7 +187,10 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_wave_per_row(
 #pragma unroll
     for (int c = 0; c < CH; c++)                   // 1.0f unless a child of the root (left scaling)
 #pragma unroll
-        for (int v = 0; v < VEC; v++) acc[c][v] *= root_scale;
+        for (int v = 0; v < VEC; v++) {
+            acc[c][v] *= root_scale;
+            if (relu) acc[c][v] = acc[c][v] < 0.0f ? 0.0f : acc[c][v];      // keeps NaN, as torch.relu does
+        }
     float* __restrict__ zr = Z + (int64_t)row * ldz + col0;
 #pragma unroll
     for (int c = 0; c < CH; c++)
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
     const float* __restrict__ X, float* __restrict__ Z, int n, int d, int vec_out, int n_slabs,
-    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz) {
+    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz, int relu) {
     // d is the true feature width: slabs may reach past it (odd widths are zero-padded in the
     // slab-major copy) and nothing is stored beyond column d; vec_out says that rows of Z are
     // float4-addressable.
@@ -332,7 +335,10 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
                 for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
             if (sub == 0) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[e] *= row_scale;      // 1.0f unless a child of the root
+                for (int e = 0; e < 4; e++) {
+                    acc[e] *= row_scale;                              // 1.0f unless a child of the root
+                    if (relu) acc[e] = acc[e] < 0.0f ? 0.0f : acc[e];  // keeps NaN, as torch.relu does
+                }
                 const int col = slab * kSlab + li * 4;
                 float* __restrict__ zr = Zs + (int64_t)row * ldz;
                 if (vec_out) {
@@ -352,9 +358,12 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 // power of two for the usual widths) apart, which maps them onto a fraction of an XCD's L2
 // channels, and rows of odd widths are not line-aligned at all; in the copy the lines of a slab
 // are consecutive and aligned.  One thread per float4 of the copy.
-template <bool VEC_IN>
+// With a mask matrix M (same shape as X, row stride ldm) the copy holds X where M > 0 and zero
+// elsewhere: the gradient of a ReLU applied to the incoming gradient in the pass that copies it.
+template <bool VEC_IN, bool MASKED>
 __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n, int d,
-                                                      int n_slabs, int64_t ldx) {
+                                                      int n_slabs, int64_t ldx, const float* __restrict__ M,
+                                                      int64_t ldm) {
     constexpr int kSlab4 = 8;                              // float4 per 128-byte slab
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int row4 = n_slabs * kSlab4;
@@ -371,6 +380,20 @@ __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ 
         if (col + 1 < d) v.y = src[1];
         if (col + 2 < d) v.z = src[2];
         if (col + 3 < d) v.w = src[3];
+    }
+    if constexpr (MASKED) {
+        const float* __restrict__ msk = M + (int64_t)r * ldm + col;
+        float4 k = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if constexpr (VEC_IN) {
+            if (col < d) k = *reinterpret_cast<const float4*>(msk);
+        } else {
+            if (col + 0 < d) k.x = msk[0];
+            if (col + 1 < d) k.y = msk[1];
+            if (col + 2 < d) k.z = msk[2];
+            if (col + 3 < d) k.w = msk[3];
+        }
+        v.x = k.x > 0.0f ? v.x : 0.0f; v.y = k.y > 0.0f ? v.y : 0.0f;
+        v.z = k.z > 0.0f ? v.z : 0.0f; v.w = k.w > 0.0f ? v.w : 0.0f;
     }
     *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * kSlab4 + w) * 4) = v;
 }
@@ -545,6 +568,17 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void scale_level0(
             for (int e = 0; e < VEC; e++) t[e] *= s;
             store_vec<VEC>(y + c * kWave * VEC, t);
         }
+}
+
+// Y = max(Y, 0) over an n x d matrix of row stride ldy: the ReLU of a multiply whose tree has more
+// than one level (there the SpMM epilogue cannot apply it: children still need their parent's
+// signed value).  One thread per element.
+__global__ __launch_bounds__(256) void relu_rows(float* __restrict__ Y, int64_t total, int d, int64_t ldy) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    float* __restrict__ y = Y + (t / d) * ldy + (t % d);
+    const float v = *y;
+    if (v < 0.0f) *y = 0.0f;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -842,15 +876,18 @@ inline int64_t matrix_bytes(int32_t n, int32_t d, int64_t ld) {
     return n > 0 && d > 0 ? ((int64_t)(n - 1) * ld + d) * 4 : 0;
 }
 
-inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s) {
+inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s,
+                           const float* mask = nullptr, int64_t ldm = 0) {
     const int ns = padded_slab_count(d);
     const int64_t blocks = ((int64_t)n * ns * 8 + 255) / 256;
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
     const dim3 grid((unsigned)blocks), block(256);
-    if (d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16))
-        hipLaunchKernelGGL(relayout_slabs<true>, grid, block, 0, s, X, workspace, n, d, ns, ldx);
-    else
-        hipLaunchKernelGGL(relayout_slabs<false>, grid, block, 0, s, X, workspace, n, d, ns, ldx);
+    const bool vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16) && (!mask || (ldm % 4 == 0 && aligned(mask, 16)));
+#define LAUNCH_RELAYOUT(V, K) \
+    hipLaunchKernelGGL((relayout_slabs<V, K>), grid, block, 0, s, X, workspace, n, d, ns, ldx, mask, ldm)
+    if (vec) { if (mask) LAUNCH_RELAYOUT(true, true); else LAUNCH_RELAYOUT(true, false); }
+    else { if (mask) LAUNCH_RELAYOUT(false, true); else LAUNCH_RELAYOUT(false, false); }
+#undef LAUNCH_RELAYOUT
     return CBM_OK;
 }
 
@@ -858,7 +895,8 @@ template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* val, const float* m,
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
-    if (flags & ~CBM_SPMM_WORKSPACE_READY) return CBM_ERR_UNSUPPORTED;
+    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU)) return CBM_ERR_UNSUPPORTED;
+    const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
     if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
@@ -902,7 +940,7 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
             const int vec_out = plan.vec_out ? 1 : 0;
 #define LAUNCH_SLAB(L, CF)                                                                                     \
     hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, CF, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, \
-                       val, m, parent, Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz)
+                       val, m, parent, Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz, relu)
             switch (lpe * 4 + coef_mode) {
                 case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream); break;
                 case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign); break;
@@ -920,7 +958,7 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
     const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
 #define LAUNCH(V, C, F)                                                                              \
     hipLaunchKernelGGL((spmm_wave_per_row<V, C, PACKED, F>), grid, block, 0, s, rowptr, idx, val, m, \
-                       parent, sc, X, Z, n, d, ldx, ldz)
+                       parent, sc, X, Z, n, d, ldx, ldz, relu)
     CBM_DISPATCH_TILING(t, LAUNCH);
 #undef LAUNCH
     return check_launch();
@@ -1067,6 +1105,21 @@ int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t 
     return check_launch();
 }
 
+int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, float* workspace, int32_t n, int32_t d, int64_t ldx,
+                                  int64_t ldm, void* stream) {
+    if (!X || !workspace || !mask) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (int rc = check_matrix(n, d, ldm)) return rc;
+    if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
+    const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+    if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
+        ranges_overlap(workspace, ws_bytes, mask, matrix_bytes(n, d, ldm)))
+        return CBM_ERR_SHAPE;
+    if (n == 0 || d == 0) return CBM_OK;
+    if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream), mask, ldm)) return rc;
+    return check_launch();
+}
+
 int64_t cbm_relayout_floats(int32_t n, int32_t d) {
     if (n <= 0 || d <= 0) return 0;
     return (int64_t)n * padded_slab_count(d) * 32;
@@ -1164,12 +1217,25 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, float* workspace,
                         int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY)) return CBM_ERR_UNSUPPORTED;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
-    int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, Y, workspace, 0, n, d, ldx, ldy, stream);
+    const bool relu = (flags & CBM_UPDATE_RELU) != 0;
+    // With a flat tree the SpMM's store is the final value of every row: the ReLU goes into its
+    // epilogue.  With deeper trees rows must keep their signed value for their children, so the
+    // ReLU is a pass of its own after the walk.
+    const bool flat = n_levels <= 1;
+    int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
+    if (relu && flat) spmm_flags |= CBM_SPMM_RELU;
+    int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, Y, workspace, spmm_flags, n, d, ldx, ldy,
+                          stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
-    return cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy,
-                             flags & ~CBM_PROP_SCALE_ROOTS, stream);
+    rc = cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, 0, stream);
+    if (rc || !relu || flat || n == 0 || d == 0) return rc;
+    const int64_t total = (int64_t)n * d, blocks = (total + 255) / 256;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    hipLaunchKernelGGL(relu_rows, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), Y, total, d, ldy);
+    return check_launch();
 }
 
 int cbm_spmm_update_static_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m,
@@ -1179,6 +1245,7 @@ int cbm_spmm_update_static_f32(const int32_t* rowptr, const uint32_t* idx, int64
                                int64_t ldy, int32_t flags, void* stream) {
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldy)) return rc;
+    if (flags & CBM_UPDATE_WORKSPACE_READY) return CBM_ERR_UNSUPPORTED;   // the scratch is not the caller's to fill
     const int64_t need = cbm_spmm_workspace_floats(n, d, ldx, ldy, X, Y);
     if (need > (int64_t)CBM_STATIC_SCRATCH_FLOATS) return CBM_ERR_SCRATCH;
     float* ws = nullptr;                                  // need == 0: this shape gathers from X in place

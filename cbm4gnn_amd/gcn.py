@@ -10,15 +10,30 @@ with a ReLU in between and shares one ``cbm_matrix`` between the layers
 dependency here, ``torch.nn.Linear`` with Xavier-uniform weights is the same layer.
 
 Unlike the reference's CBM layers, whose aggregation mutates a cached output behind autograd's
-back (so they have no usable backward), aggregation here is ``CBMMatmul``: backward is the same
+back (so they have no usable backward), aggregation here is differentiable: backward is the same
 CBM multiply with the transposed operator.
+
+``CBMGCNLayer(fused=True)`` (the default) runs the whole layer as one autograd function around
+the multiply:
+
+* the Linear output is written by the GEMM straight into a buffer whose row stride is d + 32
+  floats (an odd number of 128-byte lines), which the SpMM gathers in place -- no slab-major copy
+  of it is made (widths that are not 32, 64, 128 or 256 still take the copy);
+* the ReLU is applied in the multiply's store epilogue (``CBM_UPDATE_RELU``) and its gradient is
+  folded into the slab-major copy the backward multiply makes of the incoming gradient
+  (``cbm_relayout_slabs_masked_f32``), with the layer's own output as the mask;
+* the Linear output, the layer output, the workspace and the gradient buffer are allocated once
+  per layer and reused by every call, as the reference caches its output
+  (``cbm_message_passing.py:26-29``).  As there, the tensor a call returns is overwritten by the
+  next call of the same layer.
 """
 from __future__ import annotations
 
 import torch
 from torch import nn
 
-from .cbm import CBMMatmul, cbm_matrix, csr_spmm, schedule_rows
+from . import _lib
+from .cbm import CBMMatmul, _ld, _ptr, _wants_workspace, cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
 
 __all__ = ["CBMGCNLayer", "CSRGCNLayer", "TwoLayerGCN", "build_operator", "csr_operator", "CSRMatmul"]
 
@@ -32,16 +47,83 @@ def build_operator(edge_index, alpha: int = 2, normalized: bool = True, builder:
                       builder=builder)
 
 
+class _FusedGCNLayer(torch.autograd.Function):
+    """y = [relu](A_hat (x W^T)) on the layer's cached buffers; see the module docstring."""
+
+    @staticmethod
+    def forward(ctx, x, weight, layer):
+        op = layer.cached_a_t
+        xd = x.detach()
+        if xd.dtype != torch.float32:
+            raise RuntimeError("rhs tensor (NOT torch::kFloat32)")
+        n, d = xd.size(0), weight.size(0)
+        b = layer._layer_buffers(n, d, xd.device)
+        torch.mm(xd, weight.detach().t(), out=b["h"])
+        op._run_spmm_update(b["h"], b["y"], use_m=True, workspace=b["ws"] if b["copy_h"] else None, relu=layer.relu)
+        ctx.layer = layer
+        ctx.save_for_backward(xd, weight)
+        return b["y"].detach()                              # a fresh tensor object on the cached storage
+
+    @staticmethod
+    def backward(ctx, g):
+        layer = ctx.layer
+        x, weight = ctx.saved_tensors
+        op_t = layer.cached_a_t.transposed()
+        n, d = g.shape
+        b = layer._layer_buffers(n, d, g.device)
+        if g.stride(1) != 1 or (n > 1 and g.stride(0) < d):
+            g = g.contiguous()
+        if layer.relu:
+            # d relu: the copy the multiply gathers from holds g where the layer's output is positive
+            relayout_slabs(g, mask=b["y"], out=b["ws"])
+            op_t._run_spmm_update(g, b["gh"], use_m=True, workspace=b["ws"], workspace_ready=True)
+        else:
+            op_t._run_spmm_update(g, b["gh"], use_m=True, workspace=b["ws"] if b["copy_g"] else None)
+        gh = b["gh"]
+        gw = torch.mm(gh.t(), x) if ctx.needs_input_grad[1] else None
+        gx = torch.mm(gh, weight) if ctx.needs_input_grad[0] else None
+        return gx, gw, None
+
+
 class CBMGCNLayer(nn.Module):
-    def __init__(self, in_channels: int, out_channels: int, operator: cbm_matrix):
+    """``x -> [relu](A_hat (x W^T))``: the reference's GCN layer (``cbm_gcn.py:27-41``) with the
+    activation that follows it in the benchmark model optionally folded in (``relu=True``).
+    ``fused=False`` is the plain composition Linear -> ``CBMMatmul`` (-> ``relu``)."""
+
+    def __init__(self, in_channels: int, out_channels: int, operator: cbm_matrix, fused: bool = True, relu: bool = False):
         super().__init__()
         self.lin = nn.Linear(in_channels, out_channels, bias=False)
         nn.init.xavier_uniform_(self.lin.weight)            # 'glorot'
         self.cached_a_t = operator
+        self.fused, self.relu = bool(fused), bool(relu)
+        self._cache = None
+
+    def _layer_buffers(self, n, d, device):
+        """Device buffers of the layer for n rows of width d, allocated at the first call."""
+        key = (n, d, device)
+        if self._cache is not None and self._cache["key"] == key:
+            return self._cache
+        op = self.cached_a_t
+        lib = _lib.hip_lib()
+        y = torch.empty((n, d), dtype=torch.float32, device=device)
+        gh = torch.empty((n, d), dtype=torch.float32, device=device)
+        # Linear output with rows d + 32 floats apart when the library then gathers it in place
+        padded = torch.empty((n, d + 32), dtype=torch.float32, device=device)[:, :d]
+        in_place = d % 32 == 0 and lib.cbm_spmm_workspace_floats(n, d, _ld(padded), _ld(y), _ptr(padded), _ptr(y)) == 0
+        h = padded if in_place else torch.empty((n, d), dtype=torch.float32, device=device)
+        copy_h = (not in_place) and op.relayout and _wants_workspace(h, y, op.nnz)
+        copy_g = op.relayout and _wants_workspace(gh, y, op.transposed().nnz)
+        floats = int(lib.cbm_relayout_floats(n, d))
+        ws = torch.empty(max(floats, 1), dtype=torch.float32, device=device) if (copy_h or copy_g or self.relu) else None
+        self._cache = {"key": key, "h": h, "y": y, "gh": gh, "ws": ws, "copy_h": copy_h, "copy_g": copy_g,
+                       "h_in_place": in_place}
+        return self._cache
 
     def forward(self, x, edge_index=None):
-        x = self.lin(x)
-        return CBMMatmul.apply(x, self.cached_a_t, self.cached_a_t.col_multiplier is not None)
+        if self.fused and x.is_cuda:
+            return _FusedGCNLayer.apply(x, self.lin.weight, self)
+        y = CBMMatmul.apply(self.lin(x), self.cached_a_t, self.cached_a_t.col_multiplier is not None)
+        return y.relu() if self.relu else y
 
 
 class CSRMatmul(torch.autograd.Function):
@@ -91,11 +173,14 @@ class CSRGCNLayer(nn.Module):
 
 
 class TwoLayerGCN(nn.Module):
-    """first layer -> ReLU -> last layer (``benchmark_gcn_cpu.py:70-89`` with num_layers = 2)."""
+    """first layer -> ReLU -> last layer (``benchmark_gcn_cpu.py:70-89`` with num_layers = 2).
+    ``relu_between=False`` when the first layer applies the ReLU itself."""
 
-    def __init__(self, first: nn.Module, last: nn.Module):
+    def __init__(self, first: nn.Module, last: nn.Module, relu_between: bool = True):
         super().__init__()
         self.first_layer, self.last_layer = first, last
+        self.relu_between = bool(relu_between)
 
     def forward(self, x, edge_index=None):
-        return self.last_layer(self.first_layer(x, edge_index).relu(), edge_index)
+        h = self.first_layer(x, edge_index)
+        return self.last_layer(h.relu() if self.relu_between else h, edge_index)

@@ -43,12 +43,23 @@ enum {
 
 /* flags of cbm_spmm_f32 / csr_spmm_f32 */
 enum {
-    CBM_SPMM_WORKSPACE_READY = 1 /* workspace already holds cbm_relayout_slabs_f32(X): do not copy again */
+    CBM_SPMM_WORKSPACE_READY = 1, /* workspace already holds cbm_relayout_slabs_f32(X): do not copy again */
+    CBM_SPMM_RELU = 2             /* store max(z, 0) instead of z (after the left scale of root children) */
 };
 
-/* flags of cbm_propagate_f32 / cbm_spmm_update_f32 */
+/* flags of cbm_propagate_f32 */
 enum {
     CBM_PROP_SCALE_ROOTS = 1  /* normalised only: first do Y[r,:] *= m[r] for children of the root */
+};
+
+/* flags of cbm_spmm_update_f32 / cbm_spmm_update_static_f32 (CBM_PROP_SCALE_ROOTS is accepted and
+ * has no effect there: the SpMM epilogue scales the children of the root) */
+enum {
+    CBM_UPDATE_RELU = 2,            /* Y = max(A_hat X, 0): the activation of a GCN layer
+                                       (benchmark/parallel/benchmark_gcn_cpu.py:84-88 applies it as a
+                                       separate pass); in the SpMM epilogue when the tree is flat,
+                                       one extra pass over Y otherwise */
+    CBM_UPDATE_WORKSPACE_READY = 4  /* as CBM_SPMM_WORKSPACE_READY */
 };
 
 /* The CBM format as built on the host.  All arrays are malloc'd by cbm_build_host and are
@@ -204,6 +215,14 @@ int cbm_spmm_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz
  * Any width; workspace holds cbm_relayout_floats(n, d) floats. */
 int cbm_relayout_slabs_f32(const float* X_dev, float* workspace_dev, int32_t n, int32_t d, int64_t ldx, void* stream);
 int64_t cbm_relayout_floats(int32_t n, int32_t d);
+
+/* The same copy with a ReLU gradient folded in: the copy holds X[r][c] where mask[r][c] > 0 and 0
+ * elsewhere (mask: n x d, row stride ldm; typically the output of the forward multiply made with
+ * CBM_UPDATE_RELU, X the gradient arriving at it).  The backward multiply then runs from the copy
+ * with WORKSPACE_READY and never reads X.  No reference counterpart: the reference's layers have
+ * no backward pass (gnns/message_passing/cbm_message_passing.py:16-60 mutate a cached output). */
+int cbm_relayout_slabs_masked_f32(const float* X_dev, const float* mask_dev, float* workspace_dev, int32_t n, int32_t d,
+                                  int64_t ldx, int64_t ldm, void* stream);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
  *   m == NULL : Y[v,:] += Y[parent[v],:]

@@ -117,26 +117,155 @@ def test_alpha_sweep_graph_full_size_deep_chain_exact():
     assert torch.equal(ya, yb)
 
 
-def test_gcn_graph_full_size_against_gpu_csr():
-    """232,965 nodes, 114 M non-zeros (the GCN epoch workload), normalised, d = 128 and d = 41."""
+def _csr(ei, n):
+    order = np.lexsort((ei[1], ei[0]))
+    rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int64)
+    return rp, np.ascontiguousarray(ei[1][order].astype(np.int32))
+
+
+def _rows_fp64(rp, col, m, x, rows, transposed_scale=None):
+    """Rows ``rows`` of diag(m) A diag(m) X (m None: A X) in fp64 with SciPy, straight from the CSR
+    arrays of the edge list: an anchor that shares no code with the kernels or the oracle."""
+    import scipy.sparse as sp
+    cnt = rp[rows + 1] - rp[rows]
+    take = np.repeat(rp[rows], cnt) + (np.arange(int(cnt.sum())) - np.repeat(np.cumsum(cnt) - cnt, cnt))
+    c = col[take]
+    v = np.ones(take.shape[0]) if m is None else (np.repeat(m[rows].astype(np.float64), cnt) * m[c].astype(np.float64))
+    sub = sp.csr_matrix((v, c, np.concatenate([[0], np.cumsum(cnt)])), shape=(rows.shape[0], x.shape[0]))
+    return sub @ x.astype(np.float64)
+
+
+def _max_rel(got, want):
+    return float(np.abs(got - want).max() / np.abs(want).max())
+
+
+@pytest.fixture(scope="module")
+def c4():
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     w = graphs.workload("c4")
     print("[gpu-case] c4 full size, building", flush=True); sys.stdout.flush()
-    ei = torch.from_numpy(w.edge_index)
-    mat = cbm_matrix(ei, None, alpha=2, normalized=True)
-    m = mat.col_multiplier
-    order = np.lexsort((w.edge_index[1], w.edge_index[0]))
-    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(w.edge_index[0], minlength=w.n))]).astype(np.int32)).cuda()
-    col = torch.from_numpy(w.edge_index[1][order].astype(np.int32)).cuda()
-    val = (m[torch.from_numpy(w.edge_index[0][order].astype(np.int64))] * m[torch.from_numpy(w.edge_index[1][order].astype(np.int64))]).cuda()
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=2, normalized=True)
+    rp, col = _csr(w.edge_index, w.n)
+    return w, mat, rp, col
+
+
+def test_gcn_graph_full_size_against_cpu_rows_and_gpu_csr(c4):
+    """232,965 nodes, 114 M non-zeros (the GCN epoch workload), normalised, d = 128 and d = 41:
+    2,048 random rows of the product against an fp64 SciPy product built from the edge list, and
+    the whole product against the GPU CSR baseline."""
+    w, mat, rp, col = c4
+    m = mat.col_multiplier.numpy()
+    val = torch.from_numpy((np.repeat(m, np.diff(rp)) * m[col]).astype(np.float32)).cuda()
+    rp_d, col_d = torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda()
+    rows = np.sort(np.random.default_rng(4).choice(w.n, size=2048, replace=False))
+    rows_d = torch.from_numpy(rows).cuda()
     for d in (128, 41):
         print("[gpu-case] c4 full size, d", d, flush=True); sys.stdout.flush()
-        x = torch.randn((w.n, d), generator=torch.Generator().manual_seed(d)).cuda()
-        want = torch.empty_like(x)
-        csr_spmm(rp, col, val, x, want)
-        got = _mul(mat, x)
-        assert float((got - want).abs().max() / want.abs().max()) <= 1e-3
-        ones = _mul(mat, torch.ones_like(x))
-        # rows of D^-1/2 (A+I) D^-1/2 applied to the all-ones vector: sum_j m_i m_j over neighbours, < sqrt(deg_i) * max m
+        x = torch.randn((w.n, d), generator=torch.Generator().manual_seed(d))
+        xd = x.cuda()
+        got = _mul(mat, xd)
+        want_rows = _rows_fp64(rp, col, m, x.numpy(), rows)
+        assert _max_rel(got[rows_d].cpu().numpy().astype(np.float64), want_rows) <= 1e-4
+        base = torch.empty_like(xd)
+        csr_spmm(rp_d, col_d, val, xd, base)
+        assert _max_rel(base[rows_d].cpu().numpy().astype(np.float64), want_rows) <= 1e-4
+        assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+        ones = _mul(mat, torch.ones_like(xd))
         assert float(ones.min()) > 0.0 and torch.isfinite(ones).all()
+
+
+def test_gcn_epoch_full_size_anchored_rows(c4):
+    """One full-size forward + backward of the 2-layer GCN (602-128-41) with the fused CBM layers:
+    loss and weight gradients against the CSR-layer model, and every aggregation of the epoch --
+    both forward multiplies and both backward multiplies, on the inputs they really had -- against
+    2,048 fp64 rows computed with SciPy from the edge list."""
+    from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, csr_operator
+    w, mat, rp, col = c4
+    n, hidden, classes = w.n, 128, 41
+    dev = torch.device("cuda")
+    m = mat.col_multiplier.numpy()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((n, w.d), generator=g).to(dev)
+    labels = torch.randint(0, classes, (n,), generator=g).to(dev)
+    torch.manual_seed(0)
+    model = TwoLayerGCN(CBMGCNLayer(w.d, hidden, mat, relu=True), CBMGCNLayer(hidden, classes, mat), relu_between=False).to(dev)
+    print("[gpu-case] c4 full size gcn epoch, fused layers", flush=True); sys.stdout.flush()
+    logits = model(x)
+    loss = torch.nn.functional.cross_entropy(logits, labels)
+    loss.backward()
+    torch.cuda.synchronize()
+    rows = np.sort(np.random.default_rng(6).choice(n, size=2048, replace=False))
+    rows_d = torch.from_numpy(rows).to(dev)
+    b1, b2 = model.first_layer._cache, model.last_layer._cache
+    cpu = lambda t: t.detach().cpu().numpy()
+    # forward, layer 1: y1 = relu(A_hat h1)
+    want = np.maximum(_rows_fp64(rp, col, m, cpu(b1["h"]), rows), 0.0)
+    assert _max_rel(cpu(b1["y"][rows_d]).astype(np.float64), want) <= 1e-4
+    # forward, layer 2: logits = A_hat h2
+    want = _rows_fp64(rp, col, m, cpu(b2["h"]), rows)
+    assert _max_rel(cpu(logits[rows_d]).astype(np.float64), want) <= 1e-4
+    # backward, layer 2: gh2 = A_hat^T g_logits (the graph is symmetric), g_logits = (softmax - onehot) / n
+    g_logits = torch.softmax(logits.detach(), dim=1)
+    g_logits[torch.arange(n, device=dev), labels] -= 1.0
+    g_logits /= n
+    want = _rows_fp64(rp, col, m, cpu(g_logits), rows)
+    assert _max_rel(cpu(b2["gh"][rows_d]).astype(np.float64), want) <= 1e-4
+    # backward, layer 1: gh1 = A_hat^T (relu'(y1) * (gh2 W2))
+    g_y1 = (b2["gh"] @ model.last_layer.lin.weight.detach()) * (b1["y"] > 0)
+    want = _rows_fp64(rp, col, m, cpu(g_y1), rows)
+    assert _max_rel(cpu(b1["gh"][rows_d]).astype(np.float64), want) <= 1e-4
+    # the CSR-layer model: same loss, same weight gradients
+    print("[gpu-case] c4 full size gcn epoch, csr layers", flush=True); sys.stdout.flush()
+    ei = torch.from_numpy(w.edge_index)
+    mt = mat.col_multiplier
+    fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, mt[ei[0].long()] * mt[ei[1].long()], dev)
+    torch.manual_seed(0)
+    base = TwoLayerGCN(CSRGCNLayer(w.d, hidden, fwd, fwd), CSRGCNLayer(hidden, classes, fwd, fwd)).to(dev)
+    base_loss = torch.nn.functional.cross_entropy(base(x), labels)
+    base_loss.backward()
+    assert abs(float(loss.detach()) - float(base_loss.detach())) <= 1e-5 * abs(float(base_loss.detach()))
+    for p, q in zip(model.parameters(), base.parameters()):
+        assert float((p.grad - q.grad).abs().max() / q.grad.abs().max()) <= 1e-3
+
+
+def test_duplication_graph_full_size():
+    """12,000-node duplication graph at full size (3.64 M non-zeros, A + I normalised, d = 128),
+    alpha 0 and 8: 1,024 rows against fp64 SciPy rows, everything against the GPU CSR baseline."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c2")
+    rp, col = _csr(w.edge_index, w.n)
+    x = w.features(0)
+    xd = x.cuda()
+    rows = np.sort(np.random.default_rng(2).choice(w.n, size=1024, replace=False))
+    rows_d = torch.from_numpy(rows).cuda()
+    for alpha in (0, 8):
+        print("[gpu-case] c2 full size alpha", alpha, flush=True); sys.stdout.flush()
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=True)
+        assert mat.n_levels > 4 and mat.compression_ratio() > 1.4
+        m = mat.col_multiplier.numpy()
+        got = _mul(mat, xd)
+        want_rows = _rows_fp64(rp, col, m, x.numpy(), rows)
+        assert _max_rel(got[rows_d].cpu().numpy().astype(np.float64), want_rows) <= 1e-4
+        val = torch.from_numpy((np.repeat(m, np.diff(rp)) * m[col]).astype(np.float32)).cuda()
+        base = torch.empty_like(xd)
+        csr_spmm(torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda(), val, xd, base)
+        assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+
+
+def test_alpha_sweep_graph_same_format_for_every_alpha():
+    """On the dense-community graph alpha <= 32 prunes nothing (every admissible pair clears the
+    threshold by far more): the builder must return the arrays of alpha = 0 for the whole sweep."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c5")
+    ei = torch.from_numpy(w.edge_index)
+    print("[gpu-case] c5 alpha 0", flush=True); sys.stdout.flush()
+    ref = cbm_matrix(ei, None, alpha=0)
+    for alpha in (2, 4, 8, 16, 32):
+        print("[gpu-case] c5 alpha", alpha, flush=True); sys.stdout.flush()
+        mat = cbm_matrix(ei, None, alpha=alpha)
+        assert mat.nnz == ref.nnz and mat.n_levels == ref.n_levels
+        for name in ("rowptr", "idx", "parent", "order", "level_off"):
+            assert torch.equal(getattr(mat, name), getattr(ref, name)), (alpha, name)

@@ -366,40 +366,93 @@ def test_c_abi_status_codes_on_device_calls():
     assert int(cnt) == 0 and int(tick) >= n
 
 
-def test_two_layer_gcn_forward_backward_matches_dense(orc):
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("alpha,directed", [(2, False), (10_000, False), (2, True)])
+def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directed):
     """The GCN epoch harness (Linear -> CBM aggregate -> ReLU -> Linear -> CBM aggregate, cross
-    entropy) against the same model written with a dense normalised adjacency in torch."""
+    entropy) against the same model written with a dense normalised adjacency in torch fp64.
+    ``fused``: the layer as one autograd function (Linear output gathered in place from a padded
+    buffer, ReLU in the multiply's epilogue -- alpha = 10 000 gives the flat tree where it is
+    the SpMM's epilogue, alpha = 2 a deeper tree where it is a pass after the walk -- and its
+    gradient folded into the slab-major copy of the backward multiply); ``directed``: the backward
+    multiply runs on the transposed operator."""
     from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
     n, f_in, hidden, classes = 300, 37, 128, 41
     ei_np = graphs.add_self_loops(graphs.sbm(n, 6, 0.3, 0.02, seed=11), n)
+    if directed:
+        keep = (np.random.default_rng(5).random(ei_np.shape[1]) > 0.3) | (ei_np[0] == ei_np[1])
+        ei_np = np.ascontiguousarray(ei_np[:, keep])
     ei = torch.from_numpy(ei_np)
-    say("gcn harness")
-    op = build_operator(ei, alpha=2, normalized=True)
-    assert op.n_levels >= 2
+    say("gcn harness", fused, alpha, directed)
+    op = build_operator(ei, alpha=alpha, normalized=True)
+    assert (op.n_levels == 1) == (alpha == 10_000) and op.is_symmetric == (not directed)
     torch.manual_seed(1)
-    model = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op), CBMGCNLayer(hidden, classes, op)).cuda()
+    model = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op, fused=fused, relu=fused),
+                        CBMGCNLayer(hidden, classes, op, fused=fused), relu_between=not fused).cuda()
     x = torch.randn((n, f_in), generator=torch.Generator().manual_seed(2)).cuda()
     y = torch.randint(0, classes, (n,), generator=torch.Generator().manual_seed(3)).cuda()
-    loss = torch.nn.functional.cross_entropy(model(x), y)
-    loss.backward()
     a = torch.from_numpy(orc.dense_adjacency(np.stack([ei_np[1], ei_np[0]]), n)).double().cuda()
     m = a.sum(dim=1).pow(-0.5)
     a_hat = m[:, None] * a * m[None, :]
-    w1 = model.first_layer.lin.weight.detach().double().requires_grad_(True)
-    w2 = model.last_layer.lin.weight.detach().double().requires_grad_(True)
-    ref = a_hat @ ((a_hat @ (x.double() @ w1.t())).relu() @ w2.t())
-    ref_loss = torch.nn.functional.cross_entropy(ref, y)
-    ref_loss.backward()
-    assert abs(float(loss) - float(ref_loss)) <= 1e-4 * abs(float(ref_loss))
-    for got, want in ((model.first_layer.lin.weight.grad, w1.grad), (model.last_layer.lin.weight.grad, w2.grad)):
-        assert float((got.double() - want).abs().max() / want.abs().max()) <= 1e-3
+    for epoch in range(2):                                  # the second pass runs on the cached buffers
+        model.zero_grad(set_to_none=True)
+        xin = x.clone().requires_grad_(True)
+        logits = model(xin)
+        loss = torch.nn.functional.cross_entropy(logits, y)
+        loss.backward()
+        w1 = model.first_layer.lin.weight.detach().double().requires_grad_(True)
+        w2 = model.last_layer.lin.weight.detach().double().requires_grad_(True)
+        xr = x.double().requires_grad_(True)
+        ref = a_hat @ ((a_hat @ (xr @ w1.t())).relu() @ w2.t())
+        ref_loss = torch.nn.functional.cross_entropy(ref, y)
+        ref_loss.backward()
+        assert float((logits.detach().double() - ref).abs().max() / ref.abs().max()) <= TOL_CBM
+        assert abs(float(loss.detach()) - float(ref_loss.detach())) <= 1e-4 * abs(float(ref_loss.detach()))
+        for got, want in ((model.first_layer.lin.weight.grad, w1.grad), (model.last_layer.lin.weight.grad, w2.grad),
+                          (xin.grad, xr.grad)):
+            assert float((got.double() - want).abs().max() / want.abs().max()) <= 1e-3
+    if fused:
+        b = model.first_layer._cache
+        assert b["h_in_place"] and b["h"].stride(0) == hidden + 32 and not b["copy_h"]    # gathered in place
+        assert float(b["y"].min()) == 0.0                                               # the ReLU was applied
+        assert not model.last_layer._cache["h_in_place"]                                # width 41 takes the copy
     # the CSR-baseline model computes the same thing
     vals = op.col_multiplier[ei[0].long()] * op.col_multiplier[ei[1].long()]
     fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, vals, x.device)
+    bwd = fwd if not directed else csr_operator(ei, n, vals, x.device)
     torch.manual_seed(1)
-    base = TwoLayerGCN(CSRGCNLayer(f_in, hidden, fwd, fwd), CSRGCNLayer(hidden, classes, fwd, fwd)).cuda()
+    base = TwoLayerGCN(CSRGCNLayer(f_in, hidden, fwd, bwd), CSRGCNLayer(hidden, classes, fwd, bwd)).cuda()
     base_loss = torch.nn.functional.cross_entropy(base(x), y)
-    assert abs(float(base_loss) - float(loss)) <= 1e-5 * abs(float(loss))
+    assert abs(float(base_loss.detach()) - float(loss.detach())) <= 1e-5 * abs(float(loss.detach()))
+
+
+def test_relu_epilogue_and_masked_copy_through_the_c_abi(orc):
+    """CBM_UPDATE_RELU on a flat and on a deeper tree equals max(multiply, 0) bit for bit, for
+    widths on both SpMM kernels; cbm_relayout_slabs_masked_f32 holds x where the mask is positive."""
+    from cbm4gnn_amd.cbm import relayout_slabs
+    n = 700
+    ei = graphs.add_self_loops(graphs.sbm(n, 10, 0.3, 0.01, seed=13), n)
+    for alpha in (1, 10_000):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=True)
+        for d in (41, 128, 200):
+            say("relu epilogue", alpha, d)
+            x = torch.randn((n, d), generator=torch.Generator().manual_seed(d)).cuda()
+            want = torch.empty_like(x); mat._run_spmm_update(x, want, use_m=True)
+            got = torch.full_like(x, float("nan")); mat._run_spmm_update(x, got, use_m=True, relu=True)
+            assert float(want.min()) < 0.0 and torch.equal(got, want.clamp_min(0.0))
+            mat.relayout = False                            # wave-per-row / row-major gather
+            got2 = torch.full_like(x, float("nan")); mat._run_spmm_update(x, got2, use_m=True, relu=True)
+            want2 = torch.empty_like(x); mat._run_spmm_update(x, want2, use_m=True)
+            assert torch.equal(got2, want2.clamp_min(0.0))
+            mat.relayout = True
+            mask = torch.randn((n, d), generator=torch.Generator().manual_seed(d + 1)).cuda()
+            ws = relayout_slabs(x, mask=mask)
+            assert torch.equal(ws, relayout_slabs(torch.where(mask > 0, x, torch.zeros_like(x))))
+            via_copy = torch.empty_like(x)
+            mat._run_spmm_update(torch.full_like(x, float("nan")), via_copy, use_m=True, workspace=ws, workspace_ready=True)
+            direct = torch.empty_like(x)
+            mat._run_spmm_update(torch.where(mask > 0, x, torch.zeros_like(x)), direct, use_m=True, workspace=torch.empty_like(ws))
+            assert torch.equal(via_copy, direct)
 
 
 def test_degenerate_shapes(orc):
