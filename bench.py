@@ -252,12 +252,14 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
         # the dominant kernel alone (delta SpMM gather), same launch as inside the step; where the step
         # first copies X slab-major, that copy is made once here and timed on its own
         zd = torch.empty_like(xd)
-        ws = relayout_slabs(xd) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
+        scale = mat._device_arrays(xd.device)["m"] if w.normalized else None     # the step scales its copy by m
+        ws = relayout_slabs(xd, scale=scale) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
         relayout_ms = 0.0
         if ws is not None:
-            _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd), args.steps, args.warmup, torch)
+            _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd, scale=scale, out=ws), args.steps, args.warmup, torch)
         spmm_only = lambda: mat._run_spmm(xd, zd, use_m=w.normalized, scale_roots=w.normalized, workspace=ws,
-                                          workspace_ready=ws is not None)
+                                          workspace_ready=ws is not None,
+                                          workspace_prescaled=ws is not None and scale is not None)
         _, spmm_ms, _ = time_gpu(spmm_only, args.steps, args.warmup, torch)
         prop_ms = 0.0
         if tree_edges:

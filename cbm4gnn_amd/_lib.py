@@ -17,6 +17,8 @@ CBM_SPMM_WORKSPACE_READY = 1
 CBM_SPMM_RELU = 2
 CBM_UPDATE_RELU = 2
 CBM_UPDATE_WORKSPACE_READY = 4
+CBM_SPMM_WORKSPACE_PRESCALED = 4
+CBM_UPDATE_WORKSPACE_PRESCALED = 8
 CBM_ERR_SCRATCH = 7
 CBM_STATIC_SCRATCH_FLOATS = 32 * 1024 * 1024
 
@@ -64,7 +66,8 @@ HIP_SYMBOLS = {
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),
     "cbm_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_relayout_slabs_f32": (C.c_int, [_P, _P, _I32, _I32, _I64, _P]),
-    "cbm_relayout_slabs_masked_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_relayout_slabs_masked_f32": (C.c_int, [_P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
+    "cbm_relayout_slabs_scaled_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),

@@ -473,16 +473,23 @@ class cbm_matrix:
                 "sched_scaled": (schedule_rows(self.rowptr, self.parent, self.col_multiplier).to(device)
                                  if self.col_multiplier is not None else None),
             }
-            if st["m"] is not None and self.nnz and self.stream_coefficients:
-                # +-m[col] per delta entry, expanded once on the device (what the reference keeps
-                # as the fp32 values of its delta matrix); streamed by the SpMM instead of a gather
-                st["coef"] = torch.empty(self.nnz, dtype=torch.float32, device=device)
-                with torch.cuda.device(device):
-                    rc = _lib.hip_lib().cbm_expand_coef_f32(_ptr(st["idx"]), _ptr(st["m"]), _ptr(st["coef"]),
-                                                            self.nnz, _stream(device))
-                _lib.check(rc, "cbm_expand_coef_f32")
             self._dev[key] = st
         return st
+
+    def _coef(self, st, device):
+        """``+-m[col]`` per delta entry on ``device`` (what the reference keeps as the fp32 values of
+        its delta matrix), expanded on first need: only a normalised multiply that gathers from
+        the caller's row-major X streams it -- one that copies X slab-major scales the copy by
+        ``m`` instead and needs no coefficient per entry.  None when ``stream_coefficients`` is off."""
+        if st["m"] is None or not self.nnz or not self.stream_coefficients:
+            return None
+        if st["coef"] is None:
+            st["coef"] = torch.empty(self.nnz, dtype=torch.float32, device=device)
+            with torch.cuda.device(device):
+                rc = _lib.hip_lib().cbm_expand_coef_f32(_ptr(st["idx"]), _ptr(st["m"]), _ptr(st["coef"]),
+                                                        self.nnz, _stream(device))
+            _lib.check(rc, "cbm_expand_coef_f32")
+        return st["coef"]
 
     def to(self, device):
         """Upload the format to ``device`` now (it is otherwise uploaded at the first multiply)."""
@@ -505,7 +512,7 @@ class cbm_matrix:
         return int(_lib.hip_lib().cbm_spmm_summation_groups(x.size(1), _ld(x), _ld(y), _ptr(x), _ptr(y), int(use_ws)))
 
     # ------------------------------------------------------------------ kernels -------------
-    def _run_spmm(self, x, y, use_m, scale_roots, workspace=None, workspace_ready=False):
+    def _run_spmm(self, x, y, use_m, scale_roots, workspace=None, workspace_ready=False, workspace_prescaled=False):
         n = self.num_rows
         _check_f32_matrix(x, "rhs", n)
         _check_f32_matrix(y, "dst", n)
@@ -520,13 +527,17 @@ class cbm_matrix:
             raise ValueError("rhs and dst are on different devices")
         st = self._device_arrays(xd.device)
         ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
+        # per-entry coefficients are only read when the multiply does not scale its own copy of X
+        coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
+        flags = (_lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0) | \
+                (_lib.CBM_SPMM_WORKSPACE_PRESCALED if workspace_prescaled else 0)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
-                _ptr(st["coef"]) if use_m else None,
+                _ptr(coef),
                 _ptr(st["parent"]) if scale_roots else None,
                 _ptr(st["sched_scaled"] if (scale_roots and use_m) else st["sched"]), _ptr(xd), _ptr(yd),
-                _ptr(ws), _lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0, n, x.size(1), _ld(xd), _ld(yd),
+                _ptr(ws), flags, n, x.size(1), _ld(xd), _ld(yd),
                 _stream(xd.device))
         _lib.check(rc, "cbm_spmm_f32")
         if yd is not y:
@@ -551,11 +562,12 @@ class cbm_matrix:
         if back:
             y.copy_(yd)
 
-    def _run_spmm_update(self, x, y, use_m, flags=0, workspace=None, workspace_ready=False, relu=False):
+    def _run_spmm_update(self, x, y, use_m, flags=0, workspace=None, workspace_ready=False, relu=False,
+                         workspace_prescaled=False):
         """``y = A_hat x`` (``cbm_spmm_update_f32``).  ``workspace``: device scratch for the slab-major
         copy of ``x`` (default: one from torch's caching allocator when the shape repays the copy);
         ``workspace_ready``: it already holds that copy (``relayout_slabs``), ``x`` is not read;
-        ``relu``: ``y = max(A_hat x, 0)``."""
+        ``workspace_prescaled``: that copy was made with ``scale=m``; ``relu``: ``y = max(A_hat x, 0)``."""
         n = self.num_rows
         _check_f32_matrix(x, "rhs", n)
         _check_f32_matrix(y, "dst", n)
@@ -574,12 +586,15 @@ class cbm_matrix:
         ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         if workspace_ready:
             flags |= _lib.CBM_UPDATE_WORKSPACE_READY
+        if workspace_prescaled:
+            flags |= _lib.CBM_UPDATE_WORKSPACE_PRESCALED
         if relu:
             flags |= _lib.CBM_UPDATE_RELU
+        coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
-                _ptr(st["coef"]) if use_m else None, _ptr(st["parent"]),
+                _ptr(coef), _ptr(st["parent"]),
                 _ptr(st["sched_scaled"] if use_m else st["sched"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels,
                 _ptr(xd), _ptr(yd), _ptr(ws), n, x.size(1), _ld(xd), _ld(yd), flags, _stream(xd.device))
         _lib.check(rc, "cbm_spmm_update_f32")
@@ -706,11 +721,13 @@ class CBMMatmul(torch.autograd.Function):
         return gx, None, None
 
 
-def relayout_slabs(x, mask=None, out=None):
+def relayout_slabs(x, mask=None, out=None, scale=None):
     """Slab-major copy of ``x`` for ``cbm_spmm_f32(..., CBM_SPMM_WORKSPACE_READY)`` (None for an
     empty matrix).  With ``mask`` (same shape) the copy holds ``x`` where ``mask > 0`` and zero
-    elsewhere (``cbm_relayout_slabs_masked_f32``: a ReLU gradient folded into the copy).  ``out``:
-    a float32 device tensor of at least ``cbm_relayout_floats(n, d)`` elements to reuse."""
+    elsewhere (``cbm_relayout_slabs_masked_f32``: a ReLU gradient folded into the copy).  With
+    ``scale`` (fp32 [n], e.g. the matrix's ``col_multiplier`` on the device) row r of the copy is
+    multiplied by ``scale[r]``: announce such a copy with ``workspace_prescaled=True``.  ``out``: a
+    float32 device tensor of at least ``cbm_relayout_floats(n, d)`` elements to reuse."""
     n, d = x.shape
     floats = _lib.hip_lib().cbm_relayout_floats(n, d)
     if floats <= 0:
@@ -718,15 +735,20 @@ def relayout_slabs(x, mask=None, out=None):
     if out is not None and (out.numel() < floats or out.device != x.device or out.dtype != torch.float32):
         raise ValueError("out is too small, on another device or not float32")
     ws = out if out is not None else torch.empty(floats, dtype=torch.float32, device=x.device)
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != n or scale.device != x.device
+                              or not scale.is_contiguous()):
+        raise ValueError("scale must be a contiguous float32 vector of n elements on x's device")
     with torch.cuda.device(x.device):
-        if mask is None:
+        if mask is None and scale is None:
             rc = _lib.hip_lib().cbm_relayout_slabs_f32(_ptr(x), _ptr(ws), n, d, _ld(x), _stream(x.device))
+        elif mask is None:
+            rc = _lib.hip_lib().cbm_relayout_slabs_scaled_f32(_ptr(x), _ptr(scale), _ptr(ws), n, d, _ld(x), _stream(x.device))
         else:
             _check_f32_matrix(mask, "mask", n)
             if mask.size(1) != d or mask.device != x.device:
                 raise ValueError("mask must have the shape and device of x")
-            rc = _lib.hip_lib().cbm_relayout_slabs_masked_f32(_ptr(x), _ptr(mask), _ptr(ws), n, d, _ld(x), _ld(mask),
-                                                              _stream(x.device))
+            rc = _lib.hip_lib().cbm_relayout_slabs_masked_f32(_ptr(x), _ptr(mask), _ptr(scale), _ptr(ws), n, d, _ld(x),
+                                                              _ld(mask), _stream(x.device))
     _lib.check(rc, "cbm_relayout_slabs_f32")
     return ws
 

@@ -360,10 +360,13 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 // are consecutive and aligned.  One thread per float4 of the copy.
 // With a mask matrix M (same shape as X, row stride ldm) the copy holds X where M > 0 and zero
 // elsewhere: the gradient of a ReLU applied to the incoming gradient in the pass that copies it.
-template <bool VEC_IN, bool MASKED>
+// With a scale vector the copy holds scale[r] * X[r][:] (one correctly rounded fp32 product per
+// element): the right-hand diagonal of D^-1/2 (A + I) D^-1/2 applied once per row of X instead of
+// once per delta entry, after which the SpMM needs no coefficient per entry, only the sign bit.
+template <bool VEC_IN, bool MASKED, bool SCALED>
 __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n, int d,
                                                       int n_slabs, int64_t ldx, const float* __restrict__ M,
-                                                      int64_t ldm) {
+                                                      int64_t ldm, const float* __restrict__ scale) {
     constexpr int kSlab4 = 8;                              // float4 per 128-byte slab
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int row4 = n_slabs * kSlab4;
@@ -394,6 +397,10 @@ __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ 
         }
         v.x = k.x > 0.0f ? v.x : 0.0f; v.y = k.y > 0.0f ? v.y : 0.0f;
         v.z = k.z > 0.0f ? v.z : 0.0f; v.w = k.w > 0.0f ? v.w : 0.0f;
+    }
+    if constexpr (SCALED) {
+        const float f = scale[r];
+        v.x *= f; v.y *= f; v.z *= f; v.w *= f;
     }
     *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * kSlab4 + w) * 4) = v;
 }
@@ -877,16 +884,24 @@ inline int64_t matrix_bytes(int32_t n, int32_t d, int64_t ld) {
 }
 
 inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s,
-                           const float* mask = nullptr, int64_t ldm = 0) {
+                           const float* mask = nullptr, int64_t ldm = 0, const float* scale = nullptr) {
     const int ns = padded_slab_count(d);
     const int64_t blocks = ((int64_t)n * ns * 8 + 255) / 256;
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
     const dim3 grid((unsigned)blocks), block(256);
     const bool vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16) && (!mask || (ldm % 4 == 0 && aligned(mask, 16)));
-#define LAUNCH_RELAYOUT(V, K) \
-    hipLaunchKernelGGL((relayout_slabs<V, K>), grid, block, 0, s, X, workspace, n, d, ns, ldx, mask, ldm)
-    if (vec) { if (mask) LAUNCH_RELAYOUT(true, true); else LAUNCH_RELAYOUT(true, false); }
-    else { if (mask) LAUNCH_RELAYOUT(false, true); else LAUNCH_RELAYOUT(false, false); }
+#define LAUNCH_RELAYOUT(V, K, S) \
+    hipLaunchKernelGGL((relayout_slabs<V, K, S>), grid, block, 0, s, X, workspace, n, d, ns, ldx, mask, ldm, scale)
+    switch ((vec ? 4 : 0) | (mask ? 2 : 0) | (scale ? 1 : 0)) {
+        case 0: LAUNCH_RELAYOUT(false, false, false); break;
+        case 1: LAUNCH_RELAYOUT(false, false, true); break;
+        case 2: LAUNCH_RELAYOUT(false, true, false); break;
+        case 3: LAUNCH_RELAYOUT(false, true, true); break;
+        case 4: LAUNCH_RELAYOUT(true, false, false); break;
+        case 5: LAUNCH_RELAYOUT(true, false, true); break;
+        case 6: LAUNCH_RELAYOUT(true, true, false); break;
+        default: LAUNCH_RELAYOUT(true, true, true); break;
+    }
 #undef LAUNCH_RELAYOUT
     return CBM_OK;
 }
@@ -895,8 +910,10 @@ template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* val, const float* m,
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
-    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU)) return CBM_ERR_UNSUPPORTED;
+    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
     const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
+    if ((flags & CBM_SPMM_WORKSPACE_PRESCALED) && (!PACKED || !m || !(flags & CBM_SPMM_WORKSPACE_READY)))
+        return CBM_ERR_UNSUPPORTED;                       // only a ready copy of a normalised multiply can be pre-scaled
     if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldz)) return rc;
@@ -920,12 +937,17 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
         const int lpe = plan.lpe, n_slabs = plan.n_slabs;
         const float* Xg = X;                              // what the gather reads
         int64_t x_slab_stride = lpe * 4, x_row_stride = ldx;
+        // A normalised multiply that copies X anyway scales row c of the copy by m[c]: the entries
+        // then need no coefficient at all, only their sign (4 bytes per entry and slab less to stream).
+        bool prescaled = (flags & CBM_SPMM_WORKSPACE_PRESCALED) != 0;
         if (plan.relayout) {
-            if (!ready)
-                if (int rc = launch_relayout(X, workspace, n, d, ldx, s)) return rc;
+            if (!ready) {
+                prescaled = PACKED && m != nullptr;
+                if (int rc = launch_relayout(X, workspace, n, d, ldx, s, nullptr, 0, prescaled ? m : nullptr)) return rc;
+            }
             Xg = workspace; x_slab_stride = (int64_t)n * lpe * 4; x_row_stride = lpe * 4;
         }
-        const int coef_mode = val ? kCoefStream : (m ? kCoefSignM : kCoefSign);
+        const int coef_mode = prescaled ? kCoefSign : (val ? kCoefStream : (m ? kCoefSignM : kCoefSign));
         const DeviceFacts* facts = device_facts();
         const int per_wave = facts ? facts->cus / kXcds : 0;
         int G = facts ? facts->groups[PACKED ? 1 : 0][lpe == 8 ? 0 : 1][coef_mode] : 0;
@@ -1105,8 +1127,19 @@ int cbm_relayout_slabs_f32(const float* X, float* workspace, int32_t n, int32_t 
     return check_launch();
 }
 
-int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, float* workspace, int32_t n, int32_t d, int64_t ldx,
-                                  int64_t ldm, void* stream) {
+int cbm_relayout_slabs_scaled_f32(const float* X, const float* scale, float* workspace, int32_t n, int32_t d, int64_t ldx,
+                                  void* stream) {
+    if (!X || !workspace || !scale) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
+    if (ranges_overlap(workspace, (int64_t)n * padded_slab_count(d) * 32 * 4, X, matrix_bytes(n, d, ldx))) return CBM_ERR_SHAPE;
+    if (n == 0 || d == 0) return CBM_OK;
+    if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream), nullptr, 0, scale)) return rc;
+    return check_launch();
+}
+
+int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, const float* scale, float* workspace, int32_t n,
+                                  int32_t d, int64_t ldx, int64_t ldm, void* stream) {
     if (!X || !workspace || !mask) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldm)) return rc;
@@ -1116,7 +1149,7 @@ int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, float* work
         ranges_overlap(workspace, ws_bytes, mask, matrix_bytes(n, d, ldm)))
         return CBM_ERR_SHAPE;
     if (n == 0 || d == 0) return CBM_OK;
-    if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream), mask, ldm)) return rc;
+    if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream), mask, ldm, scale)) return rc;
     return check_launch();
 }
 
@@ -1217,7 +1250,8 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, float* workspace,
                         int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
-    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY)) return CBM_ERR_UNSUPPORTED;
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+        return CBM_ERR_UNSUPPORTED;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
     const bool relu = (flags & CBM_UPDATE_RELU) != 0;
     // With a flat tree the SpMM's store is the final value of every row: the ReLU goes into its
@@ -1225,6 +1259,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
     // ReLU is a pass of its own after the walk.
     const bool flat = n_levels <= 1;
     int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
+    if (flags & CBM_UPDATE_WORKSPACE_PRESCALED) spmm_flags |= CBM_SPMM_WORKSPACE_PRESCALED;
     if (relu && flat) spmm_flags |= CBM_SPMM_RELU;
     int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, Y, workspace, spmm_flags, n, d, ldx, ldy,
                           stream);
@@ -1245,7 +1280,8 @@ int cbm_spmm_update_static_f32(const int32_t* rowptr, const uint32_t* idx, int64
                                int64_t ldy, int32_t flags, void* stream) {
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldy)) return rc;
-    if (flags & CBM_UPDATE_WORKSPACE_READY) return CBM_ERR_UNSUPPORTED;   // the scratch is not the caller's to fill
+    if (flags & (CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+        return CBM_ERR_UNSUPPORTED;                       // the scratch is not the caller's to fill
     const int64_t need = cbm_spmm_workspace_floats(n, d, ldx, ldy, X, Y);
     if (need > (int64_t)CBM_STATIC_SCRATCH_FLOATS) return CBM_ERR_SCRATCH;
     float* ws = nullptr;                                  // need == 0: this shape gathers from X in place

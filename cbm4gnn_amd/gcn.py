@@ -16,9 +16,11 @@ CBM multiply with the transposed operator.
 ``CBMGCNLayer(fused=True)`` (the default) runs the whole layer as one autograd function around
 the multiply:
 
-* the Linear output is written by the GEMM straight into a buffer whose row stride is d + 32
-  floats (an odd number of 128-byte lines), which the SpMM gathers in place -- no slab-major copy
-  of it is made (widths that are not 32, 64, 128 or 256 still take the copy);
+* with a plain (un-normalised) operator the Linear output is written by the GEMM straight into a
+  buffer whose row stride is d + 32 floats (an odd number of 128-byte lines), which the SpMM
+  gathers in place -- no slab-major copy of it is made (widths other than 32, 64, 128 or 256
+  still take the copy).  A normalised operator keeps the copy: scaled by m on the way, it
+  spares the multiply every per-entry coefficient, which is worth more than the copy costs;
 * the ReLU is applied in the multiply's store epilogue (``CBM_UPDATE_RELU``) and its gradient is
   folded into the slab-major copy the backward multiply makes of the incoming gradient
   (``cbm_relayout_slabs_masked_f32``), with the layer's own output as the mask;
@@ -59,7 +61,8 @@ class _FusedGCNLayer(torch.autograd.Function):
         n, d = xd.size(0), weight.size(0)
         b = layer._layer_buffers(n, d, xd.device)
         torch.mm(xd, weight.detach().t(), out=b["h"])
-        op._run_spmm_update(b["h"], b["y"], use_m=True, workspace=b["ws"] if b["copy_h"] else None, relu=layer.relu)
+        op._run_spmm_update(b["h"], b["y"], use_m=op.col_multiplier is not None,
+                            workspace=b["ws"] if b["copy_h"] else None, relu=layer.relu)
         ctx.layer = layer
         ctx.save_for_backward(xd, weight)
         return b["y"].detach()                              # a fresh tensor object on the cached storage
@@ -75,10 +78,14 @@ class _FusedGCNLayer(torch.autograd.Function):
             g = g.contiguous()
         if layer.relu:
             # d relu: the copy the multiply gathers from holds g where the layer's output is positive
-            relayout_slabs(g, mask=b["y"], out=b["ws"])
-            op_t._run_spmm_update(g, b["gh"], use_m=True, workspace=b["ws"], workspace_ready=True)
+            # (and, like every copy a normalised multiply makes, g scaled by m row by row)
+            scale = op_t._device_arrays(g.device)["m"]
+            relayout_slabs(g, mask=b["y"], out=b["ws"], scale=scale)
+            op_t._run_spmm_update(g, b["gh"], use_m=scale is not None, workspace=b["ws"], workspace_ready=True,
+                                  workspace_prescaled=scale is not None)
         else:
-            op_t._run_spmm_update(g, b["gh"], use_m=True, workspace=b["ws"] if b["copy_g"] else None)
+            op_t._run_spmm_update(g, b["gh"], use_m=op_t.col_multiplier is not None,
+                                  workspace=b["ws"] if b["copy_g"] else None)
         gh = b["gh"]
         gw = torch.mm(gh.t(), x) if ctx.needs_input_grad[1] else None
         gx = torch.mm(gh, weight) if ctx.needs_input_grad[0] else None
@@ -108,8 +115,13 @@ class CBMGCNLayer(nn.Module):
         y = torch.empty((n, d), dtype=torch.float32, device=device)
         gh = torch.empty((n, d), dtype=torch.float32, device=device)
         # Linear output with rows d + 32 floats apart when the library then gathers it in place
-        padded = torch.empty((n, d + 32), dtype=torch.float32, device=device)[:, :d]
-        in_place = d % 32 == 0 and lib.cbm_spmm_workspace_floats(n, d, _ld(padded), _ld(y), _ptr(padded), _ptr(y)) == 0
+        # (plain matrices only: a normalised multiply gains more from scaling its slab-major copy by
+        # m -- the entries then carry no coefficient -- than the copy costs: 233k rows x 128, 491
+        # entries per row: 2.81 ms with the scaled copy, 3.08 ms gathered in place)
+        in_place = False
+        if d % 32 == 0 and op.col_multiplier is None:
+            padded = torch.empty((n, d + 32), dtype=torch.float32, device=device)[:, :d]
+            in_place = lib.cbm_spmm_workspace_floats(n, d, _ld(padded), _ld(y), _ptr(padded), _ptr(y)) == 0
         h = padded if in_place else torch.empty((n, d), dtype=torch.float32, device=device)
         copy_h = (not in_place) and op.relayout and _wants_workspace(h, y, op.nnz)
         copy_g = op.relayout and _wants_workspace(gh, y, op.transposed().nnz)

@@ -44,7 +44,9 @@ enum {
 /* flags of cbm_spmm_f32 / csr_spmm_f32 */
 enum {
     CBM_SPMM_WORKSPACE_READY = 1, /* workspace already holds cbm_relayout_slabs_f32(X): do not copy again */
-    CBM_SPMM_RELU = 2             /* store max(z, 0) instead of z (after the left scale of root children) */
+    CBM_SPMM_RELU = 2,            /* store max(z, 0) instead of z (after the left scale of root children) */
+    CBM_SPMM_WORKSPACE_PRESCALED = 4 /* with WORKSPACE_READY, cbm_spmm_f32 with m only: the copy was made by
+                                     cbm_relayout_slabs_scaled_f32(X, m) (or the masked variant with m) */
 };
 
 /* flags of cbm_propagate_f32 */
@@ -59,7 +61,8 @@ enum {
                                        (benchmark/parallel/benchmark_gcn_cpu.py:84-88 applies it as a
                                        separate pass); in the SpMM epilogue when the tree is flat,
                                        one extra pass over Y otherwise */
-    CBM_UPDATE_WORKSPACE_READY = 4  /* as CBM_SPMM_WORKSPACE_READY */
+    CBM_UPDATE_WORKSPACE_READY = 4, /* as CBM_SPMM_WORKSPACE_READY */
+    CBM_UPDATE_WORKSPACE_PRESCALED = 8 /* as CBM_SPMM_WORKSPACE_PRESCALED */
 };
 
 /* The CBM format as built on the host.  All arrays are malloc'd by cbm_build_host and are
@@ -198,7 +201,8 @@ int cbm_expand_coef_f32(const uint32_t* idx_dev, const float* m_dev, float* coef
  * (16-byte aligned, disjoint from X and Z): X is first copied there slab-major (zero-padded to
  * whole 128-byte slabs), so that the gathered lines of a slab are consecutive in memory instead of
  * a row apart and odd widths (d = 41, 602, unaligned rows) run on the slab kernel too.  The fp32
- * summation order with and without it can differ (cbm_spmm_summation_groups reports both).  The
+ * summation order with and without it can differ (cbm_spmm_summation_groups reports both), and
+ * with m the copy is pre-scaled (see cbm_relayout_slabs_scaled_f32): coef is then not read.  The
  * copy pays off when rows have more than a few entries.
  * nnz is the number of entries (rowptr[n]); it only sizes the launch (long rows run with fewer
  * resident wavefronts, see cbm_set_spmm_occupancy) and may be 0 if unknown.
@@ -221,8 +225,19 @@ int64_t cbm_relayout_floats(int32_t n, int32_t d);
  * CBM_UPDATE_RELU, X the gradient arriving at it).  The backward multiply then runs from the copy
  * with WORKSPACE_READY and never reads X.  No reference counterpart: the reference's layers have
  * no backward pass (gnns/message_passing/cbm_message_passing.py:16-60 mutate a cached output). */
-int cbm_relayout_slabs_masked_f32(const float* X_dev, const float* mask_dev, float* workspace_dev, int32_t n, int32_t d,
-                                  int64_t ldx, int64_t ldm, void* stream);
+int cbm_relayout_slabs_masked_f32(const float* X_dev, const float* mask_dev, const float* scale_dev /* nullable */,
+                                  float* workspace_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldm, void* stream);
+
+/* The copy with row r multiplied by scale[r] (one rounded fp32 product per element).  With
+ * scale = m this is what a normalised cbm_spmm_f32 makes by itself when it copies X: the right-hand
+ * diagonal of diag(m) A diag(m) is applied once per row of X, and the delta entries then carry
+ * only their sign (no coefficient array is streamed, coef may be NULL).  The reference applies the
+ * same diagonal per delta entry as the value +-m[col] (cbm_extensions.cpp:504-585); the two
+ * differ in fp32 rounding only: fma(+-m[c], x, acc) there, acc +- fl(m[c] * x) here.  A copy made
+ * by this call is announced to the multiply with WORKSPACE_READY | WORKSPACE_PRESCALED.
+ * cbm_relayout_slabs_masked_f32 takes the same vector (NULL = no scaling). */
+int cbm_relayout_slabs_scaled_f32(const float* X_dev, const float* scale_dev, float* workspace_dev, int32_t n, int32_t d,
+                                  int64_t ldx, void* stream);
 
 /* In-place tree propagation over Y (which holds Z on entry), level by level.
  *   m == NULL : Y[v,:] += Y[parent[v],:]

@@ -51,14 +51,40 @@ def mat_groups(mat, d, ld=None):
     return groups_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, n, d, ld))
 
 
-def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None):
-    """Reference-style CPU multiply on the PRODUCT's tree (so both sides sum in the same order)."""
+def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, prescaled=None):
+    """Reference-style CPU multiply on the PRODUCT's tree (so both sides sum in the same order).
+    ``prescaled``: the arithmetic of a normalised multiply that copies X slab-major -- row c of
+    the copy is fl(m[c] * x[c]) and the delta entries are +-1 -- instead of the reference's
+    fma(+-m[c], x[c], acc); by default whichever the multiply through ``cbm_matrix`` uses."""
     col, sign = mat.columns()
     m = orc.col_multiplier(ei, n) if normalized else None
+    g = mat_groups(mat, x.shape[1]) if groups is None else groups
+    if prescaled is None:                                  # the copy is only made for the slab kernel (g > 1)
+        prescaled = normalized and brings_workspace(mat.relayout, mat.nnz, n, x.shape[1]) and mat_groups(mat, x.shape[1]) > 1
+    if prescaled:
+        xs = (m[:, None] * x).astype(np.float32)
+        z = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
+                         threads=threads, groups=g)
+        return orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads)
     val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
     return orc.spmm_update(mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32),
-                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads,
-                           groups=mat_groups(mat, x.shape[1]) if groups is None else groups)
+                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads, groups=g)
+
+
+def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
+    """The delta SpMM alone, Z = Delta diag(m) X, in the arithmetic and order of the multiply
+    through ``cbm_matrix`` (see ``oracle_product``)."""
+    col, sign = mat.columns()
+    d = x.shape[1]
+    g = mat_groups(mat, d)
+    if not normalized:
+        return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, groups=g)
+    m = orc.col_multiplier(ei, n)
+    if brings_workspace(mat.relayout, mat.nnz, n, d) and g > 1:      # the copy of X is scaled by m
+        return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32),
+                            (m[:, None] * x).astype(np.float32), groups=g)
+    val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
+    return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=g)
 
 
 @pytest.fixture(params=["auto", "wave-per-row"])
@@ -184,10 +210,8 @@ def test_update_only_entry_points(orc):
         # spmm alone == Delta (diag m) X
         z = torch.empty((n, d), device="cuda")
         mat.omp_mkl_csr_spmm(torch.from_numpy(x).cuda(), z)
-        col, sign = mat.columns()
         m = orc.col_multiplier(ei, n) if normalized else None
-        val = (sign.numpy() * (m[col.numpy()] if normalized else 1)).astype(np.float32)
-        z_ref = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=mat_groups(mat, d))
+        z_ref = oracle_delta_spmm(orc, mat, ei, n, x, normalized)
         assert np.array_equal(z.cpu().numpy(), z_ref)
         # update alone on that Z == the oracle's walk (plain or fused) on the same Z
         y = z.clone()
@@ -367,15 +391,17 @@ def test_c_abi_status_codes_on_device_calls():
 
 
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("alpha,directed", [(2, False), (10_000, False), (2, True)])
-def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directed):
+@pytest.mark.parametrize("alpha,directed,normalized", [(2, False, True), (10_000, False, True), (2, True, True),
+                                                       (2, False, False)])
+def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directed, normalized):
     """The GCN epoch harness (Linear -> CBM aggregate -> ReLU -> Linear -> CBM aggregate, cross
     entropy) against the same model written with a dense normalised adjacency in torch fp64.
     ``fused``: the layer as one autograd function (Linear output gathered in place from a padded
     buffer, ReLU in the multiply's epilogue -- alpha = 10 000 gives the flat tree where it is
     the SpMM's epilogue, alpha = 2 a deeper tree where it is a pass after the walk -- and its
     gradient folded into the slab-major copy of the backward multiply); ``directed``: the backward
-    multiply runs on the transposed operator."""
+    multiply runs on the transposed operator; ``normalized=False``: the plain adjacency, whose
+    Linear output the fused layer lets the SpMM gather in place."""
     from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
     n, f_in, hidden, classes = 300, 37, 128, 41
     ei_np = graphs.add_self_loops(graphs.sbm(n, 6, 0.3, 0.02, seed=11), n)
@@ -383,8 +409,8 @@ def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directe
         keep = (np.random.default_rng(5).random(ei_np.shape[1]) > 0.3) | (ei_np[0] == ei_np[1])
         ei_np = np.ascontiguousarray(ei_np[:, keep])
     ei = torch.from_numpy(ei_np)
-    say("gcn harness", fused, alpha, directed)
-    op = build_operator(ei, alpha=alpha, normalized=True)
+    say("gcn harness", fused, alpha, directed, normalized)
+    op = build_operator(ei, alpha=alpha, normalized=normalized)
     assert (op.n_levels == 1) == (alpha == 10_000) and op.is_symmetric == (not directed)
     torch.manual_seed(1)
     model = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op, fused=fused, relu=fused),
@@ -393,7 +419,7 @@ def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directe
     y = torch.randint(0, classes, (n,), generator=torch.Generator().manual_seed(3)).cuda()
     a = torch.from_numpy(orc.dense_adjacency(np.stack([ei_np[1], ei_np[0]]), n)).double().cuda()
     m = a.sum(dim=1).pow(-0.5)
-    a_hat = m[:, None] * a * m[None, :]
+    a_hat = m[:, None] * a * m[None, :] if normalized else a
     for epoch in range(2):                                  # the second pass runs on the cached buffers
         model.zero_grad(set_to_none=True)
         xin = x.clone().requires_grad_(True)
@@ -413,11 +439,13 @@ def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directe
             assert float((got.double() - want).abs().max() / want.abs().max()) <= 1e-3
     if fused:
         b = model.first_layer._cache
-        assert b["h_in_place"] and b["h"].stride(0) == hidden + 32 and not b["copy_h"]    # gathered in place
+        # plain operator: the Linear output sits in a padded buffer and is gathered in place; a
+        # normalised one keeps the copy (scaled by m on the way)
+        assert b["h_in_place"] == (not normalized) and b["h"].stride(0) == (hidden if normalized else hidden + 32)
         assert float(b["y"].min()) == 0.0                                               # the ReLU was applied
         assert not model.last_layer._cache["h_in_place"]                                # width 41 takes the copy
     # the CSR-baseline model computes the same thing
-    vals = op.col_multiplier[ei[0].long()] * op.col_multiplier[ei[1].long()]
+    vals = op.col_multiplier[ei[0].long()] * op.col_multiplier[ei[1].long()] if normalized else None
     fwd = csr_operator(torch.stack([ei[1], ei[0]]), n, vals, x.device)
     bwd = fwd if not directed else csr_operator(ei, n, vals, x.device)
     torch.manual_seed(1)
@@ -448,8 +476,12 @@ def test_relu_epilogue_and_masked_copy_through_the_c_abi(orc):
             mask = torch.randn((n, d), generator=torch.Generator().manual_seed(d + 1)).cuda()
             ws = relayout_slabs(x, mask=mask)
             assert torch.equal(ws, relayout_slabs(torch.where(mask > 0, x, torch.zeros_like(x))))
+            m_dev = mat._device_arrays(x.device)["m"]
+            ws = relayout_slabs(x, mask=mask, scale=m_dev)
+            assert torch.equal(ws, relayout_slabs(torch.where(mask > 0, x, torch.zeros_like(x)), scale=m_dev))
             via_copy = torch.empty_like(x)
-            mat._run_spmm_update(torch.full_like(x, float("nan")), via_copy, use_m=True, workspace=ws, workspace_ready=True)
+            mat._run_spmm_update(torch.full_like(x, float("nan")), via_copy, use_m=True, workspace=ws, workspace_ready=True,
+                                 workspace_prescaled=True)
             direct = torch.empty_like(x)
             mat._run_spmm_update(torch.where(mask > 0, x, torch.zeros_like(x)), direct, use_m=True, workspace=torch.empty_like(ws))
             assert torch.equal(via_copy, direct)
@@ -507,9 +539,19 @@ def test_shared_slab_major_copy(orc):
     assert torch.equal(ws.view(d // 32, n, 32).permute(1, 0, 2).reshape(n, d), x)
     for alpha in (0, 1000):
         mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=True)
+        # the plain copy: the entries carry +-m[col], as when the multiply gathers from X in place
+        mat.relayout = False
         want = torch.empty_like(x); mat._run_spmm(x, want, use_m=True, scale_roots=True)
+        mat.relayout = True
         got = torch.empty_like(x); mat._run_spmm(torch.zeros_like(x), got, use_m=True, scale_roots=True,
                                                  workspace=ws, workspace_ready=True)     # X itself is not read
+        assert torch.equal(got, want)
+        # the copy scaled by m, which is what the multiply makes for itself
+        want = torch.empty_like(x); mat._run_spmm(x, want, use_m=True, scale_roots=True)
+        wm = relayout_slabs(x, scale=mat._device_arrays(x.device)["m"])
+        assert torch.equal(wm.view(d // 32, n, 32).permute(1, 0, 2).reshape(n, d), x * mat.col_multiplier.cuda()[:, None])
+        got = torch.empty_like(x); mat._run_spmm(torch.zeros_like(x), got, use_m=True, scale_roots=True,
+                                                 workspace=wm, workspace_ready=True, workspace_prescaled=True)
         assert torch.equal(got, want)
     # odd width: the copy is zero-padded to whole slabs (41 -> 2 slabs of 32)
     x41 = torch.randn((n, 41), generator=torch.Generator().manual_seed(5)).cuda()
@@ -628,9 +670,14 @@ def test_alias_free_row_stride_needs_no_copy(orc):
     say("alias-free stride")
     want = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, want)
     got = torch.full_like(x, float("nan")); mat.omp_mkl_csr_fused_spmm_update(xp, got)
+    # same summation order; the in-place gather multiplies by +-m[col] per entry, the copy is scaled by m
+    assert np.array_equal(got.cpu().numpy(), oracle_product(orc, mat, ei, n, x.cpu().numpy(), True, groups=8, prescaled=False))
+    assert np.array_equal(want.cpu().numpy(), oracle_product(orc, mat, ei, n, x.cpu().numpy(), True, groups=8, prescaled=True))
+    assert orc.max_rel_err(got.cpu().numpy(), want.cpu().numpy()) <= 1e-6
+    plain = cbm_matrix(torch.from_numpy(ei), None, alpha=1)                         # no m: bit-identical either way
+    want = torch.empty_like(x); plain.omp_mkl_csr_spmm_update(x, want)
+    got = torch.full_like(x, float("nan")); plain.omp_mkl_csr_spmm_update(xp, got)
     assert torch.equal(got, want)
-    ref = oracle_product(orc, mat, ei, n, x.cpu().numpy(), True, groups=8)
-    assert np.array_equal(got.cpu().numpy(), ref)
 
 
 @pytest.mark.parametrize("normalized", [False, True])
@@ -676,8 +723,7 @@ def test_plain_methods_on_a_normalised_matrix_apply_the_right_scaling_only(orc):
     x = np.random.default_rng(21).standard_normal((n, d)).astype(np.float32)
     m = orc.col_multiplier(ei, n)
     col, sign = mat.columns()
-    val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
-    z = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=mat_groups(mat, d))
+    z = oracle_delta_spmm(orc, mat, ei, n, x, True)
     want = orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z.copy())
     a = orc.dense_adjacency(ei, n).astype(np.float64)
     dense = a @ (m.astype(np.float64)[:, None] * x.astype(np.float64))
@@ -718,6 +764,7 @@ def test_changing_a_cached_setting_takes_effect():
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
     x = torch.randn((n, d), generator=torch.Generator().manual_seed(8)).cuda()
     say("cached settings")
+    mat.relayout = False                                    # gather in place: the entries' coefficients are used
     y1 = torch.empty_like(x); mat.omp_mkl_csr_fused_spmm_update(x, y1)
     assert mat._device_arrays(x.device)["coef"] is not None
     mat.stream_coefficients = False
