@@ -38,6 +38,27 @@ class CbmFormat(C.Structure):
     ]
 
 
+class CbmTiling(C.Structure):
+    """Mirror of ``struct cbm_tiling`` (host arrays made by ``cbm_tile_rows``)."""
+    _fields_ = [
+        ("n", C.c_int32), ("tile_rows", C.c_int32), ("panel_rows", C.c_int32), ("n_panels", C.c_int32),
+        ("n_blocks", C.c_int32), ("has_negative", C.c_int32),
+        ("nnz_local", C.c_int64), ("nnz_local_padded", C.c_int64), ("nnz_remote", C.c_int64),
+        ("panel_ptr", C.POINTER(C.c_int32)), ("blk_tile", C.POINTER(C.c_int32)), ("seg", C.POINTER(C.c_int32)),
+        ("lidx", C.POINTER(C.c_uint16)), ("rowptr_r", C.POINTER(C.c_int32)), ("idx_r", C.POINTER(C.c_uint32)),
+    ]
+
+
+class CbmTilingDev(C.Structure):
+    """Mirror of ``struct cbm_tiling_dev`` (the same arrays in device memory)."""
+    _fields_ = [
+        ("n_panels", C.c_int32), ("n_blocks", C.c_int32), ("tile_rows", C.c_int32), ("has_negative", C.c_int32),
+        ("nnz_remote", C.c_int64),
+        ("panel_ptr", C.c_void_p), ("blk_tile", C.c_void_p), ("seg", C.c_void_p), ("lidx", C.c_void_p),
+        ("rowptr_r", C.c_void_p), ("idx_r", C.c_void_p), ("sched_r", C.c_void_p), ("row_scale", C.c_void_p),
+    ]
+
+
 _P = C.c_void_p
 _I32, _I64 = C.c_int32, C.c_int64
 
@@ -48,6 +69,8 @@ HOST_SYMBOLS = {
     "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
     "cbm_build_host_timings": (None, [C.POINTER(C.c_double)]),
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
+    "cbm_tile_rows": (C.c_int, [_P, _P, _I32, _I32, _I64, _I32, C.POINTER(CbmTiling)]),
+    "cbm_tiling_free": (None, [C.POINTER(CbmTiling)]),
     "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),
     "cbm_builder_arrays": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
                                      C.POINTER(_P), C.POINTER(_I64)]),
@@ -71,6 +94,9 @@ HIP_SYMBOLS = {
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_tiled_f32": (C.c_int, [C.POINTER(CbmTilingDev), _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
+    "cbm_spmm_update_tiled_f32": (C.c_int, [C.POINTER(CbmTilingDev), _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64,
+                                            _I64, _I32, _P]),
     "csr_spmm_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_row_intersections_groups": (C.c_int, []),
     "cbm_row_intersections": (C.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _P, _I64, _P, _P]),

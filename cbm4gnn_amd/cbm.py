@@ -234,7 +234,7 @@ def _build_staged(ei_cpu, n, alpha, threads, fmt, gpu, max_levels):
 class cbm_matrix:
 
     def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
-                 deltas_format="csr", threads=0, builder="auto", max_levels=None):
+                 deltas_format="csr", threads=0, builder="auto", max_levels=None, tiling="auto"):
         ei = torch.as_tensor(edge_index)
         if ei.dim() != 2 or ei.size(0) != 2:
             raise ValueError("Edge index should have shape (2, num_edges)")
@@ -304,6 +304,7 @@ class cbm_matrix:
         self._deltas = None
         self._dev = {}
         self._stream_coefficients = True    # see the property
+        self._init_tiling(tiling)
         self.relayout = True                # False: gather from the caller's row-major X, no n*d scratch per call
         self._transposed = None
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
@@ -361,7 +362,68 @@ class cbm_matrix:
         self._deltas, self._dev, self._transposed = None, {}, None
         self._stream_coefficients = True
         self.relayout = True
+        self._init_tiling("auto")
         return self
+
+    # ------------------------------------------------------------------ tiling --------------
+    # Entries that cluster in (256-row panel, 1024-column tile) blocks -- graphs with community
+    # structure whose rows are ordered by community -- can be gathered from tiles of X staged in LDS
+    # (``cbm_spmm_tiled_f32``) instead of through L1/L2.  "auto": use it when the matrix is large
+    # and at least ``tile_min_local_fraction`` of its delta entries fall into blocks of at least
+    # ``tile_min_block_entries`` entries; "on" / "off" force the choice.
+    def _init_tiling(self, policy):
+        if policy not in ("auto", "on", "off"):
+            raise ValueError('tiling must be "auto", "on" or "off"')
+        self.tiling = policy
+        self.tile_rows = 1024
+        self.tile_min_block_entries = 4096
+        self.tile_min_local_fraction = 0.8
+        self._tiling_host = None            # None: not computed; False: computed and rejected; dict: arrays
+        self.tiling_info = None
+
+    def _host_tiling(self):
+        """The split of the delta matrix into local blocks and remote entries (``cbm_tile_rows``), or
+        False when the policy or the matrix rules it out.  Computed once."""
+        if self._tiling_host is not None:
+            return self._tiling_host
+        n = self.num_rows
+        self._tiling_host = False
+        if self.tiling == "off" or self.nnz == 0:
+            return False
+        if self.tiling == "auto" and (n < 16 * self.tile_rows or self.nnz < 32 * n):
+            return False                                    # too small for tiles of 1024 rows to pay
+        t = _lib.CbmTiling()
+        rc = _lib.host_lib().cbm_tile_rows(_ptr(self.rowptr), _ptr(self.idx), n, self.tile_rows,
+                                           self.tile_min_block_entries, 0, C.byref(t))
+        try:
+            _lib.check(rc, "cbm_tile_rows")
+            info = {"n_blocks": int(t.n_blocks), "nnz_local": int(t.nnz_local), "nnz_remote": int(t.nnz_remote),
+                    "local_fraction": t.nnz_local / max(self.nnz, 1), "has_negative": bool(t.has_negative)}
+            self.tiling_info = info
+            if t.n_blocks == 0 or (self.tiling == "auto" and info["local_fraction"] < self.tile_min_local_fraction):
+                return False
+
+            def take(ptr, count, dtype):
+                return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))
+
+            p1 = t.panel_rows + 1
+            self._tiling_host = {
+                "n_panels": int(t.n_panels), "n_blocks": int(t.n_blocks), "tile_rows": int(t.tile_rows),
+                "has_negative": int(t.has_negative), "nnz_remote": int(t.nnz_remote),
+                "panel_ptr": take(t.panel_ptr, t.n_panels + 1, np.int32), "blk_tile": take(t.blk_tile, t.n_blocks, np.int32),
+                "seg": take(t.seg, t.n_blocks * p1, np.int32),
+                "lidx": take(t.lidx, t.nnz_local_padded, np.uint16).view(torch.int16),
+                "rowptr_r": take(t.rowptr_r, n + 1, np.int32),
+                "idx_r": (take(t.idx_r, t.nnz_remote, np.uint32).view(torch.int32) if t.nnz_remote
+                          else torch.empty(0, dtype=torch.int32)),
+            }
+        finally:
+            _lib.host_lib().cbm_tiling_free(C.byref(t))
+        return self._tiling_host
+
+    def is_tiled(self):
+        """Whether multiplies of this matrix take the tiled path (decides it on first call)."""
+        return bool(self._host_tiling())
 
     # Settings the cached device arrays depend on: changing one drops the cache, so that a later
     # multiply never runs on coefficients or schedules derived from the old value.
@@ -473,8 +535,30 @@ class cbm_matrix:
                 "sched_scaled": (schedule_rows(self.rowptr, self.parent, self.col_multiplier).to(device)
                                  if self.col_multiplier is not None else None),
             }
+            th = self._host_tiling()
+            st["tiled"] = None
+            if th:
+                tensors = {k: th[k].to(device) for k in ("panel_ptr", "blk_tile", "seg", "lidx", "rowptr_r", "idx_r")}
+                tensors["sched_r"] = schedule_rows(th["rowptr_r"], None, None).to(device)
+                if self.col_multiplier is not None:          # left scale: m[r] for children of the root
+                    scale = torch.where(self.parent < 0, self.col_multiplier, torch.ones_like(self.col_multiplier))
+                    tensors["row_scale"] = scale.to(device)
+                st["tiled"] = tensors
             self._dev[key] = st
         return st
+
+    def _tiled_struct(self, st, with_scale):
+        """``struct cbm_tiling_dev`` over the device tensors of ``st`` (host-side struct, per call)."""
+        th, tt = self._tiling_host, st["tiled"]
+        return _lib.CbmTilingDev(th["n_panels"], th["n_blocks"], th["tile_rows"], th["has_negative"], th["nnz_remote"],
+                                 tt["panel_ptr"].data_ptr(), tt["blk_tile"].data_ptr(), tt["seg"].data_ptr(),
+                                 tt["lidx"].data_ptr(), tt["rowptr_r"].data_ptr(),
+                                 tt["idx_r"].data_ptr() if th["nnz_remote"] else None, tt["sched_r"].data_ptr(),
+                                 tt["row_scale"].data_ptr() if (with_scale and "row_scale" in tt) else None)
+
+    def _tiled_workspace(self, xd):
+        floats = _lib.hip_lib().cbm_relayout_floats(xd.size(0), xd.size(1))
+        return torch.empty(max(int(floats), 1), dtype=torch.float32, device=xd.device)
 
     def _coef(self, st, device):
         """``+-m[col]`` per delta entry on ``device`` (what the reference keeps as the fp32 values of
@@ -526,6 +610,18 @@ class cbm_matrix:
         if yd.device != xd.device:
             raise ValueError("rhs and dst are on different devices")
         st = self._device_arrays(xd.device)
+        if st["tiled"] is not None and self.relayout and not (workspace_ready and use_m and not workspace_prescaled):
+            ws = workspace if workspace is not None else self._tiled_workspace(xd)
+            flags = (_lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0) | \
+                    (_lib.CBM_SPMM_WORKSPACE_PRESCALED if (workspace_prescaled and use_m) else 0)
+            ts = self._tiled_struct(st, with_scale=use_m and scale_roots)
+            with torch.cuda.device(xd.device):
+                rc = _lib.hip_lib().cbm_spmm_tiled_f32(C.byref(ts), _ptr(st["m"]) if use_m else None, _ptr(xd), _ptr(yd),
+                                                       _ptr(ws), flags, n, x.size(1), _ld(xd), _ld(yd), _stream(xd.device))
+            _lib.check(rc, "cbm_spmm_tiled_f32")
+            if yd is not y:
+                y.copy_(yd)
+            return
         ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         # per-entry coefficients are only read when the multiply does not scale its own copy of X
         coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
@@ -583,13 +679,30 @@ class cbm_matrix:
         if yd.data_ptr() == xd.data_ptr():
             raise ValueError("dst must not alias rhs")
         st = self._device_arrays(xd.device)
-        ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
+        tiled = st["tiled"] is not None and self.relayout and not (workspace_ready and use_m and not workspace_prescaled)
+        if tiled:
+            ws = workspace if workspace is not None else self._tiled_workspace(xd)
+        else:
+            ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         if workspace_ready:
             flags |= _lib.CBM_UPDATE_WORKSPACE_READY
         if workspace_prescaled:
             flags |= _lib.CBM_UPDATE_WORKSPACE_PRESCALED
         if relu:
             flags |= _lib.CBM_UPDATE_RELU
+        if tiled:
+            if not use_m:
+                flags &= ~_lib.CBM_UPDATE_WORKSPACE_PRESCALED
+            ts = self._tiled_struct(st, with_scale=use_m)
+            with torch.cuda.device(xd.device):
+                rc = _lib.hip_lib().cbm_spmm_update_tiled_f32(
+                    C.byref(ts), _ptr(st["m"]) if use_m else None, _ptr(st["parent"]), _ptr(st["order"]),
+                    _ptr(st["level_off"]), _ptr(self.level_off), self.n_levels, _ptr(xd), _ptr(yd), _ptr(ws), n, x.size(1),
+                    _ld(xd), _ld(yd), flags, _stream(xd.device))
+            _lib.check(rc, "cbm_spmm_update_tiled_f32")
+            if yd is not y:
+                y.copy_(yd)
+            return
         coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
@@ -679,7 +792,8 @@ class cbm_matrix:
             return self
         if self._transposed is None:
             ei = self._edge_index_cpu
-            t = cbm_matrix(torch.stack([ei[1], ei[0]]), None, alpha=self.alpha, normalized=False, max_levels=self.max_levels)
+            t = cbm_matrix(torch.stack([ei[1], ei[0]]), None, alpha=self.alpha, normalized=False, max_levels=self.max_levels,
+                           tiling=self.tiling)
             t.col_multiplier = self.col_multiplier      # diag(m) A^T diag(m): same vector both sides
             t.normalized = self.normalized
             t._transposed = self

@@ -631,6 +631,152 @@ int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float*
     }
 }
 
+void cbm_tiling_free(cbm_tiling* t) {
+    if (!t) return;
+    free(t->panel_ptr); free(t->blk_tile); free(t->seg); free(t->lidx); free(t->rowptr_r); free(t->idx_r);
+    std::memset(t, 0, sizeof(*t));
+}
+
+int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t tile_rows, int64_t min_block_entries,
+                  int32_t threads, cbm_tiling* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if (n < 0 || (tile_rows != 1024 && tile_rows != 512) || min_block_entries < 1) return CBM_ERR_SHAPE;
+    if (!rowptr || (n > 0 && rowptr[n] > 0 && !idx)) return CBM_ERR_NULL;
+    if (threads <= 0) threads = omp_get_max_threads();
+    constexpr int P = CBM_TILING_PANEL_ROWS;
+    const int T = tile_rows;
+    const int32_t n_panels = (n + P - 1) / P, n_tiles = (n + T - 1) / T;
+    for (int32_t r = 0; r < n; r++)
+        if (rowptr[r + 1] < rowptr[r]) return CBM_ERR_SHAPE;
+    try {
+        // pass 1: per panel, the tiles that hold at least min_block_entries of its entries
+        std::vector<std::vector<int32_t>> tiles_of(n_panels);
+        int bad = 0;
+#pragma omp parallel num_threads(threads)
+        {
+            std::vector<int64_t> cnt(n_tiles, 0);
+            std::vector<int32_t> touched;
+#pragma omp for schedule(dynamic, 4)
+            for (int32_t p = 0; p < n_panels; p++) {
+                touched.clear();
+                const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
+                for (int64_t k = rowptr[(int64_t)p * P]; k < rowptr[r_end]; k++) {
+                    const uint32_t c = idx[k] & 0x7fffffffu;
+                    if (c >= (uint32_t)n) { bad = 1; continue; }
+                    const int32_t t = (int32_t)(c / (uint32_t)T);
+                    if (cnt[t]++ == 0) touched.push_back(t);
+                }
+                std::sort(touched.begin(), touched.end());
+                for (int32_t t : touched) {
+                    if (cnt[t] >= min_block_entries) tiles_of[p].push_back(t);
+                    cnt[t] = 0;
+                }
+            }
+        }
+        if (bad) return CBM_ERR_SHAPE;
+        out->n = n; out->tile_rows = T; out->panel_rows = P; out->n_panels = n_panels;
+        out->panel_ptr = (int32_t*)malloc(sizeof(int32_t) * ((size_t)n_panels + 1));
+        if (!out->panel_ptr) throw std::bad_alloc();
+        out->panel_ptr[0] = 0;
+        for (int32_t p = 0; p < n_panels; p++) out->panel_ptr[p + 1] = out->panel_ptr[p] + (int32_t)tiles_of[p].size();
+        const int32_t B = out->panel_ptr[n_panels];
+        out->n_blocks = B;
+        out->blk_tile = (int32_t*)malloc(sizeof(int32_t) * std::max<size_t>(B, 1));
+        out->seg = (int32_t*)malloc(sizeof(int32_t) * std::max<size_t>((size_t)B * (P + 1), 1));
+        out->rowptr_r = (int32_t*)malloc(sizeof(int32_t) * ((size_t)n + 1));
+        if (!out->blk_tile || !out->seg || !out->rowptr_r) throw std::bad_alloc();
+        for (int32_t p = 0; p < n_panels; p++)
+            std::copy(tiles_of[p].begin(), tiles_of[p].end(), out->blk_tile + out->panel_ptr[p]);
+        // pass 2: entries per (block, panel row) -> seg (as counts first), remote entries per row
+        std::fill(out->seg, out->seg + (size_t)B * (P + 1), 0);
+        int any_negative = 0;
+#pragma omp parallel num_threads(threads)
+        {
+            std::vector<int32_t> block_of(n_tiles, -1);
+            int neg = 0;
+#pragma omp for schedule(dynamic, 4)
+            for (int32_t p = 0; p < n_panels; p++) {
+                const int32_t b0 = out->panel_ptr[p];
+                for (size_t i = 0; i < tiles_of[p].size(); i++) block_of[tiles_of[p][i]] = b0 + (int32_t)i;
+                const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
+                for (int32_t r = p * P; r < r_end; r++) {
+                    int32_t remote = 0;
+                    for (int64_t k = rowptr[r]; k < rowptr[r + 1]; k++) {
+                        const int32_t b = block_of[(idx[k] & 0x7fffffffu) / (uint32_t)T];
+                        if (b >= 0) { out->seg[(size_t)b * (P + 1) + (r - p * P)]++; neg |= (int)(idx[k] >> 31); }
+                        else remote++;
+                    }
+                    out->rowptr_r[r + 1] = remote;
+                }
+                for (int32_t t : tiles_of[p]) block_of[t] = -1;
+            }
+            if (neg) {
+#pragma omp atomic write
+                any_negative = 1;
+            }
+        }
+        // counts -> offsets: segments padded to multiples of 8 entries, seg[] in units of 8 entries
+        int64_t at8 = 0, real = 0;
+        for (int32_t b = 0; b < B; b++) {
+            int32_t* sg = out->seg + (size_t)b * (P + 1);
+            for (int pr = 0; pr < P; pr++) {
+                const int32_t c = sg[pr];
+                real += c;
+                sg[pr] = (int32_t)at8;
+                at8 += (c + 7) / 8;
+                if (at8 > INT32_MAX) return (cbm_tiling_free(out), CBM_ERR_SHAPE);
+            }
+            sg[P] = (int32_t)at8;
+        }
+        out->rowptr_r[0] = 0;
+        for (int32_t r = 0; r < n; r++) out->rowptr_r[r + 1] += out->rowptr_r[r];
+        out->nnz_local = real;
+        out->nnz_local_padded = at8 * 8;
+        out->nnz_remote = n > 0 ? out->rowptr_r[n] : 0;
+        out->has_negative = any_negative;
+        out->lidx = (uint16_t*)malloc(sizeof(uint16_t) * std::max<size_t>((size_t)at8 * 8, 8));
+        out->idx_r = (uint32_t*)malloc(sizeof(uint32_t) * std::max<size_t>((size_t)out->nnz_remote, 1));
+        if (!out->lidx || !out->idx_r) throw std::bad_alloc();
+        // pass 3: fill.  A local entry is (row of X - first row of its tile) * 8 | sign << 15; the padding
+        // of a segment names row T, the all-zero row the kernel keeps behind the tile.
+        const uint16_t pad = (uint16_t)(T * 8);
+#pragma omp parallel num_threads(threads)
+        {
+            std::vector<int32_t> block_of(n_tiles, -1);
+            std::vector<int32_t> fill(P > 0 ? P : 1);
+#pragma omp for schedule(dynamic, 4)
+            for (int32_t p = 0; p < n_panels; p++) {
+                const int32_t b0 = out->panel_ptr[p];
+                for (size_t i = 0; i < tiles_of[p].size(); i++) block_of[tiles_of[p][i]] = b0 + (int32_t)i;
+                const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
+                for (size_t i = 0; i < tiles_of[p].size(); i++) {       // padding first, entries overwrite it
+                    const int32_t* sg = out->seg + (size_t)(b0 + i) * (P + 1);
+                    std::fill(out->lidx + (size_t)sg[0] * 8, out->lidx + (size_t)sg[P] * 8, pad);
+                }
+                for (int32_t r = p * P; r < r_end; r++) {
+                    int64_t at_r = out->rowptr_r[r];
+                    // columns ascend within a row, so the entries of one block are consecutive: a running cursor per block
+                    int32_t cur_b = -1; int64_t cur_at = 0;
+                    for (int64_t k = rowptr[r]; k < rowptr[r + 1]; k++) {
+                        const uint32_t c = idx[k] & 0x7fffffffu;
+                        const int32_t t = (int32_t)(c / (uint32_t)T);
+                        const int32_t b = block_of[t];
+                        if (b < 0) { out->idx_r[at_r++] = idx[k]; continue; }
+                        if (b != cur_b) { cur_b = b; cur_at = (int64_t)out->seg[(size_t)b * (P + 1) + (r - p * P)] * 8; }
+                        out->lidx[cur_at++] = (uint16_t)(((c - (uint32_t)t * (uint32_t)T) * 8u) | ((idx[k] >> 31) << 15));
+                    }
+                }
+                for (int32_t t : tiles_of[p]) block_of[t] = -1;
+            }
+        }
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        cbm_tiling_free(out);
+        return CBM_ERR_ALLOC;
+    }
+}
+
 int cbm_builder_create(const int32_t* row, const int32_t* col, int64_t E, int32_t N, int32_t threads,
                        cbm_builder** out) {
     if (!out) return CBM_ERR_NULL;

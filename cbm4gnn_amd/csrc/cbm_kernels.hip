@@ -353,6 +353,136 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// (1c) SpMM over blocks of entries that cluster: the rows are cut into panels of kPanelRows, the
+// columns into tiles of TILE rows of X, and the entries of every (panel, tile) block that holds
+// enough of them are stored apart ("local" entries) as 16-bit offsets into the tile.  A workgroup
+// takes a (panel, slab) pair: for each of the panel's blocks it stages the tile's 128-byte slab of
+// X rows in LDS and its 16 waves gather from there at LDS bandwidth, where the slab kernel pulls
+// every 128-byte line through L1 and L2.
+//   * Every 8-lane group of a wave owns ONE ROW of the panel (a wave works on 8 rows in lockstep,
+//     2 such sets per wave = 256 rows per workgroup) and keeps that row's running sum in 4
+//     registers per lane across all blocks: no cross-lane traffic at all, and a row's local
+//     entries are added strictly in storage order (blocks by ascending tile, columns ascending).
+//   * A lane group reads its row's entries as one 16-byte vector per 8 entries; every (row, block)
+//     segment is padded to a multiple of 8 entries with the index of an all-zero row kept behind
+//     the tile in LDS, and a group whose segment is shorter than its neighbours' gathers that row:
+//     no coefficient, no masking -- per gather 1 unpack, 1 address op, 1 ds_read_b128, 4 adds.
+//   * lidx[k] = (row of X - first row of the tile) * 8 | sign << 15  (pre-multiplied so that the
+//     byte offset into LDS is (lidx + float4 index of the lane) << 4).
+// At the end the sums are added to what the slab kernel wrote for the remaining ("remote") entries
+// of the row, scaled (left scale of the normalised multiply), passed through the ReLU if asked,
+// and stored.  Order of the fp32 sums per output element: (remote part as the slab kernel sums
+// it) + (local entries in storage order, starting from 0).
+// ---------------------------------------------------------------------------------------------
+constexpr int kPanelRows = CBM_TILING_PANEL_ROWS;           // rows of the matrix per panel
+constexpr int kTiledWaves = 16;            // one 1024-thread workgroup
+constexpr int kTiledSets = kPanelRows / (kTiledWaves * 8);   // sets of 8 rows per wave
+
+template <int TILE, bool SIGNED>
+__global__ __launch_bounds__(kWave * kTiledWaves, TILE <= 512 ? 2 : 1) void spmm_tiled_local(
+    const int32_t* __restrict__ panel_ptr, const int32_t* __restrict__ blk_tile, const int32_t* __restrict__ seg,
+    const uint16_t* __restrict__ lidx, const float* __restrict__ W, float* __restrict__ Z,
+    const float* __restrict__ row_scale, int n, int d, int n_slabs, int n_panels, int64_t ldz, int relu, int vec_out) {
+    extern __shared__ float4 tile_lds[];                   // (TILE + 1) x 8 float4; row TILE is all zero
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sub = lane >> 3, li = lane & 7;
+    if (threadIdx.x < 8) tile_lds[TILE * 8 + threadIdx.x] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    constexpr uint32_t kPad = (uint32_t)(TILE * 8) | ((uint32_t)(TILE * 8) << 16);    // two entries of the zero row
+    // Workgroup b runs on XCD b % 8.  Items (panel-major, slab-minor) are cut into 8 contiguous
+    // ranges, one per XCD, and dealt cyclically to the XCD's workgroups: the workgroups of an XCD
+    // work on neighbouring panels at the same time, which share their tiles through the XCD's L2.
+    const int xcd = blockIdx.x % kXcds, j0 = blockIdx.x / kXcds, G = gridDim.x / kXcds;
+    const int items = n_panels * n_slabs;
+    const int chunk = (items + kXcds - 1) / kXcds;
+    const int item_end = min((xcd + 1) * chunk, items);
+    for (int item = xcd * chunk + j0; item < item_end; item += G) {
+        const int panel = item / n_slabs, slab = item % n_slabs;
+        float acc[kTiledSets][4];
+#pragma unroll
+        for (int t = 0; t < kTiledSets; t++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[t][e] = 0.0f;
+        const int b_beg = panel_ptr[panel], b_end = panel_ptr[panel + 1];
+        for (int b = b_beg; b < b_end; b++) {
+            const int base = blk_tile[b] * TILE;
+            const int rows = min(TILE, n - base);
+            // this lane group's segment in each set: panel row = set * 128 + wave * 8 + sub; seg[] counts in units of 8 entries
+            int s0[kTiledSets], len[kTiledSets];
+#pragma unroll
+            for (int t = 0; t < kTiledSets; t++) {
+                const int32_t* __restrict__ sg = seg + (int64_t)b * (kPanelRows + 1) + t * (kTiledWaves * 8) + wave * 8 + sub;
+                s0[t] = sg[0]; len[t] = sg[1] - s0[t];
+            }
+            __syncthreads();                               // the previous tile is no longer read
+            const float4* __restrict__ src = reinterpret_cast<const float4*>(W + ((int64_t)slab * n + base) * 32);
+            for (int i = threadIdx.x; i < rows * 8; i += kWave * kTiledWaves) tile_lds[i] = src[i];
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < kTiledSets; t++) {
+                int longest = len[t];                       // the wave iterates to its longest segment
+#pragma unroll
+                for (int off = 8; off < kWave; off <<= 1) longest = max(longest, __shfl_xor(longest, off, kWave));
+                const uint4* __restrict__ mine = reinterpret_cast<const uint4*>(lidx) + s0[t];
+                uint4 nxt = make_uint4(kPad, kPad, kPad, kPad);
+                if (0 < len[t]) nxt = mine[0];
+                for (int j = 0; j < longest; j++) {
+                    const uint4 cur = nxt;
+                    nxt = make_uint4(kPad, kPad, kPad, kPad);
+                    if (j + 1 < len[t]) nxt = mine[j + 1];
+                    const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
+                    float4 x[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const uint32_t p = (u & 1) ? (w[u >> 1] >> 16) : (w[u >> 1] & 0xffffu);
+                        x[u] = tile_lds[(SIGNED ? (p & 0x7fffu) : p) + li];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        if constexpr (SIGNED) {
+                            const uint32_t p = (u & 1) ? (w[u >> 1] >> 16) : (w[u >> 1] & 0xffffu);
+                            const float f = __uint_as_float(0x3f800000u | ((p & 0x8000u) << 16));
+                            acc[t][0] = fmaf(f, x[u].x, acc[t][0]); acc[t][1] = fmaf(f, x[u].y, acc[t][1]);
+                            acc[t][2] = fmaf(f, x[u].z, acc[t][2]); acc[t][3] = fmaf(f, x[u].w, acc[t][3]);
+                        } else {
+                            acc[t][0] += x[u].x; acc[t][1] += x[u].y; acc[t][2] += x[u].z; acc[t][3] += x[u].w;
+                        }
+                    }
+                }
+            }
+        }
+        // epilogue: every lane group adds its row's local sum to the remote part
+#pragma unroll
+        for (int t = 0; t < kTiledSets; t++) {
+            const int row = panel * kPanelRows + t * (kTiledWaves * 8) + wave * 8 + sub;
+            const int col = slab * 32 + li * 4;
+            if (row < n && col < d) {
+                float* __restrict__ zr = Z + (int64_t)row * ldz + col;
+                const float sc = row_scale ? row_scale[row] : 1.0f;
+                if (vec_out) {
+                    float4 z = *reinterpret_cast<const float4*>(zr);
+                    z.x = (z.x + acc[t][0]) * sc; z.y = (z.y + acc[t][1]) * sc;
+                    z.z = (z.z + acc[t][2]) * sc; z.w = (z.w + acc[t][3]) * sc;
+                    if (relu) {
+                        z.x = z.x < 0.0f ? 0.0f : z.x; z.y = z.y < 0.0f ? 0.0f : z.y;
+                        z.z = z.z < 0.0f ? 0.0f : z.z; z.w = z.w < 0.0f ? 0.0f : z.w;
+                    }
+                    *reinterpret_cast<float4*>(zr) = z;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (col + e < d) {
+                            float z = (zr[e] + acc[t][e]) * sc;
+                            if (relu) z = z < 0.0f ? 0.0f : z;
+                            zr[e] = z;
+                        }
+                }
+            }
+        }
+    }
+}
+
 // Slab-major copy of X: W[s][r][0 .. 32) = X[r][32 s .. 32 s + 32), zero where the column is >= d
 // (n_slabs * 32 may exceed d).  With the caller's row-major X a slab's lines sit a whole row (a
 // power of two for the usual widths) apart, which maps them onto a fraction of an XCD's L2
@@ -1265,6 +1395,80 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
                           stream);
     if (rc) return rc;
     // children of the root were scaled by the SpMM epilogue already
+    rc = cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, 0, stream);
+    if (rc || !relu || flat || n == 0 || d == 0) return rc;
+    const int64_t total = (int64_t)n * d, blocks = (total + 255) / 256;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    hipLaunchKernelGGL(relu_rows, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), Y, total, d, ldy);
+    return check_launch();
+}
+
+int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, float* Z, float* workspace, int32_t flags,
+                       int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
+    if (!t || !X || !Z || !workspace) return CBM_ERR_NULL;
+    if (!t->panel_ptr || !t->rowptr_r || (t->n_blocks > 0 && (!t->blk_tile || !t->seg || !t->lidx))) return CBM_ERR_NULL;
+    if (t->nnz_remote > 0 && !t->idx_r) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (int rc = check_matrix(n, d, ldz)) return rc;
+    if (t->tile_rows != 1024 && t->tile_rows != 512) return CBM_ERR_SHAPE;
+    if (t->n_panels != (n + kPanelRows - 1) / kPanelRows || t->n_blocks < 0) return CBM_ERR_SHAPE;
+    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
+    const bool ready = (flags & CBM_SPMM_WORKSPACE_READY) != 0;
+    // the local entries carry no coefficient: with m, the copy they gather from must be the scaled one
+    if (ready && ((m != nullptr) != ((flags & CBM_SPMM_WORKSPACE_PRESCALED) != 0))) return CBM_ERR_UNSUPPORTED;
+    if (!ready && (flags & CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
+    if (n == 0 || d == 0) return CBM_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const DeviceFacts* facts = device_facts();
+    if (!facts || facts->cus < kXcds) return CBM_ERR_LAUNCH;
+    if (!ready) {                                         // launch_spmm checks alignment and overlap of the workspace below
+        if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
+        const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+        if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
+            ranges_overlap(workspace, ws_bytes, Z, matrix_bytes(n, d, ldz)))
+            return CBM_ERR_SHAPE;
+        if (int rc = launch_relayout(X, workspace, n, d, ldx, s, nullptr, 0, m)) return rc;
+    }
+    // remote entries: the slab kernel from the copy; left scale and ReLU wait for the local part
+    const int remote_flags = CBM_SPMM_WORKSPACE_READY | (m ? CBM_SPMM_WORKSPACE_PRESCALED : 0);
+    if (int rc = launch_spmm<true>(t->rowptr_r, t->idx_r, t->nnz_remote, nullptr, m, nullptr, t->sched_r, X, Z, workspace,
+                                   remote_flags, n, d, ldx, ldz, s))
+        return rc;
+    // local entries: tiles of the copy staged in LDS; adds to Z, then scale and ReLU
+    const size_t bytes = (size_t)(t->tile_rows + 1) * 128;
+    const int n_slabs = padded_slab_count(d);
+    const int vec_out = (d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16)) ? 1 : 0;
+    const int G = facts->cus / kXcds;                     // 129 KB of LDS: one workgroup per CU
+    const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
+#define LAUNCH_TILED(T, S)                                                                                               \
+    do {                                                                                                                 \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S>),                                   \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)                   \
+            return CBM_ERR_LAUNCH;                                                                                       \
+        hipLaunchKernelGGL((spmm_tiled_local<T, S>), dim3(G * kXcds), dim3(kWave * kTiledWaves), bytes, s, t->panel_ptr, \
+                           t->blk_tile, t->seg, t->lidx, workspace, Z, t->row_scale, n, d, n_slabs, t->n_panels, ldz,    \
+                           relu, vec_out);                                                                               \
+    } while (0)
+    if (t->tile_rows == 1024) { if (t->has_negative) LAUNCH_TILED(1024, true); else LAUNCH_TILED(1024, false); }
+    else { if (t->has_negative) LAUNCH_TILED(512, true); else LAUNCH_TILED(512, false); }
+#undef LAUNCH_TILED
+    return check_launch();
+}
+
+int cbm_spmm_update_tiled_f32(const cbm_tiling_dev* t, const float* m, const int32_t* parent, const int32_t* order,
+                              const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
+                              const float* X, float* Y, float* workspace, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
+                              int32_t flags, void* stream) {
+    if (!parent) return CBM_ERR_NULL;
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+        return CBM_ERR_UNSUPPORTED;
+    const bool relu = (flags & CBM_UPDATE_RELU) != 0;
+    const bool flat = n_levels <= 1;
+    int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
+    if (flags & CBM_UPDATE_WORKSPACE_PRESCALED) spmm_flags |= CBM_SPMM_WORKSPACE_PRESCALED;
+    if (relu && flat) spmm_flags |= CBM_SPMM_RELU;
+    int rc = cbm_spmm_tiled_f32(t, m, X, Y, workspace, spmm_flags, n, d, ldx, ldy, stream);
+    if (rc) return rc;
     rc = cbm_propagate_f32(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, 0, stream);
     if (rc || !relu || flat || n == 0 || d == 0) return rc;
     const int64_t total = (int64_t)n * d, blocks = (total + 255) / 256;

@@ -153,6 +153,37 @@ void cbm_build_host_timings(double* out4);
 int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
                       int32_t* sched_out);
 
+/* Split of a packed delta matrix (rowptr, idx as in cbm_format) into entries that cluster and the
+ * rest, for cbm_spmm_tiled_f32.  Rows are cut into panels of CBM_TILING_PANEL_ROWS, columns into
+ * tiles of tile_rows (1024); a (panel, tile) block that holds at least min_block_entries entries
+ * becomes a "local" block, whose tile of X the kernel stages in LDS; every other entry is "remote"
+ * and stays in an ordinary packed CSR.
+ *   panel_ptr[n_panels + 1]   blocks of each panel (ascending tile)
+ *   blk_tile[n_blocks]        tile index of each block (first row of X it covers = tile * tile_rows)
+ *   seg[n_blocks][panel_rows + 1]  per block and panel row: start of the row's segment in lidx, in
+ *                             units of 8 entries; a segment holds the row's entries inside the
+ *                             block, columns ascending, padded to a multiple of 8
+ *   lidx[nnz_local_padded]    (row of X - first row of the tile) * 8 | (negative ? 1 << 15 : 0);
+ *                             padding = tile_rows * 8, the all-zero row behind the tile
+ *   rowptr_r / idx_r          the remote entries, packed like idx, columns ascending
+ * threads <= 0 means all OpenMP threads.  HOST pointers; release with cbm_tiling_free.  No reference
+ * counterpart: the reference hands its delta matrix to mkl_sparse_s_mm as it is
+ * (cbm_extensions.cpp:1133-1159). */
+#define CBM_TILING_PANEL_ROWS 256
+typedef struct cbm_tiling {
+    int32_t n, tile_rows, panel_rows, n_panels, n_blocks, has_negative;
+    int64_t nnz_local, nnz_local_padded, nnz_remote;
+    int32_t* panel_ptr;
+    int32_t* blk_tile;
+    int32_t* seg;
+    uint16_t* lidx;
+    int32_t* rowptr_r;
+    uint32_t* idx_r;
+} cbm_tiling;
+int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t tile_rows, int64_t min_block_entries,
+                  int32_t threads, cbm_tiling* out);
+void cbm_tiling_free(cbm_tiling* t);
+
 /* ------------------------------------------------------------------ libcbm_hip.so ----------- */
 
 const char* cbm_version(void);
@@ -282,6 +313,43 @@ int cbm_spmm_update_static_f32(const int32_t* rowptr_dev, const uint32_t* idx_de
                                const int32_t* order_dev, const int32_t* level_off_dev,
                                const int32_t* level_off_host, int32_t n_levels, const float* X_dev, float* Y_dev,
                                int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream);
+
+/* A tiling (cbm_tile_rows) in DEVICE memory, plus what the two kernels of the tiled multiply need:
+ *   sched_r    cbm_schedule_rows(rowptr_r, NULL, NULL) of the remote part, or NULL
+ *   row_scale  [n] left scale per row: m[r] for children of the root, 1 elsewhere; NULL = no scale
+ * The struct itself lives in HOST memory. */
+typedef struct cbm_tiling_dev {
+    int32_t n_panels, n_blocks, tile_rows, has_negative;
+    int64_t nnz_remote;
+    const int32_t* panel_ptr;
+    const int32_t* blk_tile;
+    const int32_t* seg;
+    const uint16_t* lidx;
+    const int32_t* rowptr_r;
+    const uint32_t* idx_r;
+    const int32_t* sched_r;
+    const float* row_scale;
+} cbm_tiling_dev;
+
+/* cbm_spmm_f32 for a matrix whose entries cluster (community structure): Z = D diag(m) X with the
+ * remote entries gathered by the slab kernel and the local blocks gathered from tiles of X staged
+ * in LDS (1024 rows x 128 bytes per workgroup), which spares them the trip through L1 and L2.
+ * workspace is REQUIRED (cbm_relayout_floats(n, d) floats): both kernels read the slab-major
+ * copy, scaled by m when m is given (so no entry carries a coefficient).  flags: CBM_SPMM_RELU;
+ * CBM_SPMM_WORKSPACE_READY (with m: together with CBM_SPMM_WORKSPACE_PRESCALED).  Per output
+ * element the fp32 sum is (remote entries, summed as cbm_spmm_f32 sums a row) + (local entries,
+ * one after the other in ascending column order, starting from zero), then the left scale, then
+ * the ReLU.  Worth it when most entries are local: 232 965 rows x 491 entries, 89 % of them in
+ * blocks of a 50-community graph, d = 128: 1.99 ms against 2.78 ms for cbm_spmm_f32.
+ * Replaces the same mkl_sparse_s_mm call as cbm_spmm_f32 (cbm_extensions.cpp:1133-1159). */
+int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m_dev, const float* X_dev, float* Z_dev, float* workspace_dev,
+                       int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream);
+
+/* cbm_spmm_update_f32 on a tiling: cbm_spmm_tiled_f32 followed by cbm_propagate_f32. */
+int cbm_spmm_update_tiled_f32(const cbm_tiling_dev* t, const float* m_dev, const int32_t* parent_dev,
+                              const int32_t* order_dev, const int32_t* level_off_dev, const int32_t* level_off_host,
+                              int32_t n_levels, const float* X_dev, float* Y_dev, float* workspace_dev, int32_t n,
+                              int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream);
 
 /* Row intersections for the builder on the GPU: appends to pairs[] every (i, j > i, s) with
  * s = |row_i ^ row_j| and 2 s > min(nnz_i, nnz_j) + alpha, in no particular order, and adds their

@@ -58,6 +58,10 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
     fma(+-m[c], x[c], acc); by default whichever the multiply through ``cbm_matrix`` uses."""
     col, sign = mat.columns()
     m = orc.col_multiplier(ei, n) if normalized else None
+    if groups is None and prescaled is None and mat.relayout and mat.is_tiled():
+        z = oracle_delta_spmm(orc, mat, ei, n, x, normalized)
+        return (orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads) if normalized
+                else orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads))
     g = mat_groups(mat, x.shape[1]) if groups is None else groups
     if prescaled is None:                                  # the copy is only made for the slab kernel (g > 1)
         prescaled = normalized and brings_workspace(mat.relayout, mat.nnz, n, x.shape[1]) and mat_groups(mat, x.shape[1]) > 1
@@ -71,12 +75,35 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
                            mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads, groups=g)
 
 
+def tiled_split(mat):
+    """Per delta entry: does it lie in a (256-row panel, 1024-column tile) block that holds at least
+    ``tile_min_block_entries`` entries -- the definition of the local part of the tiled multiply."""
+    n = mat.num_rows
+    rp = mat.rowptr.numpy().astype(np.int64)
+    row = np.repeat(np.arange(n), np.diff(rp))
+    col = (mat.idx.numpy().view(np.uint32) & 0x7FFFFFFF).astype(np.int64)
+    n_tiles = (n + mat.tile_rows - 1) // mat.tile_rows
+    key = (row // 256) * n_tiles + col // mat.tile_rows
+    return np.bincount(key)[key] >= mat.tile_min_block_entries, row
+
+
 def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
     """The delta SpMM alone, Z = Delta diag(m) X, in the arithmetic and order of the multiply
     through ``cbm_matrix`` (see ``oracle_product``)."""
     col, sign = mat.columns()
     d = x.shape[1]
     g = mat_groups(mat, d)
+    if mat.relayout and mat.is_tiled():
+        # tiled multiply: (remote entries, 8 interleaved partial sums) + (local entries in column order,
+        # one after the other), on the copy of X scaled by m
+        local, row = tiled_split(mat)
+        xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
+        parts = []
+        for part, groups in ((~local, 8), (local, 1)):
+            rp = np.concatenate([[0], np.cumsum(np.bincount(row[part], minlength=n))]).astype(np.int32)
+            parts.append(orc.csr_spmm(rp, col.numpy()[part].astype(np.int32), sign.numpy()[part].astype(np.float32), xs,
+                                      groups=groups))
+        return parts[0] + parts[1]
     if not normalized:
         return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, groups=g)
     m = orc.col_multiplier(ei, n)
@@ -822,3 +849,44 @@ def test_gpu_built_format_counts_equal_the_oracle_build(orc):
         assert mat.nnz == fmt["nnz"] == int(fmt["d_row"].shape[0])
         assert orc.check_format(w.edge_index, w.n, mat.rowptr.numpy(), mat.idx.numpy().view(np.uint32),
                                 mat.mst_row.numpy(), mat.mst_col.numpy())
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+@pytest.mark.parametrize("alpha", [0, 10 ** 6])
+def test_tiled_multiply_against_oracle(orc, normalized, alpha):
+    """``tiling="on"``: local blocks gathered from LDS tiles, the rest by the slab kernel.  Bit for
+    bit against the oracle in the documented order -- (remote entries in 8 interleaved partial sums)
+    + (local entries one after the other) -- for signed deltas (alpha = 0) and a flat tree of
+    all-positive entries (alpha huge), widths on both store paths, with and without the ReLU, the
+    SpMM alone, and the un-fused methods."""
+    n = 3000
+    ei = graphs.add_self_loops(graphs.sbm(n, 30, 0.6, 0.002, seed=5), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=normalized, tiling="on")
+    mat.tile_min_block_entries = 1000
+    assert mat.is_tiled()
+    info = mat.tiling_info
+    assert info["nnz_local"] > 0 and info["nnz_remote"] > 0 and info["has_negative"] == (alpha == 0)
+    assert (mat.n_levels > 2) == (alpha == 0)
+    off = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=normalized, tiling="off")
+    for d in (41, 128, 200):
+        say("tiled", normalized, alpha, d)
+        x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+        got = gpu_product(mat, x, normalized)
+        want = oracle_product(orc, mat, ei, n, x, normalized)
+        assert np.array_equal(got, want)
+        assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CBM
+        assert orc.max_rel_err(got, gpu_product(off, x, normalized)) <= 1e-5
+        xd = torch.from_numpy(x).cuda()
+        z = torch.full_like(xd, float("nan")); mat.omp_mkl_csr_spmm(xd, z)                  # the SpMM alone
+        assert np.array_equal(z.cpu().numpy(), oracle_delta_spmm(orc, mat, ei, n, x, normalized))
+        r = torch.full_like(xd, float("nan")); mat._run_spmm_update(xd, r, use_m=normalized, relu=True)
+        assert np.array_equal(r.cpu().numpy(), np.maximum(want, 0.0)) and float(r.min()) == 0.0
+        if normalized:                                      # un-fused: A diag(m) X
+            p = torch.full_like(xd, float("nan")); mat.omp_mkl_csr_spmm_update(xd, p)
+            zz = oracle_delta_spmm(orc, mat, ei, n, x, True)
+            assert np.array_equal(p.cpu().numpy(), orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), zz))
+    # backward of matmul runs on the same path (the graph is symmetric)
+    xg = torch.from_numpy(x).cuda().requires_grad_(True)
+    g = torch.randn((n, 200), generator=torch.Generator().manual_seed(1)).cuda()
+    (mat.matmul(xg) * g).sum().backward()
+    assert orc.max_rel_err(xg.grad.cpu().numpy(), orc.dense_product(ei, n, g.cpu().numpy(), normalized)) <= TOL_CBM

@@ -1,0 +1,98 @@
+"""Host side of the tiled multiply (no GPU): ``cbm_tile_rows`` splits the packed delta matrix into
+local blocks and remote entries exactly as defined -- a (256-row panel, 1024-column tile) block is
+local iff it holds at least ``min_block_entries`` entries -- and lays the local entries out as the
+kernel reads them (segments per block and panel row, padded to 8 with the zero-row index)."""
+import numpy as np
+import pytest
+import torch
+
+from cbm4gnn_amd import graphs
+from cbm4gnn_amd.cbm import cbm_matrix
+
+P, T = 256, 1024
+
+
+def split_by_definition(mat, min_block_entries):
+    """(local mask per delta entry, row per entry, column per entry, sign bit per entry), NumPy."""
+    n = mat.num_rows
+    rp = mat.rowptr.numpy().astype(np.int64)
+    idx = mat.idx.numpy().view(np.uint32)
+    row = np.repeat(np.arange(n), np.diff(rp))
+    col = (idx & 0x7FFFFFFF).astype(np.int64)
+    n_tiles = (n + T - 1) // T
+    key = (row // P) * n_tiles + col // T
+    cnt = np.bincount(key, minlength=((n + P - 1) // P) * n_tiles)
+    return cnt[key] >= min_block_entries, row, col, (idx >> 31).astype(np.int64), key, cnt, n_tiles
+
+
+def decode(th, n):
+    """Every local entry the tiling arrays hold, as sorted (row, col, negative) triples, checking
+    the layout on the way."""
+    pp, bt, seg, lidx = (th[k].numpy() for k in ("panel_ptr", "blk_tile", "seg", "lidx"))
+    lidx = lidx.view(np.uint16).astype(np.int64)
+    seg = seg.reshape(-1, P + 1).astype(np.int64)
+    assert pp[0] == 0 and pp[-1] == seg.shape[0] == bt.shape[0] and (np.diff(pp) >= 0).all()
+    flat = seg.ravel()
+    assert (np.diff(flat) >= 0).all() and flat[0] == 0 and flat[-1] * 8 == lidx.shape[0]
+    assert (seg[1:, 0] == seg[:-1, P]).all()                # blocks follow each other without a gap
+    out = []
+    pad = T * 8
+    for p in range(pp.shape[0] - 1):
+        assert (np.diff(bt[pp[p]:pp[p + 1]]) > 0).all()     # ascending tiles within a panel
+        for b in range(pp[p], pp[p + 1]):
+            for pr in range(P):
+                ent = lidx[seg[b, pr] * 8:seg[b, pr + 1] * 8]
+                real = ent[ent != pad]
+                k = real.shape[0]
+                assert (ent[:k] != pad).all() and (ent[k:] == pad).all() and ent.shape[0] - k < 8   # padding only at the end
+                off = (real & 0x7FFF) // 8
+                assert ((real & 0x7FFF) % 8 == 0).all() and (off < T).all() and (np.diff(off) > 0).all()
+                r = p * P + pr
+                assert k == 0 or r < n
+                out += [(r, int(bt[b]) * T + int(o), int(v >> 15)) for o, v in zip(off, real)]
+    return sorted(out)
+
+
+@pytest.mark.parametrize("n,blocks,p_in,alpha,thr", [(3000, 30, 0.6, 0, 64), (2600, 5, 0.08, 1, 300), (1500, 2, 0.08, 0, 1)])
+def test_tiling_is_the_defined_split(n, blocks, p_in, alpha, thr):
+    ei = graphs.add_self_loops(graphs.sbm(n, blocks, p_in, 0.002, seed=n), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, tiling="on")
+    mat.tile_min_block_entries = thr
+    th = mat._host_tiling()
+    assert th and mat.is_tiled()
+    local, row, col, neg, key, cnt, n_tiles = split_by_definition(mat, thr)
+    assert mat.tiling_info["nnz_local"] == int(local.sum()) and mat.tiling_info["nnz_remote"] == int((~local).sum())
+    assert th["has_negative"] == int(neg[local].any())
+    if p_in > 0.5:
+        assert neg.any() and mat.n_levels > 2               # the deltas really carry negative entries
+    assert decode(th, n) == sorted(zip(row[local].tolist(), col[local].tolist(), neg[local].tolist()))
+    # blocks = the (panel, tile) pairs at or above the threshold, in (panel, tile) order
+    want_blocks = np.nonzero(cnt >= thr)[0]
+    pp, bt = th["panel_ptr"].numpy(), th["blk_tile"].numpy()
+    got_blocks = np.concatenate([np.full(pp[p + 1] - pp[p], p) for p in range(pp.shape[0] - 1)]) * n_tiles + bt
+    assert np.array_equal(got_blocks, want_blocks)
+    # remote part: an ordinary packed CSR of the other entries, columns ascending, signs kept
+    rr, ir = th["rowptr_r"].numpy().astype(np.int64), th["idx_r"].numpy().view(np.uint32)
+    assert np.array_equal(np.repeat(np.arange(n), np.diff(rr)), row[~local])
+    assert np.array_equal(ir, mat.idx.numpy().view(np.uint32)[~local])
+    if thr == 1:
+        assert not (~local).any() and rr[-1] == 0           # everything is local
+
+
+def test_tiling_policy():
+    n = 3000
+    ei = torch.from_numpy(graphs.add_self_loops(graphs.sbm(n, 3, 0.08, 0.002, seed=1), n))
+    assert not cbm_matrix(ei, None, tiling="off").is_tiled()
+    assert not cbm_matrix(ei, None, tiling="auto").is_tiled()        # far too small for "auto"
+    forced = cbm_matrix(ei, None, tiling="on")
+    forced.tile_min_block_entries = 10 ** 9                           # no block reaches it
+    assert not forced.is_tiled() and forced.tiling_info["n_blocks"] == 0
+    with pytest.raises(ValueError):
+        cbm_matrix(ei, None, tiling="sometimes")
+    # "auto" on a large matrix decides by the share of entries that fall into blocks
+    big = graphs.add_self_loops(graphs.sbm(20_000, 8, 0.03, 0.0001, seed=2), 20_000)   # ~75 entries per row, 8 communities
+    a = cbm_matrix(torch.from_numpy(big), None, alpha=10 ** 6, tiling="auto")
+    assert a.is_tiled() and a.tiling_info["local_fraction"] > 0.8
+    scattered = graphs.add_self_loops(graphs.erdos_renyi(20_000, 0.002, 3), 20_000)     # ~40 entries per row, no structure
+    b = cbm_matrix(torch.from_numpy(scattered), None, alpha=10 ** 6, tiling="auto")
+    assert not b.is_tiled() and b.tiling_info["local_fraction"] < 0.1
