@@ -756,15 +756,30 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                 }
                 for (int32_t r = p * P; r < r_end; r++) {
                     int64_t at_r = out->rowptr_r[r];
-                    // columns ascend within a row, so the entries of one block are consecutive: a running cursor per block
-                    int32_t cur_b = -1; int64_t cur_at = 0;
-                    for (int64_t k = rowptr[r]; k < rowptr[r + 1]; k++) {
-                        const uint32_t c = idx[k] & 0x7fffffffu;
-                        const int32_t t = (int32_t)(c / (uint32_t)T);
+                    // Columns ascend within a row, so the entries of one block form one run.  Inside a
+                    // segment the entries are stored parity-major: a row of even index lists its entries
+                    // in even columns first (ascending), then those in odd columns; a row of odd index
+                    // the other way round.  A 128-byte row of the tile covers half of the LDS banks,
+                    // chosen by the parity of its index; the kernel serves two neighbouring matrix
+                    // rows per cycle, and with this order they read opposite halves nearly always.
+                    const uint32_t first_parity = (uint32_t)(r & 1);
+                    int64_t k = rowptr[r];
+                    const int64_t k_end = rowptr[r + 1];
+                    while (k < k_end) {
+                        const uint32_t c0 = idx[k] & 0x7fffffffu;
+                        const int32_t t = (int32_t)(c0 / (uint32_t)T);
                         const int32_t b = block_of[t];
-                        if (b < 0) { out->idx_r[at_r++] = idx[k]; continue; }
-                        if (b != cur_b) { cur_b = b; cur_at = (int64_t)out->seg[(size_t)b * (P + 1) + (r - p * P)] * 8; }
-                        out->lidx[cur_at++] = (uint16_t)(((c - (uint32_t)t * (uint32_t)T) * 8u) | ((idx[k] >> 31) << 15));
+                        if (b < 0) { out->idx_r[at_r++] = idx[k++]; continue; }
+                        int64_t k1 = k;
+                        while (k1 < k_end && (int32_t)((idx[k1] & 0x7fffffffu) / (uint32_t)T) == t) k1++;
+                        int64_t at = (int64_t)out->seg[(size_t)b * (P + 1) + (r - p * P)] * 8;
+                        for (int pass = 0; pass < 2; pass++)
+                            for (int64_t q = k; q < k1; q++) {
+                                const uint32_t c = idx[q] & 0x7fffffffu;
+                                if (((c & 1u) == first_parity) != (pass == 0)) continue;
+                                out->lidx[at++] = (uint16_t)(((c - (uint32_t)t * (uint32_t)T) * 8u) | ((idx[q] >> 31) << 15));
+                            }
+                        k = k1;
                     }
                 }
                 for (int32_t t : tiles_of[p]) block_of[t] = -1;

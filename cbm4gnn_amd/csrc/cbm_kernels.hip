@@ -375,12 +375,13 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 // and stored.  Order of the fp32 sums per output element: (remote part as the slab kernel sums
 // it) + (local entries in storage order, starting from 0).
 // ---------------------------------------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));      // a native 16-byte vector (stays in registers)
 constexpr int kPanelRows = CBM_TILING_PANEL_ROWS;           // rows of the matrix per panel
 constexpr int kTiledWaves = 16;            // one 1024-thread workgroup
 constexpr int kTiledSets = kPanelRows / (kTiledWaves * 8);   // sets of 8 rows per wave
 
 template <int TILE, bool SIGNED>
-__global__ __launch_bounds__(kWave * kTiledWaves, TILE <= 512 ? 2 : 1) void spmm_tiled_local(
+__global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_tiled_local(
     const int32_t* __restrict__ panel_ptr, const int32_t* __restrict__ blk_tile, const int32_t* __restrict__ seg,
     const uint16_t* __restrict__ lidx, const float* __restrict__ W, float* __restrict__ Z,
     const float* __restrict__ row_scale, int n, int d, int n_slabs, int n_panels, int64_t ldz, int relu, int vec_out) {
@@ -405,9 +406,20 @@ __global__ __launch_bounds__(kWave * kTiledWaves, TILE <= 512 ? 2 : 1) void spmm
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[t][e] = 0.0f;
         const int b_beg = panel_ptr[panel], b_end = panel_ptr[panel + 1];
+        // The tile of block b + 1 is fetched into registers while block b is gathered from LDS, so
+        // that between two blocks only the LDS stores and two barriers are exposed.
+        constexpr int kStage = TILE * 8 / (kWave * kTiledWaves);          // float4 per thread and tile
+        f32x4 stage[kStage];
+#define CBM_FETCH_TILE(B)                                                                                            \
+    do {                                                                                                             \
+        const int base_ = blk_tile[B] * TILE;                                                                        \
+        const int rows8_ = min(TILE, n - base_) * 8;                                                                 \
+        const f32x4* __restrict__ src_ = reinterpret_cast<const f32x4*>(W + ((int64_t)slab * n + base_) * 32);       \
+        _Pragma("unroll") for (int i_ = 0; i_ < kStage; i_++)   /* all loads in flight together; rows past the */    \
+            stage[i_] = src_[min(i_ * (kWave * kTiledWaves) + (int)threadIdx.x, rows8_ - 1)]; /* matrix: never gathered */ \
+    } while (0)
+        if (b_beg < b_end) CBM_FETCH_TILE(b_beg);
         for (int b = b_beg; b < b_end; b++) {
-            const int base = blk_tile[b] * TILE;
-            const int rows = min(TILE, n - base);
             // this lane group's segment in each set: panel row = set * 128 + wave * 8 + sub; seg[] counts in units of 8 entries
             int s0[kTiledSets], len[kTiledSets];
 #pragma unroll
@@ -416,22 +428,22 @@ __global__ __launch_bounds__(kWave * kTiledWaves, TILE <= 512 ? 2 : 1) void spmm
                 s0[t] = sg[0]; len[t] = sg[1] - s0[t];
             }
             __syncthreads();                               // the previous tile is no longer read
-            const float4* __restrict__ src = reinterpret_cast<const float4*>(W + ((int64_t)slab * n + base) * 32);
-            for (int i = threadIdx.x; i < rows * 8; i += kWave * kTiledWaves) tile_lds[i] = src[i];
+#pragma unroll
+            for (int i = 0; i < kStage; i++)
+                reinterpret_cast<f32x4*>(tile_lds)[i * (kWave * kTiledWaves) + threadIdx.x] = stage[i];
             __syncthreads();
+            if (b + 1 < b_end) CBM_FETCH_TILE(b + 1);
 #pragma unroll
             for (int t = 0; t < kTiledSets; t++) {
                 int longest = len[t];                       // the wave iterates to its longest segment
 #pragma unroll
                 for (int off = 8; off < kWave; off <<= 1) longest = max(longest, __shfl_xor(longest, off, kWave));
+                longest = __builtin_amdgcn_readfirstlane(longest);
                 const uint4* __restrict__ mine = reinterpret_cast<const uint4*>(lidx) + s0[t];
-                uint4 nxt = make_uint4(kPad, kPad, kPad, kPad);
-                if (0 < len[t]) nxt = mine[0];
-                for (int j = 0; j < longest; j++) {
-                    const uint4 cur = nxt;
-                    nxt = make_uint4(kPad, kPad, kPad, kPad);
-                    if (j + 1 < len[t]) nxt = mine[j + 1];
-                    const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
+                const uint4 pad4 = make_uint4(kPad, kPad, kPad, kPad);
+                // 8 entries = one 16-byte vector; gathers, then adds in entry order
+                auto gather8 = [&](const uint4& v) {
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
                     float4 x[8];
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
@@ -449,9 +461,27 @@ __global__ __launch_bounds__(kWave * kTiledWaves, TILE <= 512 ? 2 : 1) void spmm
                             acc[t][0] += x[u].x; acc[t][1] += x[u].y; acc[t][2] += x[u].z; acc[t][3] += x[u].w;
                         }
                     }
+                };
+                // two vectors in flight, alternating registers: the load of vector j + 2 is issued
+                // before vector j is gathered
+                uint4 va = pad4, vb = pad4;
+                if (0 < len[t]) va = mine[0];
+                if (1 < len[t]) vb = mine[1];
+                for (int j = 0; j < longest; j += 2) {
+                    const uint4 ca = va;
+                    va = pad4;
+                    if (j + 2 < len[t]) va = mine[j + 2];
+                    gather8(ca);
+                    if (j + 1 < longest) {
+                        const uint4 cb = vb;
+                        vb = pad4;
+                        if (j + 3 < len[t]) vb = mine[j + 3];
+                        gather8(cb);
+                    }
                 }
             }
         }
+#undef CBM_FETCH_TILE
         // epilogue: every lane group adds its row's local sum to the remote part
 #pragma unroll
         for (int t = 0; t < kTiledSets; t++) {

@@ -162,7 +162,10 @@ int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float*
  *   blk_tile[n_blocks]        tile index of each block (first row of X it covers = tile * tile_rows)
  *   seg[n_blocks][panel_rows + 1]  per block and panel row: start of the row's segment in lidx, in
  *                             units of 8 entries; a segment holds the row's entries inside the
- *                             block, columns ascending, padded to a multiple of 8
+ *                             block, padded to a multiple of 8, parity-major: a row of even index
+ *                             lists its entries in even columns first (ascending), then those in odd
+ *                             columns (ascending); a row of odd index the other way round (the two
+ *                             rows the kernel serves in one LDS cycle then read opposite bank halves)
  *   lidx[nnz_local_padded]    (row of X - first row of the tile) * 8 | (negative ? 1 << 15 : 0);
  *                             padding = tile_rows * 8, the all-zero row behind the tile
  *   rowptr_r / idx_r          the remote entries, packed like idx, columns ascending
@@ -338,8 +341,8 @@ typedef struct cbm_tiling_dev {
  * copy, scaled by m when m is given (so no entry carries a coefficient).  flags: CBM_SPMM_RELU;
  * CBM_SPMM_WORKSPACE_READY (with m: together with CBM_SPMM_WORKSPACE_PRESCALED).  Per output
  * element the fp32 sum is (remote entries, summed as cbm_spmm_f32 sums a row) + (local entries,
- * one after the other in ascending column order, starting from zero), then the left scale, then
- * the ReLU.  Worth it when most entries are local: 232 965 rows x 491 entries, 89 % of them in
+ * one after the other in storage order -- blocks by ascending tile, parity-major inside a block,
+ * see cbm_tile_rows -- starting from zero), then the left scale, then the ReLU.  Worth it when most entries are local: 232 965 rows x 491 entries, 89 % of them in
  * blocks of a 50-community graph, d = 128: 1.99 ms against 2.78 ms for cbm_spmm_f32.
  * Replaces the same mkl_sparse_s_mm call as cbm_spmm_f32 (cbm_extensions.cpp:1133-1159). */
 int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m_dev, const float* X_dev, float* Z_dev, float* workspace_dev,

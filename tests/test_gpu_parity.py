@@ -98,12 +98,14 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         # one after the other), on the copy of X scaled by m
         local, row = tiled_split(mat)
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
-        parts = []
-        for part, groups in ((~local, 8), (local, 1)):
-            rp = np.concatenate([[0], np.cumsum(np.bincount(row[part], minlength=n))]).astype(np.int32)
-            parts.append(orc.csr_spmm(rp, col.numpy()[part].astype(np.int32), sign.numpy()[part].astype(np.float32), xs,
-                                      groups=groups))
-        return parts[0] + parts[1]
+        c, sg = col.numpy(), sign.numpy().astype(np.float32)
+        rp = np.concatenate([[0], np.cumsum(np.bincount(row[~local], minlength=n))]).astype(np.int32)
+        remote = orc.csr_spmm(rp, c[~local].astype(np.int32), sg[~local], xs, groups=8)
+        # local entries in storage order: by tile, then the columns of the row's own parity, then the others
+        lr, lc, ls = row[local], c[local], sg[local]
+        order = np.lexsort((lc, (lc + lr) % 2, lc // mat.tile_rows, lr))
+        rp = np.concatenate([[0], np.cumsum(np.bincount(lr, minlength=n))]).astype(np.int32)
+        return remote + orc.csr_spmm(rp, lc[order].astype(np.int32), ls[order], xs, groups=1)
     if not normalized:
         return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, groups=g)
     m = orc.col_multiplier(ei, n)
@@ -856,7 +858,7 @@ def test_gpu_built_format_counts_equal_the_oracle_build(orc):
 def test_tiled_multiply_against_oracle(orc, normalized, alpha):
     """``tiling="on"``: local blocks gathered from LDS tiles, the rest by the slab kernel.  Bit for
     bit against the oracle in the documented order -- (remote entries in 8 interleaved partial sums)
-    + (local entries one after the other) -- for signed deltas (alpha = 0) and a flat tree of
+    + (local entries one after the other in storage order) -- for signed deltas (alpha = 0) and a flat tree of
     all-positive entries (alpha huge), widths on both store paths, with and without the ReLU, the
     SpMM alone, and the un-fused methods."""
     n = 3000

@@ -46,8 +46,12 @@ def decode(th, n):
                 k = real.shape[0]
                 assert (ent[:k] != pad).all() and (ent[k:] == pad).all() and ent.shape[0] - k < 8   # padding only at the end
                 off = (real & 0x7FFF) // 8
-                assert ((real & 0x7FFF) % 8 == 0).all() and (off < T).all() and (np.diff(off) > 0).all()
+                assert ((real & 0x7FFF) % 8 == 0).all() and (off < T).all()
                 r = p * P + pr
+                # parity-major: the columns of the row's own parity first, each half ascending
+                first = off[off % 2 == r % 2]
+                assert np.array_equal(off, np.concatenate([first, off[off % 2 != r % 2]]))
+                assert (np.diff(first) > 0).all() and (np.diff(off[off % 2 != r % 2]) > 0).all()
                 assert k == 0 or r < n
                 out += [(r, int(bt[b]) * T + int(o), int(v >> 15)) for o, v in zip(off, real)]
     return sorted(out)
