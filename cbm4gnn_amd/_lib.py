@@ -56,6 +56,8 @@ class CbmTilingDev(C.Structure):
         ("nnz_remote", C.c_int64),
         ("panel_ptr", C.c_void_p), ("blk_tile", C.c_void_p), ("seg", C.c_void_p), ("lidx", C.c_void_p),
         ("rowptr_r", C.c_void_p), ("idx_r", C.c_void_p), ("sched_r", C.c_void_p), ("row_scale", C.c_void_p),
+        ("n_sched_r", C.c_int32), ("n_long", C.c_int32), ("n_pieces", C.c_int32), ("reserved", C.c_int32),
+        ("long_rows", C.c_void_p),
     ]
 
 
@@ -69,6 +71,8 @@ HOST_SYMBOLS = {
     "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
     "cbm_build_host_timings": (None, [C.POINTER(C.c_double)]),
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
+    "cbm_schedule_split_count": (C.c_int64, [_P, _I32, _I32, C.POINTER(C.c_int32)]),
+    "cbm_schedule_rows_split": (C.c_int, [_P, _P, _P, _I32, _I32, _P, _P]),
     "cbm_tile_rows": (C.c_int, [_P, _P, _I32, _I32, _I64, _I32, C.POINTER(CbmTiling)]),
     "cbm_tiling_free": (None, [C.POINTER(CbmTiling)]),
     "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),
@@ -94,6 +98,7 @@ HIP_SYMBOLS = {
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_tiled_workspace_floats": (C.c_int64, [C.POINTER(CbmTilingDev), _I32, _I32]),
     "cbm_spmm_tiled_f32": (C.c_int, [C.POINTER(CbmTilingDev), _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),
     "cbm_spmm_update_tiled_f32": (C.c_int, [C.POINTER(CbmTilingDev), _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64,
                                             _I64, _I32, _P]),

@@ -380,50 +380,86 @@ class cbm_matrix:
         self.tile_min_local_fraction = 0.8
         self._tiling_host = None            # None: not computed; False: computed and rejected; dict: arrays
         self.tiling_info = None
+        # Rows with more delta entries than this are cut into pieces of this many entries that different
+        # wavefronts gather (``cbm_schedule_rows_split``); 0 = never cut.  A hub row of a power-law graph
+        # would otherwise keep one wavefront per slab busy long after all others have finished.
+        self.split_chunk = 2048
 
     def _host_tiling(self):
-        """The split of the delta matrix into local blocks and remote entries (``cbm_tile_rows``), or
-        False when the policy or the matrix rules it out.  Computed once."""
+        """What the plan-based multiply (``cbm_spmm_tiled_f32``) needs on the host, or False when this
+        matrix does not use it: the split of the delta matrix into local blocks and remote entries
+        (``cbm_tile_rows``) when the tiling policy and the matrix call for it, and/or the fact that
+        rows longer than ``split_chunk`` exist and are to be cut.  Computed once."""
         if self._tiling_host is not None:
             return self._tiling_host
         n = self.num_rows
         self._tiling_host = False
-        if self.tiling == "off" or self.nnz == 0:
+        if self.nnz == 0:
             return False
-        if self.tiling == "auto" and (n < 16 * self.tile_rows or self.nnz < 32 * n):
-            return False                                    # too small for tiles of 1024 rows to pay
-        t = _lib.CbmTiling()
-        rc = _lib.host_lib().cbm_tile_rows(_ptr(self.rowptr), _ptr(self.idx), n, self.tile_rows,
-                                           self.tile_min_block_entries, 0, C.byref(t))
-        try:
-            _lib.check(rc, "cbm_tile_rows")
-            info = {"n_blocks": int(t.n_blocks), "nnz_local": int(t.nnz_local), "nnz_remote": int(t.nnz_remote),
-                    "local_fraction": t.nnz_local / max(self.nnz, 1), "has_negative": bool(t.has_negative)}
-            self.tiling_info = info
-            if t.n_blocks == 0 or (self.tiling == "auto" and info["local_fraction"] < self.tile_min_local_fraction):
-                return False
+        cut = bool(self.split_chunk) and int((self.rowptr[1:] - self.rowptr[:-1]).max()) > int(self.split_chunk)
+        tile = self.tiling != "off" and not (self.tiling == "auto" and (n < 16 * self.tile_rows or self.nnz < 32 * n))
+        arrays = None
+        if tile:                                            # "auto" on small matrices: tiles of 1024 rows cannot pay
+            t = _lib.CbmTiling()
+            rc = _lib.host_lib().cbm_tile_rows(_ptr(self.rowptr), _ptr(self.idx), n, self.tile_rows,
+                                               self.tile_min_block_entries, 0, C.byref(t))
+            try:
+                _lib.check(rc, "cbm_tile_rows")
+                info = {"n_blocks": int(t.n_blocks), "nnz_local": int(t.nnz_local), "nnz_remote": int(t.nnz_remote),
+                        "local_fraction": t.nnz_local / max(self.nnz, 1), "has_negative": bool(t.has_negative)}
+                self.tiling_info = info
+                if t.n_blocks > 0 and not (self.tiling == "auto" and info["local_fraction"] < self.tile_min_local_fraction):
 
-            def take(ptr, count, dtype):
-                return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))
+                    def take(ptr, count, dtype):
+                        return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(dtype, copy=True))
 
-            p1 = t.panel_rows + 1
-            self._tiling_host = {
-                "n_panels": int(t.n_panels), "n_blocks": int(t.n_blocks), "tile_rows": int(t.tile_rows),
-                "has_negative": int(t.has_negative), "nnz_remote": int(t.nnz_remote),
-                "panel_ptr": take(t.panel_ptr, t.n_panels + 1, np.int32), "blk_tile": take(t.blk_tile, t.n_blocks, np.int32),
-                "seg": take(t.seg, t.n_blocks * p1, np.int32),
-                "lidx": take(t.lidx, t.nnz_local_padded, np.uint16).view(torch.int16),
-                "rowptr_r": take(t.rowptr_r, n + 1, np.int32),
-                "idx_r": (take(t.idx_r, t.nnz_remote, np.uint32).view(torch.int32) if t.nnz_remote
-                          else torch.empty(0, dtype=torch.int32)),
-            }
-        finally:
-            _lib.host_lib().cbm_tiling_free(C.byref(t))
+                    p1 = t.panel_rows + 1
+                    arrays = {
+                        "n_panels": int(t.n_panels), "n_blocks": int(t.n_blocks), "tile_rows": int(t.tile_rows),
+                        "has_negative": int(t.has_negative), "nnz_remote": int(t.nnz_remote),
+                        "panel_ptr": take(t.panel_ptr, t.n_panels + 1, np.int32), "blk_tile": take(t.blk_tile, t.n_blocks, np.int32),
+                        "seg": take(t.seg, t.n_blocks * p1, np.int32),
+                        "lidx": take(t.lidx, t.nnz_local_padded, np.uint16).view(torch.int16),
+                        "rowptr_r": take(t.rowptr_r, n + 1, np.int32),
+                        "idx_r": (take(t.idx_r, t.nnz_remote, np.uint32).view(torch.int32) if t.nnz_remote
+                                  else torch.empty(0, dtype=torch.int32)),
+                    }
+            finally:
+                _lib.host_lib().cbm_tiling_free(C.byref(t))
+        if arrays is None and cut:                          # no local blocks: the whole matrix is "remote"
+            arrays = {"n_panels": (n + 255) // 256, "n_blocks": 0, "tile_rows": self.tile_rows, "has_negative": 0,
+                      "nnz_remote": self.nnz, "panel_ptr": torch.zeros((n + 255) // 256 + 1, dtype=torch.int32),
+                      "rowptr_r": self.rowptr, "idx_r": self.idx}
+        if arrays is not None:
+            arrays["cut"] = bool(self.split_chunk) and \
+                int((arrays["rowptr_r"][1:] - arrays["rowptr_r"][:-1]).max()) > int(self.split_chunk)
+            self._tiling_host = arrays
         return self._tiling_host
 
     def is_tiled(self):
-        """Whether multiplies of this matrix take the tiled path (decides it on first call)."""
-        return bool(self._host_tiling())
+        """Whether multiplies of this matrix gather local blocks from LDS tiles (decides it on first call)."""
+        th = self._host_tiling()
+        return bool(th) and th["n_blocks"] > 0
+
+    def has_cut_rows(self):
+        """Whether the multiply cuts rows longer than ``split_chunk`` into pieces."""
+        th = self._host_tiling()
+        return bool(th) and th["cut"]
+
+    def _split_schedule(self, rowptr, parent, m):
+        """(sched [count, 4], long_rows [n_long, 4], pieces) of ``cbm_schedule_rows_split``, CPU tensors."""
+        n = rowptr.numel() - 1
+        n_long = C.c_int32()
+        count = _lib.host_lib().cbm_schedule_split_count(_ptr(rowptr), n, int(self.split_chunk), C.byref(n_long))
+        if count < 0:
+            raise ValueError("cbm_schedule_split_count: bad row offsets or chunk size")
+        sched = torch.empty((count, 4), dtype=torch.int32)
+        long_rows = torch.empty((max(n_long.value, 1), 4), dtype=torch.int32)
+        rc = _lib.host_lib().cbm_schedule_rows_split(_ptr(rowptr), _ptr(parent), _ptr(m), n, int(self.split_chunk), _ptr(sched),
+                                                     _ptr(long_rows))
+        _lib.check(rc, "cbm_schedule_rows_split")
+        long_rows = long_rows[:n_long.value]
+        return sched, long_rows, int(long_rows[:, 2].sum()) if n_long.value else 0
 
     # Settings the cached device arrays depend on: changing one drops the cache, so that a later
     # multiply never runs on coefficients or schedules derived from the old value.
@@ -538,9 +574,26 @@ class cbm_matrix:
             th = self._host_tiling()
             st["tiled"] = None
             if th:
-                tensors = {k: th[k].to(device) for k in ("panel_ptr", "blk_tile", "seg", "lidx", "rowptr_r", "idx_r")}
-                tensors["sched_r"] = schedule_rows(th["rowptr_r"], None, None).to(device)
-                if self.col_multiplier is not None:          # left scale: m[r] for children of the root
+                tiled = th["n_blocks"] > 0
+                if tiled:
+                    tensors = {k: th[k].to(device) for k in ("panel_ptr", "blk_tile", "seg", "lidx", "rowptr_r", "idx_r")}
+                else:                                        # the remote part is the matrix itself
+                    tensors = {"panel_ptr": th["panel_ptr"].to(device), "rowptr_r": st["rowptr"], "idx_r": st["idx"]}
+                # schedules of the remote part.  With local blocks the left scale is applied by their kernel
+                # (row_scale); without, by the schedule, which then exists with and without the scales.
+                scaled = (None, None) if (tiled or self.col_multiplier is None) else (self.parent, self.col_multiplier)
+                for name, (par, mm) in (("plain", (None, None)), ("scaled", scaled)):
+                    if name == "scaled" and par is None:
+                        continue
+                    if th["cut"]:
+                        sched, long_rows, pieces = self._split_schedule(th["rowptr_r"], par, mm)
+                        tensors["sched_" + name] = sched.to(device)
+                        tensors["long_" + name] = long_rows.to(device)
+                        tensors["n_long"], tensors["n_pieces"], tensors["n_sched"] = long_rows.size(0), pieces, sched.size(0)
+                    else:
+                        tensors["sched_" + name] = schedule_rows(th["rowptr_r"], par, mm).to(device)
+                        tensors["n_long"], tensors["n_pieces"], tensors["n_sched"] = 0, 0, 0
+                if tiled and self.col_multiplier is not None:    # left scale: m[r] for children of the root
                     scale = torch.where(self.parent < 0, self.col_multiplier, torch.ones_like(self.col_multiplier))
                     tensors["row_scale"] = scale.to(device)
                 st["tiled"] = tensors
@@ -550,15 +603,31 @@ class cbm_matrix:
     def _tiled_struct(self, st, with_scale):
         """``struct cbm_tiling_dev`` over the device tensors of ``st`` (host-side struct, per call)."""
         th, tt = self._tiling_host, st["tiled"]
+        tiled = th["n_blocks"] > 0
+        flavour = "scaled" if (with_scale and not tiled and "sched_scaled" in tt) else "plain"
+        ptr = lambda name: tt[name].data_ptr() if (name in tt and tt[name].numel()) else None
         return _lib.CbmTilingDev(th["n_panels"], th["n_blocks"], th["tile_rows"], th["has_negative"], th["nnz_remote"],
-                                 tt["panel_ptr"].data_ptr(), tt["blk_tile"].data_ptr(), tt["seg"].data_ptr(),
-                                 tt["lidx"].data_ptr(), tt["rowptr_r"].data_ptr(),
-                                 tt["idx_r"].data_ptr() if th["nnz_remote"] else None, tt["sched_r"].data_ptr(),
-                                 tt["row_scale"].data_ptr() if (with_scale and "row_scale" in tt) else None)
+                                 ptr("panel_ptr"), ptr("blk_tile"), ptr("seg"), ptr("lidx"), ptr("rowptr_r"), ptr("idx_r"),
+                                 ptr("sched_" + flavour), ptr("row_scale") if (with_scale and tiled) else None,
+                                 tt["n_sched"], tt["n_long"], tt["n_pieces"], 0, ptr("long_" + flavour))
 
-    def _tiled_workspace(self, xd):
-        floats = _lib.hip_lib().cbm_relayout_floats(xd.size(0), xd.size(1))
-        return torch.empty(max(int(floats), 1), dtype=torch.float32, device=xd.device)
+    def workspace_floats(self, n, d, device):
+        """Floats of workspace a multiply of an [n, d] matrix on ``device`` uses at most: the slab-major
+        copy of X, plus the piece sums of cut rows."""
+        floats = int(_lib.hip_lib().cbm_relayout_floats(n, d))
+        st = self._device_arrays(device)
+        if st["tiled"] is not None:
+            floats = max(floats, int(_lib.hip_lib().cbm_spmm_tiled_workspace_floats(C.byref(self._tiled_struct(st, False)), n, d)))
+        return max(floats, 1)
+
+    def _tiled_workspace(self, xd, workspace=None):
+        need = self.workspace_floats(xd.size(0), xd.size(1), xd.device)
+        if workspace is None:
+            return torch.empty(need, dtype=torch.float32, device=xd.device)
+        if workspace.numel() < need:
+            raise ValueError(f"workspace holds {workspace.numel()} floats, this multiply needs {need} "
+                             "(cbm_matrix.workspace_floats)")
+        return workspace
 
     def _coef(self, st, device):
         """``+-m[col]`` per delta entry on ``device`` (what the reference keeps as the fp32 values of
@@ -611,7 +680,7 @@ class cbm_matrix:
             raise ValueError("rhs and dst are on different devices")
         st = self._device_arrays(xd.device)
         if st["tiled"] is not None and self.relayout and not (workspace_ready and use_m and not workspace_prescaled):
-            ws = workspace if workspace is not None else self._tiled_workspace(xd)
+            ws = self._tiled_workspace(xd, workspace)
             flags = (_lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0) | \
                     (_lib.CBM_SPMM_WORKSPACE_PRESCALED if (workspace_prescaled and use_m) else 0)
             ts = self._tiled_struct(st, with_scale=use_m and scale_roots)
@@ -681,7 +750,7 @@ class cbm_matrix:
         st = self._device_arrays(xd.device)
         tiled = st["tiled"] is not None and self.relayout and not (workspace_ready and use_m and not workspace_prescaled)
         if tiled:
-            ws = workspace if workspace is not None else self._tiled_workspace(xd)
+            ws = self._tiled_workspace(xd, workspace)
         else:
             ws = workspace if workspace is not None else (_workspace(xd, yd, self.nnz) if self.relayout else None)
         if workspace_ready:

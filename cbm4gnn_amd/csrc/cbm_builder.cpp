@@ -631,6 +631,59 @@ int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float*
     }
 }
 
+int64_t cbm_schedule_split_count(const int32_t* rowptr, int32_t n, int32_t chunk, int32_t* n_long_out) {
+    if (!rowptr || n < 0 || chunk < 64) return -1;
+    int64_t count = 0;
+    int32_t n_long = 0;
+    for (int32_t r = 0; r < n; r++) {
+        const int64_t len = (int64_t)rowptr[r + 1] - rowptr[r];
+        if (len < 0) return -1;
+        if (len > chunk) { count += (len + chunk - 1) / chunk; n_long++; }
+        else count++;
+    }
+    if (n_long_out) *n_long_out = n_long;
+    return count;
+}
+
+int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n, int32_t chunk,
+                            int32_t* sched_out, int32_t* long_rows_out) {
+    if (!rowptr || !sched_out) return CBM_ERR_NULL;
+    int32_t n_long = 0;
+    const int64_t count = cbm_schedule_split_count(rowptr, n, chunk, &n_long);
+    if (count < 0 || count > INT32_MAX) return CBM_ERR_SHAPE;
+    if (n_long > 0 && !long_rows_out) return CBM_ERR_NULL;
+    try {
+        // descriptors of rows and pieces, then the same stable counting sort by gather rounds as cbm_schedule_rows
+        struct Item { int32_t start, end, row; float scale; };
+        std::vector<Item> items;
+        items.reserve((size_t)count);
+        int32_t slot = 0, at_long = 0;
+        for (int32_t r = 0; r < n; r++) {
+            const int32_t b = rowptr[r], e = rowptr[r + 1];
+            const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
+            if (e - b <= chunk) { items.push_back({b, e, r, scale}); continue; }
+            int32_t* lr = long_rows_out + 4 * (size_t)at_long++;
+            lr[0] = r; lr[1] = slot;
+            for (int32_t k = b; k < e; k += chunk) items.push_back({k, std::min(k + chunk, e), (slot++) | CBM_SCHED_PIECE, 1.0f});
+            lr[2] = slot - lr[1];
+            std::memcpy(&lr[3], &scale, sizeof(float));
+        }
+        int32_t max_rounds = 0;
+        for (const Item& it : items) max_rounds = std::max(max_rounds, (it.end - it.start + 63) / 64);
+        std::vector<int64_t> first(max_rounds + 2, 0);
+        for (const Item& it : items) first[max_rounds - (it.end - it.start + 63) / 64 + 1]++;
+        for (int32_t b = 0; b <= max_rounds; b++) first[b + 1] += first[b];
+        for (const Item& it : items) {
+            int32_t* o = sched_out + 4 * first[max_rounds - (it.end - it.start + 63) / 64]++;
+            o[0] = it.start; o[1] = it.end; o[2] = it.row;
+            std::memcpy(&o[3], &it.scale, sizeof(float));
+        }
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        return CBM_ERR_ALLOC;
+    }
+}
+
 void cbm_tiling_free(cbm_tiling* t) {
     if (!t) return;
     free(t->panel_ptr); free(t->blk_tile); free(t->seg); free(t->lidx); free(t->rowptr_r); free(t->idx_r);

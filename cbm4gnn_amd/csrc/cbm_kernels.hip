@@ -22,6 +22,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 #include <type_traits>
@@ -226,7 +227,10 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
     const float* __restrict__ X, float* __restrict__ Z, int n, int d, int vec_out, int n_slabs,
-    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz, int relu) {
+    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz, int relu, float* __restrict__ partials) {
+    // n is the number of row descriptors (rows of the matrix, unless the schedule cuts long rows
+    // into pieces: a descriptor whose row field has CBM_SCHED_PIECE set is a piece, and its sum goes
+    // to slot (row field & ~CBM_SCHED_PIECE) of `partials`, n_slabs x 32 floats per slot, unscaled).
     // d is the true feature width: slabs may reach past it (odd widths are zero-padded in the
     // slab-major copy) and nothing is stored beyond column d; vec_out says that rows of Z are
     // float4-addressable.
@@ -333,7 +337,9 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
             for (int off = LPE; off < kWave; off <<= 1)
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], off, kWave);
-            if (sub == 0) {
+            if (sub == 0 && (row & CBM_SCHED_PIECE)) {                  // a piece of a cut row: raw sum to its slot
+                store_vec<4>(partials + ((int64_t)(row & ~CBM_SCHED_PIECE) * n_slabs + slab) * kSlab + li * 4, acc);
+            } else if (sub == 0) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     acc[e] *= row_scale;                              // 1.0f unless a child of the root
@@ -748,6 +754,24 @@ __global__ __launch_bounds__(256) void relu_rows(float* __restrict__ Y, int64_t 
     if (v < 0.0f) *y = 0.0f;
 }
 
+// Rows that the schedule cut into pieces: Z[row] = (piece sums added in order, from 0) * scale,
+// then the ReLU if asked.  long_rows = { row, first slot, pieces, bits(scale) } per cut row; a slot
+// holds n_slabs x 32 floats.  blockIdx.x = cut row, threads along the columns.
+__global__ __launch_bounds__(256) void combine_pieces(const int4* __restrict__ long_rows, const float* __restrict__ partials,
+                                                      float* __restrict__ Z, int d, int n_slabs, int64_t ldz,
+                                                      int apply_scale, int relu) {
+    const int4 lr = long_rows[blockIdx.x];
+    const float scale = apply_scale ? __int_as_float(lr.w) : 1.0f;
+    const int64_t slot_floats = (int64_t)n_slabs * 32;
+    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < d; j += gridDim.y * blockDim.x) {
+        float acc = 0.0f;
+        for (int k = 0; k < lr.z; k++) acc += partials[(int64_t)(lr.y + k) * slot_floats + j];
+        acc *= scale;
+        if (relu) acc = acc < 0.0f ? 0.0f : acc;
+        Z[(int64_t)lr.x * ldz + j] = acc;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side: shape selection and dispatch
 // ---------------------------------------------------------------------------------------------
@@ -1066,10 +1090,13 @@ inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t 
     return CBM_OK;
 }
 
+// n_desc / partials: a schedule that cuts long rows has n_desc >= n descriptors and needs the scratch
+// area for the piece sums (slab kernel only); n_desc = 0 means one descriptor per row.
 template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* val, const float* m,
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
-                int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s) {
+                int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s, int32_t n_desc = 0,
+                float* partials = nullptr) {
     if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
     const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
     if ((flags & CBM_SPMM_WORKSPACE_PRESCALED) && (!PACKED || !m || !(flags & CBM_SPMM_WORKSPACE_READY)))
@@ -1115,14 +1142,15 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
             const int cap = per_wave * slab_waves_per_simd(nnz, n, lpe);
             if (cap > 0 && G > cap) G = cap;
             // no more waves than rows: with fewer rows than resident waves shrink the grid
+            const int n_rows = n_desc > 0 ? n_desc : n;         // descriptors the waves walk
             const int share = n_slabs >= kXcds ? 1 : kXcds / n_slabs;
-            const int need = (n + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
+            const int need = (n_rows + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
             if (G > need) G = need;
             const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
             const int vec_out = plan.vec_out ? 1 : 0;
 #define LAUNCH_SLAB(L, CF)                                                                                     \
     hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, CF, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, \
-                       val, m, parent, Xg, Z, n, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz, relu)
+                       val, m, parent, Xg, Z, n_rows, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz, relu, partials)
             switch (lpe * 4 + coef_mode) {
                 case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream); break;
                 case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign); break;
@@ -1136,6 +1164,7 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
         }
         if (ready) return CBM_ERR_LAUNCH;                 // no occupancy information: cannot honour the copy
     }
+    if (n_desc > 0) return CBM_ERR_UNSUPPORTED;           // a cut schedule runs on the slab kernel only
     const Tiling t = pick_tiling(d, ldx, ldz, X, Z);
     const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
 #define LAUNCH(V, C, F)                                                                              \
@@ -1433,9 +1462,17 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
     return check_launch();
 }
 
+int64_t cbm_spmm_tiled_workspace_floats(const cbm_tiling_dev* t, int32_t n, int32_t d) {
+    if (!t || n <= 0 || d <= 0) return 0;
+    return ((int64_t)n + (t->n_long > 0 ? t->n_pieces : 0)) * padded_slab_count(d) * 32;
+}
+
 int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, float* Z, float* workspace, int32_t flags,
                        int32_t n, int32_t d, int64_t ldx, int64_t ldz, void* stream) {
     if (!t || !X || !Z || !workspace) return CBM_ERR_NULL;
+    if (t->n_long < 0 || t->n_pieces < 0 || t->n_sched_r < 0) return CBM_ERR_SHAPE;
+    if (t->n_long > 0 && (!t->long_rows || !t->sched_r || t->n_sched_r < n || !aligned(t->long_rows, 16))) return CBM_ERR_NULL;
+    if (t->n_long == 0 && t->n_sched_r != 0 && t->n_sched_r != n) return CBM_ERR_SHAPE;
     if (!t->panel_ptr || !t->rowptr_r || (t->n_blocks > 0 && (!t->blk_tile || !t->seg || !t->lidx))) return CBM_ERR_NULL;
     if (t->nnz_remote > 0 && !t->idx_r) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
@@ -1459,17 +1496,28 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
             return CBM_ERR_SHAPE;
         if (int rc = launch_relayout(X, workspace, n, d, ldx, s, nullptr, 0, m)) return rc;
     }
-    // remote entries: the slab kernel from the copy; left scale and ReLU wait for the local part
-    const int remote_flags = CBM_SPMM_WORKSPACE_READY | (m ? CBM_SPMM_WORKSPACE_PRESCALED : 0);
+    // remote entries: the slab kernel from the copy.  With local blocks the left scale and the ReLU
+    // wait for the kernel of the local part; without any, this launch (and the combine pass for cut
+    // rows) is the whole multiply and applies them.
+    const bool has_local = t->n_blocks > 0;
+    const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
+    const int n_slabs = padded_slab_count(d);
+    float* partials = t->n_long > 0 ? workspace + (int64_t)n * n_slabs * 32 : nullptr;
+    const int remote_flags = CBM_SPMM_WORKSPACE_READY | (m ? CBM_SPMM_WORKSPACE_PRESCALED : 0) |
+                             ((relu && !has_local) ? CBM_SPMM_RELU : 0);
     if (int rc = launch_spmm<true>(t->rowptr_r, t->idx_r, t->nnz_remote, nullptr, m, nullptr, t->sched_r, X, Z, workspace,
-                                   remote_flags, n, d, ldx, ldz, s))
+                                   remote_flags, n, d, ldx, ldz, s, t->n_long > 0 ? t->n_sched_r : 0, partials))
         return rc;
+    if (t->n_long > 0) {                                  // pieces of cut rows -> their rows of Z
+        const dim3 grid((unsigned)t->n_long, (unsigned)std::min(8, (d + 255) / 256));
+        hipLaunchKernelGGL(combine_pieces, grid, dim3(256), 0, s, reinterpret_cast<const int4*>(t->long_rows), partials, Z,
+                           d, n_slabs, ldz, has_local ? 0 : 1, (relu && !has_local) ? 1 : 0);
+    }
+    if (!has_local) return check_launch();
     // local entries: tiles of the copy staged in LDS; adds to Z, then scale and ReLU
     const size_t bytes = (size_t)(t->tile_rows + 1) * 128;
-    const int n_slabs = padded_slab_count(d);
     const int vec_out = (d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16)) ? 1 : 0;
     const int G = facts->cus / kXcds;                     // 129 KB of LDS: one workgroup per CU
-    const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
 #define LAUNCH_TILED(T, S)                                                                                               \
     do {                                                                                                                 \
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S>),                                   \

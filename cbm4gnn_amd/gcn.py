@@ -119,14 +119,16 @@ class CBMGCNLayer(nn.Module):
         # m -- the entries then carry no coefficient -- than the copy costs: 233k rows x 128, 491
         # entries per row: 2.81 ms with the scaled copy, 3.08 ms gathered in place)
         in_place = False
-        if d % 32 == 0 and op.col_multiplier is None:
+        tiled = op._device_arrays(device)["tiled"] is not None or op.transposed()._device_arrays(device)["tiled"] is not None
+        if d % 32 == 0 and op.col_multiplier is None and not tiled:     # (the plan-based multiply always copies)
             padded = torch.empty((n, d + 32), dtype=torch.float32, device=device)[:, :d]
             in_place = lib.cbm_spmm_workspace_floats(n, d, _ld(padded), _ld(y), _ptr(padded), _ptr(y)) == 0
         h = padded if in_place else torch.empty((n, d), dtype=torch.float32, device=device)
         copy_h = (not in_place) and op.relayout and _wants_workspace(h, y, op.nnz)
         copy_g = op.relayout and _wants_workspace(gh, y, op.transposed().nnz)
-        floats = int(lib.cbm_relayout_floats(n, d))
-        ws = torch.empty(max(floats, 1), dtype=torch.float32, device=device) if (copy_h or copy_g or self.relu) else None
+        floats = max(op.workspace_floats(n, d, device), op.transposed().workspace_floats(n, d, device))
+        copy_h, copy_g = copy_h or tiled, copy_g or tiled
+        ws = torch.empty(floats, dtype=torch.float32, device=device) if (copy_h or copy_g or self.relu) else None
         self._cache = {"key": key, "h": h, "y": y, "gh": gh, "ws": ws, "copy_h": copy_h, "copy_g": copy_g,
                        "h_in_place": in_place}
         return self._cache

@@ -153,6 +153,20 @@ void cbm_build_host_timings(double* out4);
 int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
                       int32_t* sched_out);
 
+/* cbm_schedule_rows for matrices with very long rows (hubs of a power-law graph): a row with more
+ * than `chunk` entries (chunk >= 64) is cut into pieces of `chunk` entries, each with a descriptor
+ * of its own { start, end, slot | CBM_SCHED_PIECE, bits(1.0f) }, so that different wavefronts
+ * gather different pieces; a piece's sum goes to slot `slot` of a scratch area instead of Z, and
+ * the pieces of a row are added in order afterwards (no atomics: the result does not depend on
+ * which wavefront ran which piece).  long_rows_out gets 4 int32 per cut row: { row, first slot,
+ * number of pieces, bit pattern of the left scale }.  cbm_schedule_split_count returns the number
+ * of descriptors (and the number of cut rows), -1 on bad input.  Used through cbm_spmm_tiled_f32.
+ * HOST pointers.  No reference counterpart (MKL schedules rows internally). */
+#define CBM_SCHED_PIECE 0x40000000
+int64_t cbm_schedule_split_count(const int32_t* rowptr, int32_t n, int32_t chunk, int32_t* n_long_out);
+int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n, int32_t chunk,
+                            int32_t* sched_out, int32_t* long_rows_out);
+
 /* Split of a packed delta matrix (rowptr, idx as in cbm_format) into entries that cluster and the
  * rest, for cbm_spmm_tiled_f32.  Rows are cut into panels of CBM_TILING_PANEL_ROWS, columns into
  * tiles of tile_rows (1024); a (panel, tile) block that holds at least min_block_entries entries
@@ -317,8 +331,16 @@ int cbm_spmm_update_static_f32(const int32_t* rowptr_dev, const uint32_t* idx_de
                                const int32_t* level_off_host, int32_t n_levels, const float* X_dev, float* Y_dev,
                                int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream);
 
-/* A tiling (cbm_tile_rows) in DEVICE memory, plus what the two kernels of the tiled multiply need:
- *   sched_r    cbm_schedule_rows(rowptr_r, NULL, NULL) of the remote part, or NULL
+/* A tiling (cbm_tile_rows) in DEVICE memory, plus what the kernels of the tiled multiply need:
+ *   sched_r    row schedule of the remote part, or NULL (natural order).  With local blocks
+ *              (n_blocks > 0) its left scales must all be 1 (cbm_schedule_rows(rowptr_r, NULL, NULL)
+ *              or cbm_schedule_rows_split with parent = m = NULL): the kernel of the local part
+ *              applies row_scale.  Without local blocks (n_blocks = 0, e.g. cbm_tile_rows with a
+ *              min_block_entries no block reaches: the struct then only carries a split schedule)
+ *              the schedule carries the left scales and row_scale is not read.
+ *   n_sched_r  descriptors in sched_r; 0 means n (one per row, no row is cut)
+ *   n_long / long_rows   rows cut by cbm_schedule_rows_split, 4 int32 each; their piece sums use
+ *              (number of pieces) x 32 x ceil(d / 32) floats of the workspace behind the copy of X
  *   row_scale  [n] left scale per row: m[r] for children of the root, 1 elsewhere; NULL = no scale
  * The struct itself lives in HOST memory. */
 typedef struct cbm_tiling_dev {
@@ -332,12 +354,18 @@ typedef struct cbm_tiling_dev {
     const uint32_t* idx_r;
     const int32_t* sched_r;
     const float* row_scale;
+    int32_t n_sched_r, n_long, n_pieces, reserved;
+    const int32_t* long_rows;
 } cbm_tiling_dev;
+
+/* Floats of workspace cbm_spmm_tiled_f32 needs: the slab-major copy of X plus the piece sums of
+ * cut rows. */
+int64_t cbm_spmm_tiled_workspace_floats(const cbm_tiling_dev* t, int32_t n, int32_t d);
 
 /* cbm_spmm_f32 for a matrix whose entries cluster (community structure): Z = D diag(m) X with the
  * remote entries gathered by the slab kernel and the local blocks gathered from tiles of X staged
  * in LDS (1024 rows x 128 bytes per workgroup), which spares them the trip through L1 and L2.
- * workspace is REQUIRED (cbm_relayout_floats(n, d) floats): both kernels read the slab-major
+ * workspace is REQUIRED (cbm_spmm_tiled_workspace_floats(t, n, d) floats): both kernels read the slab-major
  * copy, scaled by m when m is given (so no entry carries a coefficient).  flags: CBM_SPMM_RELU;
  * CBM_SPMM_WORKSPACE_READY (with m: together with CBM_SPMM_WORKSPACE_PRESCALED).  Per output
  * element the fp32 sum is (remote entries, summed as cbm_spmm_f32 sums a row) + (local entries,

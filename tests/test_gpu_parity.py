@@ -58,7 +58,7 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
     fma(+-m[c], x[c], acc); by default whichever the multiply through ``cbm_matrix`` uses."""
     col, sign = mat.columns()
     m = orc.col_multiplier(ei, n) if normalized else None
-    if groups is None and prescaled is None and mat.relayout and mat.is_tiled():
+    if groups is None and prescaled is None and mat.relayout and (mat.is_tiled() or mat.has_cut_rows()):
         z = oracle_delta_spmm(orc, mat, ei, n, x, normalized)
         return (orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads) if normalized
                 else orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads))
@@ -87,12 +87,51 @@ def tiled_split(mat):
     return np.bincount(key)[key] >= mat.tile_min_block_entries, row
 
 
+def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8):
+    """CSR product in ``groups`` interleaved partial sums per row, where a row with more than
+    ``chunk`` entries is cut into pieces of ``chunk`` entries: each piece is summed like a row of its
+    own and the piece sums are then added one after the other, starting from zero -- the order of
+    ``cbm_schedule_rows_split`` + ``combine_pieces``.  chunk = 0: nothing is cut."""
+    rp = np.asarray(rp, np.int64)
+    n = rp.shape[0] - 1
+    lens = np.diff(rp)
+    long_rows = np.nonzero(lens > chunk)[0] if chunk else np.empty(0, np.int64)
+    if long_rows.size == 0:
+        return orc.csr_spmm(rp.astype(np.int32), col, sgn, xs, groups=groups)
+    starts, ends, owner = [], [], []
+    for r in long_rows:
+        for k in range(rp[r], rp[r + 1], chunk):
+            starts.append(k); ends.append(min(k + chunk, rp[r + 1])); owner.append(r)
+    # auxiliary matrix: the original rows (cut rows emptied) followed by one row per piece
+    keep = np.ones(col.shape[0], bool)
+    for r in long_rows:
+        keep[rp[r]:rp[r + 1]] = False
+    piece_idx = np.concatenate([np.arange(a, b) for a, b in zip(starts, ends)])
+    aux_col = np.concatenate([col[keep], col[piece_idx]])
+    aux_sgn = np.concatenate([sgn[keep], sgn[piece_idx]])
+    aux_len = np.concatenate([np.where(lens > chunk, 0, lens), np.array(ends) - np.array(starts)])
+    aux_rp = np.concatenate([[0], np.cumsum(aux_len)]).astype(np.int32)
+    y = orc.csr_spmm(aux_rp, aux_col.astype(np.int32), aux_sgn.astype(np.float32), xs, groups=groups)
+    z = y[:n].copy()
+    for r in long_rows:
+        acc = np.zeros(xs.shape[1], np.float32)
+        for p in np.nonzero(np.array(owner) == r)[0]:
+            acc = acc + y[n + p]
+        z[r] = acc
+    return z
+
+
 def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
     """The delta SpMM alone, Z = Delta diag(m) X, in the arithmetic and order of the multiply
     through ``cbm_matrix`` (see ``oracle_product``)."""
     col, sign = mat.columns()
     d = x.shape[1]
     g = mat_groups(mat, d)
+    if mat.relayout and not mat.is_tiled() and mat.has_cut_rows():
+        # long rows cut into pieces; the plan-based multiply always gathers from the (scaled) copy
+        xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
+        return grouped_with_cuts(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
+                                 mat.split_chunk)
     if mat.relayout and mat.is_tiled():
         # tiled multiply: (remote entries, 8 interleaved partial sums) + (local entries in column order,
         # one after the other), on the copy of X scaled by m
@@ -100,7 +139,7 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
         c, sg = col.numpy(), sign.numpy().astype(np.float32)
         rp = np.concatenate([[0], np.cumsum(np.bincount(row[~local], minlength=n))]).astype(np.int32)
-        remote = orc.csr_spmm(rp, c[~local].astype(np.int32), sg[~local], xs, groups=8)
+        remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs, mat.split_chunk if mat.has_cut_rows() else 0)
         # local entries in storage order: by tile, then the columns of the row's own parity, then the others
         lr, lc, ls = row[local], c[local], sg[local]
         order = np.lexsort((lc, (lc + lr) % 2, lc // mat.tile_rows, lr))
@@ -892,3 +931,88 @@ def test_tiled_multiply_against_oracle(orc, normalized, alpha):
     g = torch.randn((n, 200), generator=torch.Generator().manual_seed(1)).cuda()
     (mat.matmul(xg) * g).sum().backward()
     assert orc.max_rel_err(xg.grad.cpu().numpy(), orc.dense_product(ei, n, g.cpu().numpy(), normalized)) <= TOL_CBM
+
+
+def hub_graph(n, per_row, seed):
+    """Directed graph with one hub ROW: row 0 is adjacent to every column; every other row has a
+    self loop and ``per_row`` random columns.  (The hub is a row only: column 0 stays ordinary.)"""
+    rng = np.random.default_rng(seed)
+    rows = np.concatenate([np.zeros(n, np.int64), np.repeat(np.arange(1, n), per_row), np.arange(1, n)])
+    cols = np.concatenate([np.arange(n), rng.integers(0, n, size=(n - 1) * per_row), np.arange(1, n)])
+    ei = np.unique(np.stack([rows, cols]), axis=1)
+    return np.ascontiguousarray(ei.astype(np.int32))
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+def test_hub_row_is_cut_into_pieces(orc, normalized):
+    """A 200,000-entry hub row (and a second, 5,000-entry one): the schedule cuts them into pieces
+    of 2,048 entries that different wavefronts gather; the piece sums are added in order.  Bit for
+    bit against the oracle in that order, for both store paths, with the ReLU, and the SpMM alone."""
+    n = 200_000
+    ei = hub_graph(n, 6, seed=3)
+    second = np.stack([np.full(5000, 7, np.int32), np.arange(1000, 6000, dtype=np.int32)])   # row 7 gets 5,000 more
+    ei = np.ascontiguousarray(np.unique(np.concatenate([ei, second], axis=1), axis=1))
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+    lens = np.diff(mat.rowptr.numpy())
+    assert lens.max() > 190_000 and (lens > mat.split_chunk).sum() >= 2
+    assert mat.has_cut_rows() and not mat.is_tiled()
+    for d in (64, 41):
+        say("hub row", normalized, d)
+        x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+        got = gpu_product(mat, x, normalized)
+        want = oracle_product(orc, mat, ei, n, x, normalized)
+        assert np.array_equal(got, want)
+        # anchors that share no code with the oracle's SpMM: the hub row itself and a sample, in fp64
+        rows = np.concatenate([[0, 7], np.random.default_rng(1).choice(n, 200, replace=False)])
+        m = orc.col_multiplier(ei, n).astype(np.float64) if normalized else np.ones(n)
+        order = np.lexsort((ei[1], ei[0]))
+        rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))])
+        cs = ei[1][order]
+        for r in rows:
+            c = cs[rp[r]:rp[r + 1]]
+            ref = m[r] * (m[c][:, None] * x[c].astype(np.float64)).sum(axis=0)
+            assert np.abs(got[r] - ref).max() <= TOL_CBM * max(np.abs(ref).max(), 1e-3)
+        xd = torch.from_numpy(x).cuda()
+        r_ = torch.full_like(xd, float("nan")); mat._run_spmm_update(xd, r_, use_m=normalized, relu=True)
+        assert np.array_equal(r_.cpu().numpy(), np.maximum(want, 0.0))
+        z = torch.full_like(xd, float("nan")); mat.omp_mkl_csr_spmm(xd, z)
+        assert np.array_equal(z.cpu().numpy(), oracle_delta_spmm(orc, mat, ei, n, x, normalized))
+    # never cut: same product to rounding, and the cut version is the faster one by far
+    whole = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+    whole.split_chunk = 0
+    assert not whole.has_cut_rows()
+    assert orc.max_rel_err(gpu_product(whole, x, normalized), got) <= 1e-5
+
+
+def test_tiled_blocks_and_cut_rows_together(orc):
+    """Local blocks (a dense community among the first 2,000 nodes) and a hub row whose entries are
+    mostly remote and get cut: remote pieces -> combine -> local kernel (adds, scales, ReLU)."""
+    n = 20_000
+    hub = hub_graph(n, 4, seed=9)
+    dense = graphs.sbm(2000, 1, 0.3, 0.0, seed=9)
+    ei = np.ascontiguousarray(np.unique(np.concatenate([hub, dense], axis=1), axis=1).astype(np.int32))
+    for normalized in (False, True):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=10 ** 6, normalized=normalized, tiling="on")
+        mat.tile_min_block_entries = 1500
+        assert mat.is_tiled() and mat.has_cut_rows()
+        th = mat._host_tiling()
+        assert int(np.diff(th["rowptr_r"].numpy()).max()) > 4 * mat.split_chunk and mat.tiling_info["nnz_local"] > 100_000
+        for d in (96, 41):
+            say("tiled + cut", normalized, d)
+            x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+            got = gpu_product(mat, x, normalized)
+            assert np.array_equal(got, oracle_product(orc, mat, ei, n, x, normalized))
+            assert orc.max_rel_err(got[:3000], orc.csr_spmm(*_normalised_csr(orc, ei, n, normalized), x)[:3000]) <= TOL_CBM
+            xd = torch.from_numpy(x).cuda()
+            r_ = torch.full_like(xd, float("nan")); mat._run_spmm_update(xd, r_, use_m=normalized, relu=True)
+            assert np.array_equal(r_.cpu().numpy(), np.maximum(got, 0.0))
+
+
+def _normalised_csr(orc, ei, n, normalized):
+    order = np.lexsort((ei[1], ei[0]))
+    rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int32)
+    col = ei[1][order].astype(np.int32)
+    if not normalized:
+        return rp, col, None
+    m = orc.col_multiplier(ei, n)
+    return rp, col, (m[ei[0][order]] * m[col]).astype(np.float32)

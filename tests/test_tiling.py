@@ -100,3 +100,49 @@ def test_tiling_policy():
     scattered = graphs.add_self_loops(graphs.erdos_renyi(20_000, 0.002, 3), 20_000)     # ~40 entries per row, no structure
     b = cbm_matrix(torch.from_numpy(scattered), None, alpha=10 ** 6, tiling="auto")
     assert not b.is_tiled() and b.tiling_info["local_fraction"] < 0.1
+
+
+def test_split_schedule_covers_every_entry_once():
+    """``cbm_schedule_rows_split``: rows above the chunk size become pieces of at most ``chunk``
+    entries with consecutive slots, every other row keeps one descriptor with its left scale, and
+    the descriptors are ordered by descending number of 64-entry gather rounds (stable)."""
+    rng = np.random.default_rng(0)
+    lens = rng.integers(0, 40, size=500)
+    lens[[3, 77, 400]] = [10_000, 2049, 4096]              # three rows to cut at chunk = 2048; 4096 = exactly two pieces
+    lens[5] = 2048                                          # exactly the chunk: not cut
+    rowptr = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+    n = lens.shape[0]
+    parent = torch.from_numpy(np.where(rng.random(n) < 0.5, -1, 0).astype(np.int32))
+    m = torch.from_numpy(rng.random(n).astype(np.float32) + 0.5)
+    mat = cbm_matrix.__new__(cbm_matrix)
+    mat.split_chunk = 2048
+    sched, long_rows, pieces = mat._split_schedule(rowptr, parent, m)
+    assert long_rows[:, 0].tolist() == [3, 77, 400] and long_rows[:, 2].tolist() == [5, 2, 2] and pieces == 9
+    assert long_rows[:, 1].tolist() == [0, 5, 7]
+    assert sched.shape[0] == n - 3 + 9
+    PIECE = 0x40000000
+    covered = np.zeros(int(rowptr[-1]), np.int32)
+    slots_seen = []
+    rounds = []
+    for s0, s1, row, w in sched.tolist():
+        covered[s0:s1] += 1
+        rounds.append((s1 - s0 + 63) // 64)
+        scale = np.array([w], np.int32).view(np.float32)[0]
+        if row & PIECE:
+            slot = row & ~PIECE
+            slots_seen.append(slot)
+            owner = [r for r, f, k, _ in long_rows.tolist() if f <= slot < f + k][0]
+            assert rowptr[owner] <= s0 < s1 <= rowptr[owner + 1] and s1 - s0 <= 2048 and scale == 1.0
+            assert (s0 - int(rowptr[owner])) // 2048 == slot - [f for r, f, k, _ in long_rows.tolist() if r == owner][0]
+        else:
+            assert s0 == rowptr[row] and s1 == rowptr[row + 1] and s1 - s0 <= 2048
+            assert scale == (float(m[row]) if parent[row] < 0 else 1.0)
+    assert (covered == 1).all() and sorted(slots_seen) == list(range(9))
+    assert rounds == sorted(rounds, reverse=True)
+    for r, f, k, w in long_rows.tolist():                   # the left scale of a cut row travels with it
+        assert np.array([w], np.int32).view(np.float32)[0] == (float(m[r]) if parent[r] < 0 else 1.0)
+    # nothing to cut: the plain schedule
+    mat.split_chunk = 1 << 20
+    s2, l2, p2 = mat._split_schedule(rowptr, parent, m)
+    from cbm4gnn_amd.cbm import schedule_rows
+    assert l2.shape[0] == 0 and p2 == 0 and torch.equal(s2, schedule_rows(rowptr, parent, m))
