@@ -43,6 +43,9 @@ namespace {
 #ifndef CBM_SLAB_ROUNDS
 #define CBM_SLAB_ROUNDS 8                  // load instructions in flight per wave in the slab kernel
 #endif
+#ifndef CBM_TILED_VECS
+#define CBM_TILED_VECS 6                   // 16-byte index vectors requested together per row in the tiled kernel
+#endif
 #ifndef CBM_XCD_REMAP
 #define CBM_XCD_REMAP 1
 #endif
@@ -468,22 +471,18 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
                         }
                     }
                 };
-                // two vectors in flight, alternating registers: the load of vector j + 2 is issued
-                // before vector j is gathered
-                uint4 va = pad4, vb = pad4;
-                if (0 < len[t]) va = mine[0];
-                if (1 < len[t]) vb = mine[1];
-                for (int j = 0; j < longest; j += 2) {
-                    const uint4 ca = va;
-                    va = pad4;
-                    if (j + 2 < len[t]) va = mine[j + 2];
-                    gather8(ca);
-                    if (j + 1 < longest) {
-                        const uint4 cb = vb;
-                        vb = pad4;
-                        if (j + 3 < len[t]) vb = mine[j + 3];
-                        gather8(cb);
+                // four index vectors (32 entries) are requested together, then gathered: one wait per
+                // 32 gathers; the other wavefronts of the SIMD cover it
+                for (int j = 0; j < longest; j += CBM_TILED_VECS) {
+                    uint4 v[CBM_TILED_VECS];
+#pragma unroll
+                    for (int q = 0; q < CBM_TILED_VECS; q++) {
+                        v[q] = pad4;
+                        if (j + q < len[t]) v[q] = mine[j + q];
                     }
+#pragma unroll
+                    for (int q = 0; q < CBM_TILED_VECS; q++)
+                        if (j + q < longest) gather8(v[q]);
                 }
             }
         }
