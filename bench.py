@@ -513,7 +513,9 @@ def main():
         # X rows are re-used out of L2 / the memory-side cache.  frac_traffic: counter-measured HBM-side
         # bytes over the same launch time (what the memory system really moved).  frac_compulsory: the
         # lower bound (X once, Y once, indices once) over the same time.
-        "roofline": {"bound": "hbm", "kernel": "spmm_slab_per_xcd" if ex["slab"] else "spmm_wave_per_row",
+        "roofline": {"bound": "hbm",
+                     "kernel": ("spmm_slab_per_xcd+spmm_tiled_local" if mat.is_tiled() else
+                                "spmm_slab_per_xcd" if ex["slab"] else "spmm_wave_per_row"),
                      "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": traffic,
                      "frac_traffic": (traffic / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS) if traffic else None,
