@@ -1016,3 +1016,60 @@ def _normalised_csr(orc, ei, n, normalized):
         return rp, col, None
     m = orc.col_multiplier(ei, n)
     return rp, col, (m[ei[0][order]] * m[col]).astype(np.float32)
+
+
+def test_status_codes_of_the_plan_based_entry_points():
+    """cbm_spmm_tiled_f32 / cbm_spmm_update_tiled_f32 / the scaled and masked copies refuse bad
+    arguments with a status code before anything is enqueued."""
+    lib = _lib.hip_lib()
+    n, d = 3000, 64
+    ei = graphs.add_self_loops(graphs.sbm(n, 30, 0.6, 0.002, seed=5), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=True, tiling="on")
+    mat.tile_min_block_entries = 1000
+    dev = torch.device("cuda")
+    st = mat._device_arrays(dev)
+    assert st["tiled"] is not None
+    ts = mat._tiled_struct(st, True)
+    x = torch.randn((n, d), device=dev)
+    y = torch.full((n, d), 5.0, device=dev)
+    ws = torch.empty(mat.workspace_floats(n, d, dev), device=dev)
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    say("plan status codes")
+    call = lambda t, m, xx, yy, w, flags, nn=n, dd=d, ldx=d, ldy=d: lib.cbm_spmm_tiled_f32(
+        C.byref(t) if t is not None else None, p(m), p(xx), p(yy), p(w), flags, nn, dd, ldx, ldy, None)
+    m = st["m"]
+    assert call(None, m, x, y, ws, 0) == 1                          # no plan
+    assert call(ts, m, x, y, None, 0) == 1                          # the workspace is required
+    assert call(ts, m, x, y, ws, 0, ldx=d - 1) == 3                 # stride below the width
+    assert call(ts, m, x, y, ws, 0, nn=n - 300) == 3                # the plan was made for another row count
+    assert call(ts, m, x, x, ws, 0) == 3                            # in place
+    assert call(ts, m, x, y, x, 0) == 3                             # workspace overlaps X
+    assert call(ts, m, x, y, ws, 64) == 6                           # unknown flag
+    assert call(ts, m, x, y, ws, _lib.CBM_SPMM_WORKSPACE_READY) == 6         # with m, a ready copy must be the scaled one
+    assert call(ts, None, x, y, ws, _lib.CBM_SPMM_WORKSPACE_READY | _lib.CBM_SPMM_WORKSPACE_PRESCALED) == 6
+    assert call(ts, m, x, y, ws, _lib.CBM_SPMM_WORKSPACE_PRESCALED) == 6     # PRESCALED without READY
+    bad = _lib.CbmTilingDev.from_buffer_copy(ts); bad.tile_rows = 777
+    assert call(bad, m, x, y, ws, 0) == 3
+    bad = _lib.CbmTilingDev.from_buffer_copy(ts); bad.n_long = 2; bad.long_rows = None
+    assert call(bad, m, x, y, ws, 0) == 1
+    torch.cuda.synchronize()
+    assert bool((y == 5.0).all())                                   # none of the refused calls wrote anything
+    assert call(ts, m, x, y, ws, 0) == 0
+    lo = mat.level_off
+    upd = lambda flags: lib.cbm_spmm_update_tiled_f32(C.byref(ts), p(m), p(st["parent"]), p(st["order"]), p(st["level_off"]),
+                                                      p(lo), mat.n_levels, p(x), p(y), p(ws), n, d, d, d, flags, None)
+    assert upd(128) == 6 and upd(0) == 0
+    assert lib.cbm_spmm_update_tiled_f32(C.byref(ts), p(m), None, p(st["order"]), p(st["level_off"]), p(lo), mat.n_levels,
+                                         p(x), p(y), p(ws), n, d, d, d, 0, None) == 1
+    # copies
+    assert lib.cbm_relayout_slabs_scaled_f32(p(x), None, p(ws), n, d, d, None) == 1
+    assert lib.cbm_relayout_slabs_scaled_f32(p(x), p(m), p(x), n, d, d, None) == 3
+    assert lib.cbm_relayout_slabs_masked_f32(p(x), None, p(m), p(ws), n, d, d, d, None) == 1
+    assert lib.cbm_relayout_slabs_masked_f32(p(x), p(y), None, p(y), n, d, d, d, None) == 3      # copy over its own mask
+    assert lib.cbm_relayout_slabs_masked_f32(p(x), p(y), None, p(ws), n, d, d, d - 1, None) == 3
+    assert lib.cbm_spmm_tiled_workspace_floats(C.byref(ts), n, d) == n * d
+    assert lib.cbm_spmm_tiled_workspace_floats(None, n, d) == 0
+    torch.cuda.synchronize()
+    # a workspace that is too small for the Python layer's own check
+    with pytest.raises(ValueError, match="workspace"):
+        mat._run_spmm_update(x, y, use_m=True, workspace=torch.empty(16, device=dev))
