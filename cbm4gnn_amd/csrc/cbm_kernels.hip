@@ -387,18 +387,23 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 typedef float f32x4 __attribute__((ext_vector_type(4)));      // a native 16-byte vector (stays in registers)
 constexpr int kPanelRows = CBM_TILING_PANEL_ROWS;           // rows of the matrix per panel
 constexpr int kTiledWaves = 16;            // one 1024-thread workgroup
-constexpr int kTiledSets = kPanelRows / (kTiledWaves * 8);   // sets of 8 rows per wave
 
-template <int TILE, bool SIGNED>
+// LPE lanes serve one row: 8 for the 128-byte slabs, 4 for the 64-byte half slab of the last
+// d % 32 columns (then 16 rows per wave in lockstep, one set per wave, and W / Z / d are those of
+// the half slab: W its copy, Z already offset to its first column, d its width, n_slabs = 1).
+template <int TILE, bool SIGNED, int LPE>
 __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_tiled_local(
     const int32_t* __restrict__ panel_ptr, const int32_t* __restrict__ blk_tile, const int32_t* __restrict__ seg,
     const uint16_t* __restrict__ lidx, const float* __restrict__ W, float* __restrict__ Z,
     const float* __restrict__ row_scale, int n, int d, int n_slabs, int n_panels, int64_t ldz, int relu, int vec_out) {
-    extern __shared__ float4 tile_lds[];                   // (TILE + 1) x 8 float4; row TILE is all zero
+    constexpr int kGroups = kWave / LPE;                   // rows a wave serves in lockstep
+    constexpr int kTiledSets = kPanelRows / (kTiledWaves * kGroups);
+    constexpr int kRowFloats = LPE * 4;
+    extern __shared__ float4 tile_lds[];                   // (TILE + 1) x LPE float4; row TILE is all zero
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int sub = lane >> 3, li = lane & 7;
-    if (threadIdx.x < 8) tile_lds[TILE * 8 + threadIdx.x] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const int sub = lane / LPE, li = lane % LPE;
+    if (threadIdx.x < LPE) tile_lds[TILE * LPE + threadIdx.x] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     constexpr uint32_t kPad = (uint32_t)(TILE * 8) | ((uint32_t)(TILE * 8) << 16);    // two entries of the zero row
     // Workgroup b runs on XCD b % 8.  Items (panel-major, slab-minor) are cut into 8 contiguous
     // ranges, one per XCD, and dealt cyclically to the XCD's workgroups: the workgroups of an XCD
@@ -417,23 +422,24 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
         const int b_beg = panel_ptr[panel], b_end = panel_ptr[panel + 1];
         // The tile of block b + 1 is fetched into registers while block b is gathered from LDS, so
         // that between two blocks only the LDS stores and two barriers are exposed.
-        constexpr int kStage = TILE * 8 / (kWave * kTiledWaves);          // float4 per thread and tile
+        constexpr int kStage = TILE * LPE / (kWave * kTiledWaves);        // float4 per thread and tile
         f32x4 stage[kStage];
 #define CBM_FETCH_TILE(B)                                                                                            \
     do {                                                                                                             \
         const int base_ = blk_tile[B] * TILE;                                                                        \
-        const int rows8_ = min(TILE, n - base_) * 8;                                                                 \
-        const f32x4* __restrict__ src_ = reinterpret_cast<const f32x4*>(W + ((int64_t)slab * n + base_) * 32);       \
+        const int rows8_ = min(TILE, n - base_) * LPE;                                                               \
+        const f32x4* __restrict__ src_ = reinterpret_cast<const f32x4*>(W + ((int64_t)slab * n + base_) * kRowFloats); \
         _Pragma("unroll") for (int i_ = 0; i_ < kStage; i_++)   /* all loads in flight together; rows past the */    \
             stage[i_] = src_[min(i_ * (kWave * kTiledWaves) + (int)threadIdx.x, rows8_ - 1)]; /* matrix: never gathered */ \
     } while (0)
         if (b_beg < b_end) CBM_FETCH_TILE(b_beg);
         for (int b = b_beg; b < b_end; b++) {
-            // this lane group's segment in each set: panel row = set * 128 + wave * 8 + sub; seg[] counts in units of 8 entries
+            // this lane group's segment in each set: panel row = set * (16 waves x rows per wave) + wave * rows per wave
+            // + lane group; seg[] counts in units of 8 entries
             int s0[kTiledSets], len[kTiledSets];
 #pragma unroll
             for (int t = 0; t < kTiledSets; t++) {
-                const int32_t* __restrict__ sg = seg + (int64_t)b * (kPanelRows + 1) + t * (kTiledWaves * 8) + wave * 8 + sub;
+                const int32_t* __restrict__ sg = seg + (int64_t)b * (kPanelRows + 1) + t * (kTiledWaves * kGroups) + wave * kGroups + sub;
                 s0[t] = sg[0]; len[t] = sg[1] - s0[t];
             }
             __syncthreads();                               // the previous tile is no longer read
@@ -446,7 +452,7 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
             for (int t = 0; t < kTiledSets; t++) {
                 int longest = len[t];                       // the wave iterates to its longest segment
 #pragma unroll
-                for (int off = 8; off < kWave; off <<= 1) longest = max(longest, __shfl_xor(longest, off, kWave));
+                for (int off = LPE; off < kWave; off <<= 1) longest = max(longest, __shfl_xor(longest, off, kWave));
                 longest = __builtin_amdgcn_readfirstlane(longest);
                 const uint4* __restrict__ mine = reinterpret_cast<const uint4*>(lidx) + s0[t];
                 const uint4 pad4 = make_uint4(kPad, kPad, kPad, kPad);
@@ -457,7 +463,8 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
                         const uint32_t p = (u & 1) ? (w[u >> 1] >> 16) : (w[u >> 1] & 0xffffu);
-                        x[u] = tile_lds[(SIGNED ? (p & 0x7fffu) : p) + li];
+                        const uint32_t at = SIGNED ? (p & 0x7fffu) : p;      // row of the tile x 8
+                        x[u] = tile_lds[(LPE == 8 ? at : at >> 1) + li];
                     }
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
@@ -490,8 +497,8 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
         // epilogue: every lane group adds its row's local sum to the remote part
 #pragma unroll
         for (int t = 0; t < kTiledSets; t++) {
-            const int row = panel * kPanelRows + t * (kTiledWaves * 8) + wave * 8 + sub;
-            const int col = slab * 32 + li * 4;
+            const int row = panel * kPanelRows + t * (kTiledWaves * kGroups) + wave * kGroups + sub;
+            const int col = slab * kRowFloats + li * 4;
             if (row < n && col < d) {
                 float* __restrict__ zr = Z + (int64_t)row * ldz + col;
                 const float sc = row_scale ? row_scale[row] : 1.0f;
@@ -530,11 +537,13 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
 // once per delta entry, after which the SpMM needs no coefficient per entry, only the sign bit.
 template <bool VEC_IN, bool MASKED, bool SCALED>
 __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ X, float* __restrict__ W, int n, int d,
-                                                      int n_slabs, int64_t ldx, const float* __restrict__ M,
+                                                      int n_slabs, int tail4, int64_t ldx, const float* __restrict__ M,
                                                       int64_t ldm, const float* __restrict__ scale) {
+    // n_slabs full slabs of 8 float4 per row, then (tail4 = 4) one half slab of 4 float4 per row,
+    // stored behind all full slabs: W[s][r][0 .. 32) for s < n_slabs, then T[r][0 .. 16).
     constexpr int kSlab4 = 8;                              // float4 per 128-byte slab
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int row4 = n_slabs * kSlab4;
+    const int row4 = n_slabs * kSlab4 + tail4;
     if (t >= (int64_t)n * row4) return;
     const int r = (int)(t / row4), q = (int)(t % row4);
     const int s = q / kSlab4, w = q % kSlab4;
@@ -567,7 +576,9 @@ __global__ __launch_bounds__(256) void relayout_slabs(const float* __restrict__ 
         const float f = scale[r];
         v.x *= f; v.y *= f; v.z *= f; v.w *= f;
     }
-    *reinterpret_cast<float4*>(W + (((int64_t)s * n + r) * kSlab4 + w) * 4) = v;
+    float* __restrict__ dst = s < n_slabs ? W + (((int64_t)s * n + r) * kSlab4 + w) * 4
+                                          : W + (int64_t)n * n_slabs * 32 + ((int64_t)r * tail4 + w) * 4;
+    *reinterpret_cast<float4*>(dst) = v;
 }
 
 // coef[k] = +-m[col(k)]: the packed entries expanded once so the SpMM can stream coefficients.
@@ -755,13 +766,13 @@ __global__ __launch_bounds__(256) void relu_rows(float* __restrict__ Y, int64_t 
 
 // Rows that the schedule cut into pieces: Z[row] = (piece sums added in order, from 0) * scale,
 // then the ReLU if asked.  long_rows = { row, first slot, pieces, bits(scale) } per cut row; a slot
-// holds n_slabs x 32 floats.  blockIdx.x = cut row, threads along the columns.
+// holds slot_floats floats, Z and d are those of the column range the slots cover.  blockIdx.x =
+// cut row, threads along the columns.
 __global__ __launch_bounds__(256) void combine_pieces(const int4* __restrict__ long_rows, const float* __restrict__ partials,
-                                                      float* __restrict__ Z, int d, int n_slabs, int64_t ldz,
+                                                      float* __restrict__ Z, int d, int64_t slot_floats, int64_t ldz,
                                                       int apply_scale, int relu) {
     const int4 lr = long_rows[blockIdx.x];
     const float scale = apply_scale ? __int_as_float(lr.w) : 1.0f;
-    const int64_t slot_floats = (int64_t)n_slabs * 32;
     for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < d; j += gridDim.y * blockDim.x) {
         float acc = 0.0f;
         for (int k = 0; k < lr.z; k++) acc += partials[(int64_t)(lr.y + k) * slot_floats + j];
@@ -922,6 +933,7 @@ struct SlabPlan {
     int n_slabs = 0;        // slabs the kernel walks (odd widths: padded count)
     bool relayout = false;  // the gather reads the slab-major copy in the workspace
     bool vec_out = false;   // rows of Z are float4-addressable
+    int tail = 0;           // floats of the half slab behind the n_slabs full ones (copy only): 0 or 16
 };
 
 // Slabs of the slab-major copy: ceil(d / 32), rounded up to 1, 2, 4 or 8 when below 8 so that
@@ -931,6 +943,25 @@ inline int padded_slab_count(int d) {
     if (ns < kXcds) { int q = 1; while (q < ns) q *= 2; ns = q; }
     return ns;
 }
+
+// Layout of the slab-major copy of an n x d matrix: n_full slabs of 32 floats per row and, when
+// the last d % 32 columns are at most 16, one half slab of 16 floats per row behind them (gathered
+// with 4 lanes per entry, 16 entries per instruction: a width of 41 moves 48 floats per entry
+// instead of 64).  The half slab is only taken where the full slabs still split evenly over the 8
+// XCDs without padding (0, 1, 2, 4 or a multiple of 8 of them).
+struct CopyLayout {
+    int n_full = 0, tail = 0;                              // tail: 0 or 16 floats
+    int64_t row_floats() const { return (int64_t)n_full * 32 + tail; }
+};
+inline CopyLayout copy_layout(int d) {
+    CopyLayout c;
+    const int nf = d / 32, rem = d % 32;
+    const bool even_split = nf <= 2 || nf == 4 || nf % kXcds == 0;
+    if (rem >= 1 && rem <= 16 && even_split) { c.n_full = nf; c.tail = 16; }
+    else c.n_full = padded_slab_count(d);
+    return c;
+}
+inline int64_t copy_floats(int64_t rows, int d) { return rows * copy_layout(d).row_floats(); }
 
 // With a workspace every width runs on 128-byte slabs read from the slab-major copy (zero-padded
 // for widths that are not a multiple of 32), unless the caller's row stride makes the copy
@@ -959,7 +990,8 @@ inline SlabPlan plan_slabs(int d, int64_t ldx, int64_t ldz, const void* X, const
     // at a stride of 288 floats, 431 us at 256, 400 us with the copy).
     const bool alias_free = direct.lpe == 8 && ldx % 32 == 0 && (ldx / 32) % 2 == 1 && aligned(X, 128);
     if (force_copy || (have_workspace && !alias_free)) {
-        p.lpe = 8; p.n_slabs = padded_slab_count(d); p.relayout = true;
+        const CopyLayout c = copy_layout(d);
+        p.lpe = 8; p.n_slabs = c.n_full; p.tail = c.tail; p.relayout = true;
         return p;
     }
     return direct.lpe ? direct : p;
@@ -1015,7 +1047,7 @@ inline int slab_waves_per_simd(int64_t nnz, int32_t n, int lpe) {
 constexpr int kMaxDevices = 64;
 struct DeviceFacts {
     int cus = 0;
-    int groups[2][2][3] = {};                              // [PACKED][lpe == 16][coefficient mode]
+    int groups[2][3][3] = {};                              // [PACKED][lpe: 8, 16, 4][coefficient mode]
 };
 DeviceFacts g_facts[kMaxDevices];
 std::atomic<int> g_facts_ready[kMaxDevices];               // zero-initialised
@@ -1029,8 +1061,13 @@ int resident_groups_per_xcd(K kernel, int cus) {
     return (cus / kXcds) * per_cu;
 }
 
+constexpr int kTailRounds = 4;                             // 4 lanes per entry: 16 entries per instruction, 64 per round
+
 template <bool PACKED>
-void fill_groups(int (&g)[2][3], int cus) {
+void fill_groups(int (&g)[3][3], int cus) {
+    g[2][kCoefStream] = resident_groups_per_xcd(spmm_slab_per_xcd<4, PACKED, kCoefStream, kTailRounds>, cus);
+    g[2][kCoefSign] = resident_groups_per_xcd(spmm_slab_per_xcd<4, PACKED, kCoefSign, kTailRounds>, cus);
+    g[2][kCoefSignM] = resident_groups_per_xcd(spmm_slab_per_xcd<4, PACKED, kCoefSignM, kTailRounds>, cus);
     g[0][kCoefStream] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefStream, CBM_SLAB_ROUNDS>, cus);
     g[0][kCoefSign] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSign, CBM_SLAB_ROUNDS>, cus);
     g[0][kCoefSignM] = resident_groups_per_xcd(spmm_slab_per_xcd<8, PACKED, kCoefSignM, CBM_SLAB_ROUNDS>, cus);
@@ -1068,13 +1105,14 @@ inline int64_t matrix_bytes(int32_t n, int32_t d, int64_t ld) {
 
 inline int launch_relayout(const float* X, float* workspace, int32_t n, int32_t d, int64_t ldx, hipStream_t s,
                            const float* mask = nullptr, int64_t ldm = 0, const float* scale = nullptr) {
-    const int ns = padded_slab_count(d);
-    const int64_t blocks = ((int64_t)n * ns * 8 + 255) / 256;
+    const CopyLayout c = copy_layout(d);
+    const int ns = c.n_full, tail4 = c.tail / 4;
+    const int64_t blocks = ((int64_t)n * (ns * 8 + tail4) + 255) / 256;
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
     const dim3 grid((unsigned)blocks), block(256);
     const bool vec = d % 4 == 0 && ldx % 4 == 0 && aligned(X, 16) && (!mask || (ldm % 4 == 0 && aligned(mask, 16)));
 #define LAUNCH_RELAYOUT(V, K, S) \
-    hipLaunchKernelGGL((relayout_slabs<V, K, S>), grid, block, 0, s, X, workspace, n, d, ns, ldx, mask, ldm, scale)
+    hipLaunchKernelGGL((relayout_slabs<V, K, S>), grid, block, 0, s, X, workspace, n, d, ns, tail4, ldx, mask, ldm, scale)
     switch ((vec ? 4 : 0) | (mask ? 2 : 0) | (scale ? 1 : 0)) {
         case 0: LAUNCH_RELAYOUT(false, false, false); break;
         case 1: LAUNCH_RELAYOUT(false, false, true); break;
@@ -1095,7 +1133,7 @@ template <bool PACKED>
 int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* val, const float* m,
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s, int32_t n_desc = 0,
-                float* partials = nullptr) {
+                float* partials = nullptr, int32_t n_pieces = 0) {
     if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
     const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
     if ((flags & CBM_SPMM_WORKSPACE_PRESCALED) && (!PACKED || !m || !(flags & CBM_SPMM_WORKSPACE_READY)))
@@ -1109,7 +1147,7 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
     const bool ready = (flags & CBM_SPMM_WORKSPACE_READY) != 0;
     if (workspace) {                                      // the slab-major copy must be disjoint from X and Z
         if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
-        const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+        const int64_t ws_bytes = copy_floats(n, d) * 4;
         if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
             ranges_overlap(workspace, ws_bytes, Z, matrix_bytes(n, d, ldz)))
             return CBM_ERR_SHAPE;
@@ -1136,31 +1174,45 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
         const int coef_mode = prescaled ? kCoefSign : (val ? kCoefStream : (m ? kCoefSignM : kCoefSign));
         const DeviceFacts* facts = device_facts();
         const int per_wave = facts ? facts->cus / kXcds : 0;
-        int G = facts ? facts->groups[PACKED ? 1 : 0][lpe == 8 ? 0 : 1][coef_mode] : 0;
-        if (G > 0) {
-            const int cap = per_wave * slab_waves_per_simd(nnz, n, lpe);
+        const int n_rows = n_desc > 0 ? n_desc : n;             // descriptors the waves walk
+        // One launch over `slabs` slabs of `L` float4 per row: the full slabs, then (copy only) the half slab
+        // of the last d % 32 columns as a launch of its own with 4 lanes per entry.
+        auto launch = [&](int L, int slabs, const float* Xl, int64_t slab_stride, int64_t row_stride, float* Zl, int d_l,
+                          float* partials_l) -> int {
+            int G = facts ? facts->groups[PACKED ? 1 : 0][L == 8 ? 0 : (L == 16 ? 1 : 2)][coef_mode] : 0;
+            if (G <= 0) return CBM_ERR_LAUNCH;
+            const int cap = per_wave * slab_waves_per_simd(nnz, n, L);
             if (cap > 0 && G > cap) G = cap;
             // no more waves than rows: with fewer rows than resident waves shrink the grid
-            const int n_rows = n_desc > 0 ? n_desc : n;         // descriptors the waves walk
-            const int share = n_slabs >= kXcds ? 1 : kXcds / n_slabs;
+            const int share = slabs >= kXcds ? 1 : kXcds / slabs;
             const int need = (n_rows + share * kWavesPerBlock - 1) / (share * kWavesPerBlock);
             if (G > need) G = need;
             const dim3 grid(G * kXcds), block(kWave * kWavesPerBlock);
-            const int vec_out = plan.vec_out ? 1 : 0;
-#define LAUNCH_SLAB(L, CF)                                                                                     \
-    hipLaunchKernelGGL((spmm_slab_per_xcd<L, PACKED, CF, CBM_SLAB_ROUNDS>), grid, block, 0, s, rowptr, sc, idx, \
-                       val, m, parent, Xg, Z, n_rows, d, vec_out, n_slabs, x_slab_stride, x_row_stride, ldz, relu, partials)
-            switch (lpe * 4 + coef_mode) {
-                case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream); break;
-                case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign); break;
-                case 8 * 4 + kCoefSignM: LAUNCH_SLAB(8, kCoefSignM); break;
-                case 16 * 4 + kCoefStream: LAUNCH_SLAB(16, kCoefStream); break;
-                case 16 * 4 + kCoefSign: LAUNCH_SLAB(16, kCoefSign); break;
-                default: LAUNCH_SLAB(16, kCoefSignM); break;
+            const int vec_out = (plan.vec_out && aligned(Zl, 16)) ? 1 : 0;
+#define LAUNCH_SLAB(LL, CF, UU)                                                                                  \
+    hipLaunchKernelGGL((spmm_slab_per_xcd<LL, PACKED, CF, UU>), grid, block, 0, s, rowptr, sc, idx, val, m, parent, \
+                       Xl, Zl, n_rows, d_l, vec_out, slabs, slab_stride, row_stride, ldz, relu, partials_l)
+            switch (L * 4 + coef_mode) {
+                case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream, CBM_SLAB_ROUNDS); break;
+                case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign, CBM_SLAB_ROUNDS); break;
+                case 8 * 4 + kCoefSignM: LAUNCH_SLAB(8, kCoefSignM, CBM_SLAB_ROUNDS); break;
+                case 16 * 4 + kCoefStream: LAUNCH_SLAB(16, kCoefStream, CBM_SLAB_ROUNDS); break;
+                case 16 * 4 + kCoefSign: LAUNCH_SLAB(16, kCoefSign, CBM_SLAB_ROUNDS); break;
+                case 16 * 4 + kCoefSignM: LAUNCH_SLAB(16, kCoefSignM, CBM_SLAB_ROUNDS); break;
+                case 4 * 4 + kCoefStream: LAUNCH_SLAB(4, kCoefStream, kTailRounds); break;
+                case 4 * 4 + kCoefSign: LAUNCH_SLAB(4, kCoefSign, kTailRounds); break;
+                default: LAUNCH_SLAB(4, kCoefSignM, kTailRounds); break;
             }
 #undef LAUNCH_SLAB
-            return check_launch();
-        }
+            return CBM_OK;
+        };
+        int rc = CBM_OK;
+        if (n_slabs > 0)
+            rc = launch(lpe, n_slabs, Xg, x_slab_stride, x_row_stride, Z, plan.tail ? n_slabs * 32 : d, partials);
+        if (rc == CBM_OK && plan.tail)                        // partials of the tail: behind those of the full slabs
+            rc = launch(4, 1, workspace + (int64_t)n * n_slabs * 32, 0, plan.tail, Z + n_slabs * 32, d - n_slabs * 32,
+                        partials ? partials + (int64_t)n_pieces * n_slabs * 32 : nullptr);
+        if (rc == CBM_OK) return check_launch();
         if (ready) return CBM_ERR_LAUNCH;                 // no occupancy information: cannot honour the copy
     }
     if (n_desc > 0) return CBM_ERR_UNSUPPORTED;           // a cut schedule runs on the slab kernel only
@@ -1320,7 +1372,7 @@ int cbm_relayout_slabs_scaled_f32(const float* X, const float* scale, float* wor
     if (!X || !workspace || !scale) return CBM_ERR_NULL;
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
-    if (ranges_overlap(workspace, (int64_t)n * padded_slab_count(d) * 32 * 4, X, matrix_bytes(n, d, ldx))) return CBM_ERR_SHAPE;
+    if (ranges_overlap(workspace, copy_floats(n, d) * 4, X, matrix_bytes(n, d, ldx))) return CBM_ERR_SHAPE;
     if (n == 0 || d == 0) return CBM_OK;
     if (int rc = launch_relayout(X, workspace, n, d, ldx, static_cast<hipStream_t>(stream), nullptr, 0, scale)) return rc;
     return check_launch();
@@ -1332,7 +1384,7 @@ int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, const float
     if (int rc = check_matrix(n, d, ldx)) return rc;
     if (int rc = check_matrix(n, d, ldm)) return rc;
     if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
-    const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+    const int64_t ws_bytes = copy_floats(n, d) * 4;
     if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
         ranges_overlap(workspace, ws_bytes, mask, matrix_bytes(n, d, ldm)))
         return CBM_ERR_SHAPE;
@@ -1343,7 +1395,7 @@ int cbm_relayout_slabs_masked_f32(const float* X, const float* mask, const float
 
 int64_t cbm_relayout_floats(int32_t n, int32_t d) {
     if (n <= 0 || d <= 0) return 0;
-    return (int64_t)n * padded_slab_count(d) * 32;
+    return copy_floats(n, d);
 }
 
 int cbm_row_intersections_groups(void) {
@@ -1392,13 +1444,19 @@ int cbm_set_spmm_kernel(int kind) {
 
 int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z, int32_t have_workspace) {
     const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, have_workspace != 0, false);
-    return p.lpe ? kWave / p.lpe : 1;
+    if (!p.lpe) return 1;
+    return p.n_slabs > 0 ? kWave / p.lpe : kWave / 4;      // only the half slab: d <= 16
+}
+
+int cbm_spmm_tail_columns(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z, int32_t have_workspace) {
+    const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, have_workspace != 0, false);
+    return (p.lpe && p.tail) ? d - p.n_slabs * 32 : 0;
 }
 
 int64_t cbm_spmm_workspace_floats(int32_t n, int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z) {
     if (n <= 0 || d <= 0) return 0;
     const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, true, false);
-    return p.relayout ? (int64_t)n * p.n_slabs * 32 : 0;
+    return p.relayout ? copy_floats(n, d) : 0;
 }
 
 int cbm_expand_coef_f32(const uint32_t* idx, const float* m, float* coef, int64_t nnz, void* stream) {
@@ -1463,7 +1521,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
 
 int64_t cbm_spmm_tiled_workspace_floats(const cbm_tiling_dev* t, int32_t n, int32_t d) {
     if (!t || n <= 0 || d <= 0) return 0;
-    return ((int64_t)n + (t->n_long > 0 ? t->n_pieces : 0)) * padded_slab_count(d) * 32;
+    return copy_floats((int64_t)n + (t->n_long > 0 ? t->n_pieces : 0), d);
 }
 
 int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, float* Z, float* workspace, int32_t flags,
@@ -1489,7 +1547,7 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     if (!facts || facts->cus < kXcds) return CBM_ERR_LAUNCH;
     if (!ready) {                                         // launch_spmm checks alignment and overlap of the workspace below
         if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
-        const int64_t ws_bytes = (int64_t)n * padded_slab_count(d) * 32 * 4;
+        const int64_t ws_bytes = copy_floats(n, d) * 4;
         if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
             ranges_overlap(workspace, ws_bytes, Z, matrix_bytes(n, d, ldz)))
             return CBM_ERR_SHAPE;
@@ -1500,34 +1558,47 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     // rows) is the whole multiply and applies them.
     const bool has_local = t->n_blocks > 0;
     const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
-    const int n_slabs = padded_slab_count(d);
-    float* partials = t->n_long > 0 ? workspace + (int64_t)n * n_slabs * 32 : nullptr;
+    const CopyLayout lay = copy_layout(d);
+    const int n_full = lay.n_full, d_full = lay.tail ? n_full * 32 : d, d_tail = lay.tail ? d - n_full * 32 : 0;
+    float* partials = t->n_long > 0 ? workspace + copy_floats(n, d) : nullptr;
     const int remote_flags = CBM_SPMM_WORKSPACE_READY | (m ? CBM_SPMM_WORKSPACE_PRESCALED : 0) |
                              ((relu && !has_local) ? CBM_SPMM_RELU : 0);
     if (int rc = launch_spmm<true>(t->rowptr_r, t->idx_r, t->nnz_remote, nullptr, m, nullptr, t->sched_r, X, Z, workspace,
-                                   remote_flags, n, d, ldx, ldz, s, t->n_long > 0 ? t->n_sched_r : 0, partials))
+                                   remote_flags, n, d, ldx, ldz, s, t->n_long > 0 ? t->n_sched_r : 0, partials, t->n_pieces))
         return rc;
-    if (t->n_long > 0) {                                  // pieces of cut rows -> their rows of Z
-        const dim3 grid((unsigned)t->n_long, (unsigned)std::min(8, (d + 255) / 256));
-        hipLaunchKernelGGL(combine_pieces, grid, dim3(256), 0, s, reinterpret_cast<const int4*>(t->long_rows), partials, Z,
-                           d, n_slabs, ldz, has_local ? 0 : 1, (relu && !has_local) ? 1 : 0);
+    if (t->n_long > 0) {                                  // pieces of cut rows -> their rows of Z, per column range
+        const int4* lr = reinterpret_cast<const int4*>(t->long_rows);
+        const int scale_here = has_local ? 0 : 1, relu_here = (relu && !has_local) ? 1 : 0;
+        if (n_full > 0)
+            hipLaunchKernelGGL(combine_pieces, dim3((unsigned)t->n_long, (unsigned)std::min(8, (d_full + 255) / 256)), dim3(256),
+                               0, s, lr, partials, Z, d_full, (int64_t)n_full * 32, ldz, scale_here, relu_here);
+        if (lay.tail)
+            hipLaunchKernelGGL(combine_pieces, dim3((unsigned)t->n_long, 1u), dim3(256), 0, s, lr,
+                               partials + (int64_t)t->n_pieces * n_full * 32, Z + n_full * 32, d_tail, (int64_t)lay.tail, ldz,
+                               scale_here, relu_here);
     }
     if (!has_local) return check_launch();
     // local entries: tiles of the copy staged in LDS; adds to Z, then scale and ReLU
-    const size_t bytes = (size_t)(t->tile_rows + 1) * 128;
-    const int vec_out = (d % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16)) ? 1 : 0;
     const int G = facts->cus / kXcds;                     // 129 KB of LDS: one workgroup per CU
-#define LAUNCH_TILED(T, S)                                                                                               \
+#define LAUNCH_TILED(T, S, L, WL, ZL, DL, SLABS)                                                                         \
     do {                                                                                                                 \
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S>),                                   \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)                   \
+        const size_t bytes_ = (size_t)(T + 1) * L * 16;                                                                  \
+        const int vec_ = (d % 4 == 0 && ldz % 4 == 0 && aligned(ZL, 16)) ? 1 : 0;                                        \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S, L>),                                \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes_) != hipSuccess)                  \
             return CBM_ERR_LAUNCH;                                                                                       \
-        hipLaunchKernelGGL((spmm_tiled_local<T, S>), dim3(G * kXcds), dim3(kWave * kTiledWaves), bytes, s, t->panel_ptr, \
-                           t->blk_tile, t->seg, t->lidx, workspace, Z, t->row_scale, n, d, n_slabs, t->n_panels, ldz,    \
-                           relu, vec_out);                                                                               \
+        hipLaunchKernelGGL((spmm_tiled_local<T, S, L>), dim3(G * kXcds), dim3(kWave * kTiledWaves), bytes_, s,           \
+                           t->panel_ptr, t->blk_tile, t->seg, t->lidx, WL, ZL, t->row_scale, n, DL, SLABS, t->n_panels,  \
+                           ldz, relu, vec_);                                                                             \
     } while (0)
-    if (t->tile_rows == 1024) { if (t->has_negative) LAUNCH_TILED(1024, true); else LAUNCH_TILED(1024, false); }
-    else { if (t->has_negative) LAUNCH_TILED(512, true); else LAUNCH_TILED(512, false); }
+#define LAUNCH_TILED_BOTH(T, S)                                                                                          \
+    do {                                                                                                                 \
+        if (n_full > 0) LAUNCH_TILED(T, S, 8, workspace, Z, d_full, n_full);                                             \
+        if (lay.tail) LAUNCH_TILED(T, S, 4, workspace + (int64_t)n * n_full * 32, Z + n_full * 32, d_tail, 1);          \
+    } while (0)
+    if (t->tile_rows == 1024) { if (t->has_negative) LAUNCH_TILED_BOTH(1024, true); else LAUNCH_TILED_BOTH(1024, false); }
+    else { if (t->has_negative) LAUNCH_TILED_BOTH(512, true); else LAUNCH_TILED_BOTH(512, false); }
+#undef LAUNCH_TILED_BOTH
 #undef LAUNCH_TILED
     return check_launch();
 }

@@ -224,9 +224,18 @@ int cbm_set_spmm_occupancy(int waves_per_simd);
 int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev,
                               int32_t have_workspace);
 
+/* Trailing columns of this shape that the SpMM sums in 16 interleaved partial sums instead of the
+ * number cbm_spmm_summation_groups reports: with a workspace, when the last d mod 32 columns are
+ * at most 16 (and the full 128-byte slabs split evenly over the XCDs: 0, 1, 2, 4 or a multiple of
+ * 8 of them), those columns are kept as a 64-byte half slab in the slab-major copy and gathered
+ * with 4 lanes per entry -- a width of 41 then moves 48 floats per delta entry instead of 64.
+ * 0 = no such columns.  No reference counterpart. */
+int cbm_spmm_tail_columns(int32_t d, int64_t ldx, int64_t ldz, const void* X_dev, const void* Z_dev, int32_t have_workspace);
+
 /* Floats of workspace that cbm_spmm_f32 / cbm_spmm_update_f32 / csr_spmm_f32 use for this shape when
  * given one: the size of the slab-major copy of X (n rows x 128-byte slabs, the slab count
- * rounded up for odd widths), or 0 where the copy would buy nothing: d = 32, 64, 128 or 256 with
+ * rounded up for odd widths, or a 64-byte half slab for the last columns, see
+ * cbm_spmm_tail_columns), or 0 where the copy would buy nothing: d = 32, 64, 128 or 256 with
  * 128-byte-aligned rows whose stride ldx is an ODD number of 128-byte lines (e.g. ldx = d + 32),
  * which spreads the lines of a slab over all L2 channels by itself.  The workspace stays
  * optional: without it, widths that are a multiple of 32 gather from the row-major X and all

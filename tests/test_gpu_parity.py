@@ -39,6 +39,20 @@ def groups_for(d, ld=None, workspace=False):
     return int(_lib.hip_lib().cbm_spmm_summation_groups(d, ld, ld, C.c_void_p(256), C.c_void_p(256), int(workspace)))
 
 
+def tail_for(d, ld=None, workspace=False):
+    """Trailing columns that the SpMM sums in 16 partial sums (the 64-byte half slab of the copy)."""
+    ld = d if ld is None else ld
+    return int(_lib.hip_lib().cbm_spmm_tail_columns(d, ld, ld, C.c_void_p(256), C.c_void_p(256), int(workspace)))
+
+
+def grouped_spmm(orc, rp, col, val, xs, groups, tail=0, threads=1):
+    """``orc.csr_spmm`` in ``groups`` interleaved partial sums, the last ``tail`` columns in 16."""
+    y = orc.csr_spmm(rp, col, val, xs, threads=threads, groups=groups)
+    if tail and groups != 16:
+        y[:, xs.shape[1] - tail:] = orc.csr_spmm(rp, col, val, xs, threads=threads, groups=16)[:, xs.shape[1] - tail:]
+    return y
+
+
 def brings_workspace(relayout, nnz, n, d, ld=None):
     """The Python layer's rule: a workspace when rows average >= 24 entries, or when the width would
     otherwise run one wavefront per row."""
@@ -49,6 +63,10 @@ def mat_groups(mat, d, ld=None):
     """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough."""
     n = mat.num_rows
     return groups_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, n, d, ld))
+
+
+def mat_tail(mat, d, ld=None):
+    return tail_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, mat.num_rows, d, ld))
 
 
 def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, prescaled=None):
@@ -63,16 +81,18 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
         return (orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads) if normalized
                 else orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads))
     g = mat_groups(mat, x.shape[1]) if groups is None else groups
+    tail = mat_tail(mat, x.shape[1]) if groups is None else 0
     if prescaled is None:                                  # the copy is only made for the slab kernel (g > 1)
         prescaled = normalized and brings_workspace(mat.relayout, mat.nnz, n, x.shape[1]) and mat_groups(mat, x.shape[1]) > 1
     if prescaled:
         xs = (m[:, None] * x).astype(np.float32)
-        z = orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
-                         threads=threads, groups=g)
+        z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs, g, tail,
+                         threads)
         return orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads)
     val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
-    return orc.spmm_update(mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32),
-                           mat.mst_row.numpy(), mat.mst_col.numpy(), x, m, threads=threads, groups=g)
+    z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32), x, g, tail, threads)
+    return (orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads) if m is None
+            else orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads))
 
 
 def tiled_split(mat):
@@ -87,7 +107,7 @@ def tiled_split(mat):
     return np.bincount(key)[key] >= mat.tile_min_block_entries, row
 
 
-def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8):
+def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8, tail=0):
     """CSR product in ``groups`` interleaved partial sums per row, where a row with more than
     ``chunk`` entries is cut into pieces of ``chunk`` entries: each piece is summed like a row of its
     own and the piece sums are then added one after the other, starting from zero -- the order of
@@ -97,7 +117,7 @@ def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8):
     lens = np.diff(rp)
     long_rows = np.nonzero(lens > chunk)[0] if chunk else np.empty(0, np.int64)
     if long_rows.size == 0:
-        return orc.csr_spmm(rp.astype(np.int32), col, sgn, xs, groups=groups)
+        return grouped_spmm(orc, rp.astype(np.int32), col, sgn, xs, groups, tail)
     starts, ends, owner = [], [], []
     for r in long_rows:
         for k in range(rp[r], rp[r + 1], chunk):
@@ -111,7 +131,7 @@ def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8):
     aux_sgn = np.concatenate([sgn[keep], sgn[piece_idx]])
     aux_len = np.concatenate([np.where(lens > chunk, 0, lens), np.array(ends) - np.array(starts)])
     aux_rp = np.concatenate([[0], np.cumsum(aux_len)]).astype(np.int32)
-    y = orc.csr_spmm(aux_rp, aux_col.astype(np.int32), aux_sgn.astype(np.float32), xs, groups=groups)
+    y = grouped_spmm(orc, aux_rp, aux_col.astype(np.int32), aux_sgn.astype(np.float32), xs, groups, tail)
     z = y[:n].copy()
     for r in long_rows:
         acc = np.zeros(xs.shape[1], np.float32)
@@ -127,11 +147,14 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
     col, sign = mat.columns()
     d = x.shape[1]
     g = mat_groups(mat, d)
+    tail = mat_tail(mat, d)
+    plan_tail = tail_for(d, workspace=True)               # the plan-based multiply always copies
+    plan_groups = groups_for(d, workspace=True)
     if mat.relayout and not mat.is_tiled() and mat.has_cut_rows():
         # long rows cut into pieces; the plan-based multiply always gathers from the (scaled) copy
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
         return grouped_with_cuts(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
-                                 mat.split_chunk)
+                                 mat.split_chunk, plan_groups, plan_tail)
     if mat.relayout and mat.is_tiled():
         # tiled multiply: (remote entries, 8 interleaved partial sums) + (local entries in column order,
         # one after the other), on the copy of X scaled by m
@@ -139,20 +162,21 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
         c, sg = col.numpy(), sign.numpy().astype(np.float32)
         rp = np.concatenate([[0], np.cumsum(np.bincount(row[~local], minlength=n))]).astype(np.int32)
-        remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs, mat.split_chunk if mat.has_cut_rows() else 0)
+        remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs,
+                                   mat.split_chunk if mat.has_cut_rows() else 0, plan_groups, plan_tail)
         # local entries in storage order: by tile, then the columns of the row's own parity, then the others
         lr, lc, ls = row[local], c[local], sg[local]
         order = np.lexsort((lc, (lc + lr) % 2, lc // mat.tile_rows, lr))
         rp = np.concatenate([[0], np.cumsum(np.bincount(lr, minlength=n))]).astype(np.int32)
         return remote + orc.csr_spmm(rp, lc[order].astype(np.int32), ls[order], xs, groups=1)
     if not normalized:
-        return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, groups=g)
+        return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, g, tail)
     m = orc.col_multiplier(ei, n)
     if brings_workspace(mat.relayout, mat.nnz, n, d) and g > 1:      # the copy of X is scaled by m
-        return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32),
-                            (m[:, None] * x).astype(np.float32), groups=g)
+        return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32),
+                            (m[:, None] * x).astype(np.float32), g, tail)
     val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
-    return orc.csr_spmm(mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, groups=g)
+    return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, g, tail)
 
 
 @pytest.fixture(params=["auto", "wave-per-row"])
@@ -198,7 +222,10 @@ def test_widths_against_oracle(orc, d, normalized, spmm_kernel):
     assert mat.n_levels >= 2 and (mat.idx < 0).any()
     if spmm_kernel == "auto":
         assert mat_groups(mat, d) > 1                      # every width takes the slab kernel (rows are long enough)
-        assert groups_for(d, workspace=True) == 8           # 128-byte slabs from the slab-major copy
+        # 128-byte slabs from the slab-major copy; the last d % 32 <= 16 columns as a 64-byte half slab
+        # where the full slabs split evenly over the XCDs (widths up to 16: the half slab alone)
+        assert groups_for(d, workspace=True) == (16 if d <= 16 else 8)
+        assert tail_for(d, workspace=True) == {1: 1, 3: 3, 10: 10, 41: 9, 258: 2, 1028: 4, 2052: 4}.get(d, 0)
         # without a workspace only multiples of 32 run on slabs; 256-byte slabs (4 groups) where 8 of them fit
         assert groups_for(d) == (1 if d % 32 else (4 if d % 64 == 0 and d >= 512 else 8))
     else:
@@ -621,12 +648,19 @@ def test_shared_slab_major_copy(orc):
         got = torch.empty_like(x); mat._run_spmm(torch.zeros_like(x), got, use_m=True, scale_roots=True,
                                                  workspace=wm, workspace_ready=True, workspace_prescaled=True)
         assert torch.equal(got, want)
-    # odd width: the copy is zero-padded to whole slabs (41 -> 2 slabs of 32)
     x41 = torch.randn((n, 41), generator=torch.Generator().manual_seed(5)).cuda()
+    # odd width: one full slab, then the last 9 columns zero-padded to a 64-byte half slab behind it
     w41 = relayout_slabs(x41)
-    assert w41.numel() == n * 64
-    back = w41.view(2, n, 32).permute(1, 0, 2).reshape(n, 64)
-    assert torch.equal(back[:, :41], x41) and float(back[:, 41:].abs().max()) == 0.0
+    assert w41.numel() == n * 48
+    assert torch.equal(w41[:n * 32].view(n, 32), x41[:, :32])
+    half = w41[n * 32:].view(n, 16)
+    assert torch.equal(half[:, :9], x41[:, 32:]) and float(half[:, 9:].abs().max()) == 0.0
+    # 100 columns: three full slabs do not split evenly over 8 XCDs, so four zero-padded full slabs
+    x100 = torch.randn((n, 100), generator=torch.Generator().manual_seed(6)).cuda()
+    w100 = relayout_slabs(x100)
+    assert w100.numel() == n * 128
+    back = w100.view(4, n, 32).permute(1, 0, 2).reshape(n, 128)
+    assert torch.equal(back[:, :100], x100) and float(back[:, 100:].abs().max()) == 0.0
 
 
 def test_launch_size_does_not_change_results(orc):
