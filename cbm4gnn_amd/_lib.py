@@ -19,8 +19,11 @@ CBM_UPDATE_RELU = 2
 CBM_UPDATE_WORKSPACE_READY = 4
 CBM_SPMM_WORKSPACE_PRESCALED = 4
 CBM_UPDATE_WORKSPACE_PRESCALED = 8
+CBM_ERR_NULL = 1
+CBM_ERR_SHAPE = 3
 CBM_ERR_SCRATCH = 7
 CBM_STATIC_SCRATCH_FLOATS = 32 * 1024 * 1024
+CBM_PATH_MAX_LEVELS = 16
 
 
 class CbmLibraryError(RuntimeError):
@@ -98,6 +101,8 @@ HIP_SYMBOLS = {
     "cbm_relayout_slabs_scaled_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_update_paths_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_update_paths_scratch_floats": (C.c_int64, [_I32, _I32, _I32]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_tiled_workspace_floats": (C.c_int64, [C.POINTER(CbmTilingDev), _I32, _I32]),
     "cbm_spmm_tiled_f32": (C.c_int, [C.POINTER(CbmTilingDev), _P, _P, _P, _P, _I32, _I32, _I32, _I64, _I64, _P]),

@@ -384,6 +384,13 @@ class cbm_matrix:
         # wavefronts gather (``cbm_schedule_rows_split``); 0 = never cut.  A hub row of a power-law graph
         # would otherwise keep one wavefront per slab busy long after all others have finished.
         self.split_chunk = 2048
+        # Trees of 2 .. CBM_PATH_MAX_LEVELS levels are walked in ONE launch after the SpMM (every row sums down
+        # its own ancestor path, ``cbm_spmm_update_paths_f32``) while the product is at most this many bytes:
+        # there a launch per level costs more than the level's work.  0 = always walk level by level.
+        self.path_walk_max_bytes = 64 << 20
+
+    def _walks_paths(self, n, d):
+        return (1 < self.n_levels <= _lib.CBM_PATH_MAX_LEVELS and 0 < 4 * n * d <= int(self.path_walk_max_bytes))
 
     def _host_tiling(self):
         """What the plan-based multiply (``cbm_spmm_tiled_f32``) needs on the host, or False when this
@@ -773,6 +780,20 @@ class cbm_matrix:
                 y.copy_(yd)
             return
         coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
+        if self._walks_paths(n, x.size(1)):
+            zs = torch.empty(_lib.hip_lib().cbm_spmm_update_paths_scratch_floats(n, x.size(1), self.n_levels),
+                             dtype=torch.float32, device=xd.device)
+            with torch.cuda.device(xd.device):
+                rc = _lib.hip_lib().cbm_spmm_update_paths_f32(
+                    _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
+                    _ptr(coef), _ptr(st["parent"]),
+                    _ptr(st["sched_scaled"] if use_m else st["sched"]), _ptr(st["order"]), _ptr(st["level_off"]),
+                    _ptr(self.level_off), self.n_levels, _ptr(xd), _ptr(yd), _ptr(ws), _ptr(zs), n, x.size(1), _ld(xd),
+                    _ld(yd), flags, _stream(xd.device))
+            _lib.check(rc, "cbm_spmm_update_paths_f32")
+            if yd is not y:
+                y.copy_(yd)
+            return
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_update_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,

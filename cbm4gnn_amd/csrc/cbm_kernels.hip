@@ -730,6 +730,84 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
     }
 }
 
+// The walk of a SHALLOW tree in one launch, out of place: the wavefront of row v follows parent[]
+// up to the child of the root above it (at most kMaxPathLevels - 1 steps, the ids kept one per
+// lane), then adds the rows of Z down that path with exactly the arithmetic of propagate_row, so
+// Y[v] comes out bit-identical to the level-by-level walk.  Every row recomputes the values of
+// its ancestors instead of waiting for them: sum(depth) row reads instead of N, but no launch per
+// level, and the ReLU can go into the store (no row is read back).  Z must not be Y: other
+// wavefronts read the rows of Z while this one writes Y.
+constexpr int kMaxPathLevels = CBM_PATH_MAX_LEVELS;
+constexpr int kPathAhead = 4;              // rows of the path requested together
+
+template <int VEC, int CH, bool NORM, bool FULL>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void propagate_paths(
+    const int32_t* __restrict__ parent, const float* __restrict__ m, const float* __restrict__ Z,
+    float* __restrict__ Y, int n, int d, int dv, int64_t ldz, int64_t ldy, int relu) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int v = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (v >= n) return;
+    const int col0 = blockIdx.y * (kWave * VEC * CH) + lane * VEC;
+    // lane t keeps the ancestor t steps above v (lane 0: v itself); k = steps to the child of the root
+    int path = v, k = 0;
+    for (int u = __builtin_amdgcn_readfirstlane(parent[v]); u >= 0 && k < kMaxPathLevels - 1;
+         u = __builtin_amdgcn_readfirstlane(parent[u])) {
+        k++;
+        if (lane == k) path = u;
+    }
+    float my_m = 1.0f;
+    if constexpr (NORM) if (lane <= k) my_m = m[path];
+    float acc[CH][VEC];
+    {
+        const float* __restrict__ z = Z + (int64_t)bcast_i(path, k) * ldz + col0;
+#pragma unroll
+        for (int c = 0; c < CH; c++)
+            if (FULL || col0 + c * kWave * VEC < d) load_vec<VEC>(z + c * kWave * VEC, acc[c]);
+    }
+    float mu = bcast_f(my_m, k);
+    for (int t = k - 1; t >= 0; t -= kPathAhead) {
+        float z[kPathAhead][CH][VEC];
+#pragma unroll
+        for (int a = 0; a < kPathAhead; a++) {             // past the end of the path: row v again, unused
+            const float* __restrict__ zr = Z + (int64_t)bcast_i(path, max(t - a, 0)) * ldz + col0;
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+                if (FULL || col0 + c * kWave * VEC < d) load_vec<VEC>(zr + c * kWave * VEC, z[a][c]);
+        }
+#pragma unroll
+        for (int a = 0; a < kPathAhead; a++)
+            if (t - a >= 0) {
+                const float mv = bcast_f(my_m, t - a);
+                const float inv_mu = 1.0f / mu;
+#pragma unroll
+                for (int c = 0; c < CH; c++)
+                    if (FULL || col0 + c * kWave * VEC < d) {
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) {
+                            if constexpr (NORM) {
+                                const int j = col0 + c * kWave * VEC + e;
+                                acc[c][e] = (j < dv) ? fmaf(acc[c][e], inv_mu, z[a][c][e]) * mv
+                                                     : (z[a][c][e] + acc[c][e] / mu) * mv;
+                            } else {
+                                acc[c][e] = z[a][c][e] + acc[c][e];
+                            }
+                        }
+                    }
+                mu = mv;
+            }
+    }
+    float* __restrict__ y = Y + (int64_t)v * ldy + col0;
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+        if (FULL || col0 + c * kWave * VEC < d) {
+            if (relu) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[c][e] = acc[c][e] < 0.0f ? 0.0f : acc[c][e];   // keeps NaN
+            }
+            store_vec<VEC>(y + c * kWave * VEC, acc[c]);
+        }
+}
+
 // Y[r,:] *= m[r] for the rows of level 0 (children of the root), cbm_extensions.cpp:910-940.
 template <int VEC, int CH, bool FULL>
 __global__ __launch_bounds__(kWave * kWavesPerBlock) void scale_level0(
@@ -1517,6 +1595,54 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
     hipLaunchKernelGGL(relu_rows, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), Y, total, d, ldy);
     return check_launch();
+}
+
+int cbm_spmm_update_paths_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m, const float* coef,
+                              const int32_t* parent, const int32_t* row_sched, const int32_t* order,
+                              const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels, const float* X,
+                              float* Y, float* workspace, float* z_scratch, int32_t n, int32_t d, int64_t ldx, int64_t ldy,
+                              int32_t flags, void* stream) {
+    if (n_levels < 2 || n_levels > kMaxPathLevels || n <= 0 || d <= 0)     // flat or deep: the level plan
+        return cbm_spmm_update_f32(rowptr, idx, nnz, m, coef, parent, row_sched, order, level_off_dev, level_off_host,
+                                   n_levels, X, Y, workspace, n, d, ldx, ldy, flags, stream);
+    if (!parent || !z_scratch || !Y) return CBM_ERR_NULL;
+    if (X == Y) return CBM_ERR_SHAPE;                    // as cbm_spmm_update_f32
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+        return CBM_ERR_UNSUPPORTED;
+    if (int rc = check_matrix(n, d, ldy)) return rc;
+    if (int rc = validate_levels(level_off_host, n_levels, n)) return rc;
+    if (!aligned(z_scratch, 16)) return CBM_ERR_SHAPE;
+    const int64_t ldz = (d + 3) & ~3;                     // rows of the scratch start on 16 bytes
+    const int64_t z_bytes = (int64_t)n * ldz * 4;
+    if (ranges_overlap(z_scratch, z_bytes, Y, matrix_bytes(n, d, ldy)) ||
+        ranges_overlap(z_scratch, z_bytes, X, matrix_bytes(n, d, ldx)) ||
+        (workspace && ranges_overlap(z_scratch, z_bytes, workspace, copy_floats(n, d) * 4)))
+        return CBM_ERR_SHAPE;
+    int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
+    if (flags & CBM_UPDATE_WORKSPACE_PRESCALED) spmm_flags |= CBM_SPMM_WORKSPACE_PRESCALED;
+    // children of the root are scaled by the SpMM epilogue: their rows of the scratch are final
+    if (int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, z_scratch, workspace, spmm_flags, n, d, ldx,
+                              ldz, stream))
+        return rc;
+    const Tiling t = pick_tiling(d, ldz, ldy, z_scratch, Y);
+    const dim3 grid((n + kWavesPerBlock - 1) / kWavesPerBlock, t.grid_y), block(kWave * kWavesPerBlock);
+    const int dv = d - d % 8, relu = (flags & CBM_UPDATE_RELU) ? 1 : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define LAUNCH(V, C, F)                                                                                         \
+    do {                                                                                                        \
+        if (m) hipLaunchKernelGGL((propagate_paths<V, C, true, F>), grid, block, 0, s, parent, m, z_scratch, Y, \
+                                  n, d, dv, ldz, ldy, relu);                                                    \
+        else hipLaunchKernelGGL((propagate_paths<V, C, false, F>), grid, block, 0, s, parent, m, z_scratch, Y,  \
+                                n, d, dv, ldz, ldy, relu);                                                      \
+    } while (0)
+    CBM_DISPATCH_TILING(t, LAUNCH);
+#undef LAUNCH
+    return check_launch();
+}
+
+int64_t cbm_spmm_update_paths_scratch_floats(int32_t n, int32_t d, int32_t n_levels) {
+    if (n <= 0 || d <= 0 || n_levels < 2 || n_levels > kMaxPathLevels) return 0;
+    return (int64_t)n * ((d + 3) & ~3);
 }
 
 int64_t cbm_spmm_tiled_workspace_floats(const cbm_tiling_dev* t, int32_t n, int32_t d) {

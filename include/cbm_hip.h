@@ -322,14 +322,38 @@ int cbm_spmm_update_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int6
                         const float* X_dev, float* Y_dev, float* workspace_dev, int32_t n, int32_t d,
                         int64_t ldx, int64_t ldy, int32_t flags, void* stream);
 
+/* Deepest tree (levels, children of the root = level 0) that cbm_spmm_update_paths_f32 walks in one launch. */
+#define CBM_PATH_MAX_LEVELS 16
+
+/* cbm_spmm_update_f32 for SHALLOW trees, where a launch per level costs more than the level's work
+ * (replaces the same reference functions).  With 2 <= n_levels <= CBM_PATH_MAX_LEVELS the SpMM writes
+ * Z into z_scratch (n rows of stride (d + 3) & ~3 floats, 16-byte aligned, cbm_spmm_update_paths_scratch_floats)
+ * and ONE more launch finishes the product: the wavefront of row v follows parent[] up to the child of
+ * the root above it and adds the rows of Z down that path, with the arithmetic of cbm_propagate_f32
+ * step by step, so Y is bit for bit what cbm_spmm_update_f32 returns; CBM_UPDATE_RELU goes into that
+ * launch's store.  Rows recompute their ancestors' values (sum of depths row reads instead of n), which
+ * pays while the rows stay in cache and the levels are few: the caller decides.  Any other depth (flat,
+ * or deeper than the limit) is handed to cbm_spmm_update_f32 unchanged and z_scratch is not touched.
+ * z_scratch must not overlap X, Y or the workspace. */
+int cbm_spmm_update_paths_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz, const float* m_dev,
+                              const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
+                              const int32_t* order_dev, const int32_t* level_off_dev,
+                              const int32_t* level_off_host, int32_t n_levels, const float* X_dev, float* Y_dev,
+                              float* workspace_dev, float* z_scratch_dev, int32_t n, int32_t d, int64_t ldx,
+                              int64_t ldy, int32_t flags, void* stream);
+
+/* Floats of z_scratch that cbm_spmm_update_paths_f32 uses: n * ((d + 3) & ~3) for 2 <= n_levels <=
+ * CBM_PATH_MAX_LEVELS, else 0 (the call then falls back to cbm_spmm_update_f32). */
+int64_t cbm_spmm_update_paths_scratch_floats(int32_t n, int32_t d, int32_t n_levels);
+
 /* cbm_spmm_update_f32 for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring the
  * workspace of the slab-major copy of X either.  No counterpart in the reference.  Same arguments
  * minus the workspace, same result bit for bit as cbm_spmm_update_f32 with a workspace of
  * cbm_spmm_workspace_floats() floats: the copy goes to a static device array of
  * CBM_STATIC_SCRATCH_FLOATS floats (128 MiB) that every device the library runs on holds until the
- * process ends.  A shape whose copy needs more (n * 32 * ceil(d / 32) floats, slab count rounded up
- * to 1, 2, 4 or 8 below 8) is rejected with CBM_ERR_SCRATCH and nothing is enqueued.  The call
+ * process ends.  A shape whose copy needs more (cbm_relayout_floats(n, d) floats) is rejected with
+ * CBM_ERR_SCRATCH and nothing is enqueued.  The call
  * allocates and frees nothing, on host or device.  All calls on one device share that device's
  * array: calls that may overlap in time on one device (different streams, different threads)
  * race on it; serialise them.  The array keeps the previous call's contents; every float the

@@ -582,6 +582,69 @@ def test_relu_epilogue_and_masked_copy_through_the_c_abi(orc):
             assert torch.equal(via_copy, direct)
 
 
+def test_path_walk_equals_the_level_by_level_walk(orc):
+    """cbm_spmm_update_paths_f32 (one launch after the SpMM: every row sums down its own ancestor path)
+    returns what the level-by-level walk returns, bit for bit: plain and normalised, with and without the
+    ReLU, widths with a scalar tail (d mod 8 != 0), a strided destination, the deepest tree it takes;
+    deeper and flat trees are handed to the level plan."""
+    from cbm4gnn_amd.cbm import _ptr
+    n = 900
+    ei = graphs.add_self_loops(graphs.sbm(n, 6, 0.6, 0.01, seed=21), n)
+    for normalized in (False, True):
+        for max_levels in (None, _lib.CBM_PATH_MAX_LEVELS, 3):
+            mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized, max_levels=max_levels)
+            say("path walk", normalized, max_levels, "levels", mat.n_levels)
+            assert mat.n_levels >= 3
+            for d in (10, 41, 128, 1028):
+                x = torch.randn((n, d), generator=torch.Generator().manual_seed(d)).cuda()
+                for relu in (False, True):
+                    mat.path_walk_max_bytes = 0
+                    want = torch.empty_like(x); mat._run_spmm_update(x, want, use_m=normalized, relu=relu)
+                    mat.path_walk_max_bytes = 64 << 20
+                    assert mat._walks_paths(n, d) == (mat.n_levels <= _lib.CBM_PATH_MAX_LEVELS)
+                    got = torch.full((n, d + 8), float("nan"), device="cuda")[:, :d]
+                    mat._run_spmm_update(x, got, use_m=normalized, relu=relu)
+                    assert torch.equal(got, want)
+            # and against the oracle, end to end
+            x = np.random.default_rng(5).standard_normal((n, 64)).astype(np.float32)
+            assert np.array_equal(gpu_product(mat, x, normalized), oracle_product(orc, mat, ei, n, x, normalized))
+    # the C-ABI: overlapping scratch is refused, depths out of range fall back without touching the scratch
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=False, max_levels=4)
+    st = mat._device_arrays(torch.device("cuda", 0))
+    d = 64
+    x = torch.randn((n, d), generator=torch.Generator().manual_seed(1)).cuda()
+    y = torch.empty_like(x)
+    lib = _lib.hip_lib()
+    assert lib.cbm_spmm_update_paths_scratch_floats(n, d, 4) == n * d
+    assert lib.cbm_spmm_update_paths_scratch_floats(n, 41, 4) == n * 44
+    assert lib.cbm_spmm_update_paths_scratch_floats(n, d, 1) == 0
+    assert lib.cbm_spmm_update_paths_scratch_floats(n, d, _lib.CBM_PATH_MAX_LEVELS + 1) == 0
+
+    def call(scratch, n_levels=mat.n_levels, level_off=mat.level_off):
+        return lib.cbm_spmm_update_paths_f32(
+            _ptr(st["rowptr"]), _ptr(st["idx"]), mat.nnz, None, None, _ptr(st["parent"]), _ptr(st["sched"]), _ptr(st["order"]),
+            _ptr(st["level_off"]), _ptr(level_off), n_levels, _ptr(x), _ptr(y), None, scratch, n, d, d, d, 0, None)
+    assert call(C.c_void_p(y.data_ptr() + 64)) == _lib.CBM_ERR_SHAPE
+    assert call(C.c_void_p(x.data_ptr())) == _lib.CBM_ERR_SHAPE
+    assert call(None) == _lib.CBM_ERR_NULL
+    scratch = torch.full((n * d,), 7.0, device="cuda")
+    assert call(_ptr(scratch)) == 0
+    torch.cuda.synchronize()
+    want = torch.empty_like(x); mat.path_walk_max_bytes = 0; mat._run_spmm_update(x, want, use_m=False)
+    assert torch.equal(y, want) and float(scratch.min()) != 7.0
+    flat = cbm_matrix(torch.from_numpy(ei), None, alpha=10_000, normalized=False)
+    assert flat.n_levels == 1
+    fs = flat._device_arrays(torch.device("cuda", 0))
+    scratch.fill_(7.0)
+    rc = lib.cbm_spmm_update_paths_f32(
+        _ptr(fs["rowptr"]), _ptr(fs["idx"]), flat.nnz, None, None, _ptr(fs["parent"]), _ptr(fs["sched"]), _ptr(fs["order"]),
+        _ptr(fs["level_off"]), _ptr(flat.level_off), 1, _ptr(x), _ptr(y), None, _ptr(scratch), n, d, d, d, 0, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and float(scratch.min()) == 7.0 and float(scratch.max()) == 7.0
+    want = torch.empty_like(x); flat._run_spmm_update(x, want, use_m=False)
+    assert torch.equal(y, want)
+
+
 def test_degenerate_shapes(orc):
     # empty rows, a single-row matrix, d = 1, more slabs than rows
     ei = np.array([[0, 1, 2, 4, 2], [0, 2, 1, 2, 4]], np.int32)      # row 3 is empty
