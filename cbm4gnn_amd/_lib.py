@@ -92,6 +92,7 @@ HIP_SYMBOLS = {
     "cbm_set_spmm_occupancy": (C.c_int, [C.c_int]),
     "cbm_spmm_summation_groups": (C.c_int, [_I32, _I64, _I64, _P, _P, _I32]),
     "cbm_spmm_tail_columns": (C.c_int, [_I32, _I64, _I64, _P, _P, _I32]),
+    "cbm_set_tiled_fused": (C.c_int, [C.c_int]),
     "cbm_relayout_floats": (C.c_int64, [_I32, _I32]),
     "cbm_spmm_workspace_floats": (C.c_int64, [_I32, _I32, _I64, _I64, _P, _P]),
     "cbm_expand_coef_f32": (C.c_int, [_P, _P, _P, _I64, _P]),

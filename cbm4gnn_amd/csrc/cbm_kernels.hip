@@ -46,6 +46,12 @@ namespace {
 #ifndef CBM_TILED_VECS
 #define CBM_TILED_VECS 6                   // 16-byte index vectors requested together per row in the tiled kernel
 #endif
+#ifndef CBM_TILED_REMOTE_U8
+#define CBM_TILED_REMOTE_U8 8              // remote entries per row in flight in the tiled kernel, 128-byte slabs (2 rows per lane)
+#endif
+#ifndef CBM_TILED_REMOTE_U4
+#define CBM_TILED_REMOTE_U4 8              // the same for the 64-byte half slab (1 row per lane)
+#endif
 #ifndef CBM_XCD_REMAP
 #define CBM_XCD_REMAP 1
 #endif
@@ -391,10 +397,16 @@ constexpr int kTiledWaves = 16;            // one 1024-thread workgroup
 // LPE lanes serve one row: 8 for the 128-byte slabs, 4 for the 64-byte half slab of the last
 // d % 32 columns (then 16 rows per wave in lockstep, one set per wave, and W / Z / d are those of
 // the half slab: W its copy, Z already offset to its first column, d its width, n_slabs = 1).
-template <int TILE, bool SIGNED, int LPE>
+// FUSED: the same lane group also gathers its row's REMOTE entries (rowptr_r / idx_r, packed like
+// idx) straight from the slab-major copy in global memory once the panel's blocks are done, eight
+// entries per row and set in flight, added strictly in order; nothing is read from Z and no launch
+// of the slab kernel is needed.  While one workgroup waits on the fabric in that phase, the
+// workgroups of other CUs are in their LDS phase: the two resources overlap across the chip.
+template <int TILE, bool SIGNED, int LPE, bool FUSED>
 __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_tiled_local(
     const int32_t* __restrict__ panel_ptr, const int32_t* __restrict__ blk_tile, const int32_t* __restrict__ seg,
-    const uint16_t* __restrict__ lidx, const float* __restrict__ W, float* __restrict__ Z,
+    const uint16_t* __restrict__ lidx, const int32_t* __restrict__ rowptr_r, const uint32_t* __restrict__ idx_r,
+    const float* __restrict__ W, float* __restrict__ Z,
     const float* __restrict__ row_scale, int n, int d, int n_slabs, int n_panels, int64_t ldz, int relu, int vec_out) {
     constexpr int kGroups = kWave / LPE;                   // rows a wave serves in lockstep
     constexpr int kTiledSets = kPanelRows / (kTiledWaves * kGroups);
@@ -494,6 +506,70 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
             }
         }
 #undef CBM_FETCH_TILE
+        float racc[kTiledSets][4];                         // FUSED: the remote entries' sum, in entry order
+        if constexpr (FUSED) {
+            int rs[kTiledSets], rn[kTiledSets], longest = 0;
+#pragma unroll
+            for (int t = 0; t < kTiledSets; t++) {
+                const int row = panel * kPanelRows + t * (kTiledWaves * kGroups) + wave * kGroups + sub;
+                rs[t] = 0; rn[t] = 0;
+                if (row < n) { rs[t] = rowptr_r[row]; rn[t] = rowptr_r[row + 1] - rs[t]; }
+                longest = max(longest, rn[t]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) racc[t][e] = 0.0f;
+            }
+#pragma unroll
+            for (int off = LPE; off < kWave; off <<= 1) longest = max(longest, __shfl_xor(longest, off, kWave));
+            longest = __builtin_amdgcn_readfirstlane(longest);
+            // uniform base of the slab + 32-bit byte offset per lane (the host checks n * 16 LPE < 2^32)
+            const char* __restrict__ Ws = reinterpret_cast<const char*>(W + (int64_t)slab * n * kRowFloats);
+            const uint32_t lane_off = (uint32_t)li * 16u;
+            // entries per row in flight: the registers of the LDS phase are free here
+            constexpr int kRU = LPE == 8 ? CBM_TILED_REMOTE_U8 : CBM_TILED_REMOTE_U4;
+            constexpr int kPer = (kRU + LPE - 1) / LPE;    // index words per lane and round
+            // word q of lane li of a group holds entry k + q * LPE + li of the group's row; next
+            // round's indices are requested before this round's rows
+            uint32_t mine[kTiledSets][kPer], nxt[kTiledSets][kPer];
+            auto fetch_idx = [&](int k, uint32_t (&out)[kTiledSets][kPer]) {
+#pragma unroll
+                for (int t = 0; t < kTiledSets; t++)
+#pragma unroll
+                    for (int q = 0; q < kPer; q++) {
+                        const int kk = k + q * LPE + li;
+                        out[t][q] = (q * LPE + li < kRU && kk < rn[t]) ? idx_r[rs[t] + kk] : 0u;
+                    }
+            };
+            if (longest > 0) fetch_idx(0, nxt);
+            for (int k = 0; k < longest; k += kRU) {
+#pragma unroll
+                for (int t = 0; t < kTiledSets; t++)
+#pragma unroll
+                    for (int q = 0; q < kPer; q++) mine[t][q] = nxt[t][q];
+                if (k + kRU < longest) fetch_idx(k + kRU, nxt);
+                f32x4 x[kTiledSets][kRU];
+                uint32_t p[kTiledSets][kRU];
+#pragma unroll
+                for (int t = 0; t < kTiledSets; t++)
+#pragma unroll
+                    for (int u = 0; u < kRU; u++) {
+                        p[t][u] = (uint32_t)__shfl((int)mine[t][u / LPE], (lane & ~(LPE - 1)) + (u % LPE), kWave);
+                        // past the row's end: row 0, masked below
+                        x[t][u] = *reinterpret_cast<const f32x4*>(Ws + ((p[t][u] & 0x7fffffffu) * (uint32_t)(LPE * 16) + lane_off));
+                    }
+#pragma unroll
+                for (int t = 0; t < kTiledSets; t++)
+#pragma unroll
+                    for (int u = 0; u < kRU; u++) {
+                        const bool live = k + u < rn[t];
+                        const float f = SIGNED ? __uint_as_float(0x3f800000u | (p[t][u] & 0x80000000u)) : 1.0f;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float v = live ? x[t][u][e] : 0.0f;
+                            racc[t][e] = SIGNED ? fmaf(f, v, racc[t][e]) : racc[t][e] + v;
+                        }
+                    }
+            }
+        }
         // epilogue: every lane group adds its row's local sum to the remote part
 #pragma unroll
         for (int t = 0; t < kTiledSets; t++) {
@@ -502,7 +578,21 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
             if (row < n && col < d) {
                 float* __restrict__ zr = Z + (int64_t)row * ldz + col;
                 const float sc = row_scale ? row_scale[row] : 1.0f;
-                if (vec_out) {
+                if constexpr (FUSED) {
+                    float z[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        z[e] = (racc[t][e] + acc[t][e]) * sc;
+                        if (relu) z[e] = z[e] < 0.0f ? 0.0f : z[e];
+                    }
+                    if (vec_out) {
+                        *reinterpret_cast<float4*>(zr) = make_float4(z[0], z[1], z[2], z[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (col + e < d) zr[e] = z[e];
+                    }
+                } else if (vec_out) {
                     float4 z = *reinterpret_cast<const float4*>(zr);
                     z.x = (z.x + acc[t][0]) * sc; z.y = (z.y + acc[t][1]) * sc;
                     z.z = (z.z + acc[t][2]) * sc; z.w = (z.w + acc[t][3]) * sc;
@@ -1111,6 +1201,9 @@ inline int check_matrix(int32_t n, int32_t d, int64_t ld) {
 // rows averaging 13 entries at the register limit (6 costs 7 %); 256-byte slabs are fastest at
 // 3-4 on every graph tried.
 std::atomic<int> g_spmm_occupancy{0};                      // 0 = automatic
+// Tiled multiply: 1 = the kernel of the local blocks gathers the remote entries too (when no row is
+// cut), 0 = the remote entries always go through the slab kernel first.  A tuning hook.
+std::atomic<int> g_tiled_fused{1};
 inline int slab_waves_per_simd(int64_t nnz, int32_t n, int lpe) {
     const int fixed = g_spmm_occupancy.load(std::memory_order_relaxed);
     if (fixed > 0) return fixed;
@@ -1526,6 +1619,11 @@ int cbm_spmm_summation_groups(int32_t d, int64_t ldx, int64_t ldz, const void* X
     return p.n_slabs > 0 ? kWave / p.lpe : kWave / 4;      // only the half slab: d <= 16
 }
 
+int cbm_set_tiled_fused(int on) {
+    g_tiled_fused.store(on ? 1 : 0, std::memory_order_relaxed);
+    return CBM_OK;
+}
+
 int cbm_spmm_tail_columns(int32_t d, int64_t ldx, int64_t ldz, const void* X, const void* Z, int32_t have_workspace) {
     const SlabPlan p = plan_slabs(d, ldx, ldz, X, Z, have_workspace != 0, false);
     return (p.lpe && p.tail) ? d - p.n_slabs * 32 : 0;
@@ -1668,15 +1766,19 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     if (ready && ((m != nullptr) != ((flags & CBM_SPMM_WORKSPACE_PRESCALED) != 0))) return CBM_ERR_UNSUPPORTED;
     if (!ready && (flags & CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
     if (n == 0 || d == 0) return CBM_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const DeviceFacts* facts = device_facts();
-    if (!facts || facts->cus < kXcds) return CBM_ERR_LAUNCH;
-    if (!ready) {                                         // launch_spmm checks alignment and overlap of the workspace below
-        if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
-        const int64_t ws_bytes = copy_floats(n, d) * 4;
+    // as cbm_spmm_f32: X and Z must not share a byte, nor the workspace with either
+    if (X == Z || ranges_overlap(X, matrix_bytes(n, d, ldx), Z, matrix_bytes(n, d, ldz))) return CBM_ERR_SHAPE;
+    if (!aligned(workspace, 16)) return CBM_ERR_SHAPE;
+    {
+        const int64_t ws_bytes = cbm_spmm_tiled_workspace_floats(t, n, d) * 4;
         if (ranges_overlap(workspace, ws_bytes, X, matrix_bytes(n, d, ldx)) ||
             ranges_overlap(workspace, ws_bytes, Z, matrix_bytes(n, d, ldz)))
             return CBM_ERR_SHAPE;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const DeviceFacts* facts = device_facts();
+    if (!facts || facts->cus < kXcds) return CBM_ERR_LAUNCH;
+    if (!ready) {
         if (int rc = launch_relayout(X, workspace, n, d, ldx, s, nullptr, 0, m)) return rc;
     }
     // remote entries: the slab kernel from the copy.  With local blocks the left scale and the ReLU
@@ -1689,9 +1791,14 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     float* partials = t->n_long > 0 ? workspace + copy_floats(n, d) : nullptr;
     const int remote_flags = CBM_SPMM_WORKSPACE_READY | (m ? CBM_SPMM_WORKSPACE_PRESCALED : 0) |
                              ((relu && !has_local) ? CBM_SPMM_RELU : 0);
-    if (int rc = launch_spmm<true>(t->rowptr_r, t->idx_r, t->nnz_remote, nullptr, m, nullptr, t->sched_r, X, Z, workspace,
-                                   remote_flags, n, d, ldx, ldz, s, t->n_long > 0 ? t->n_sched_r : 0, partials, t->n_pieces))
-        return rc;
+    // With local blocks and no cut rows, the kernel of the local part gathers the remote entries too.
+    const bool fused = has_local && t->n_long == 0 && (int64_t)n * 128 < ((int64_t)1 << 32) &&
+                       g_tiled_fused.load(std::memory_order_relaxed) != 0;
+    if (!fused)
+        if (int rc = launch_spmm<true>(t->rowptr_r, t->idx_r, t->nnz_remote, nullptr, m, nullptr, t->sched_r, X, Z, workspace,
+                                       remote_flags, n, d, ldx, ldz, s, t->n_long > 0 ? t->n_sched_r : 0, partials,
+                                       t->n_pieces))
+            return rc;
     if (t->n_long > 0) {                                  // pieces of cut rows -> their rows of Z, per column range
         const int4* lr = reinterpret_cast<const int4*>(t->long_rows);
         const int scale_here = has_local ? 0 : 1, relu_here = (relu && !has_local) ? 1 : 0;
@@ -1706,16 +1813,21 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     if (!has_local) return check_launch();
     // local entries: tiles of the copy staged in LDS; adds to Z, then scale and ReLU
     const int G = facts->cus / kXcds;                     // 129 KB of LDS: one workgroup per CU
-#define LAUNCH_TILED(T, S, L, WL, ZL, DL, SLABS)                                                                         \
+#define LAUNCH_TILED_F(T, S, L, F, WL, ZL, DL, SLABS)                                                                    \
     do {                                                                                                                 \
         const size_t bytes_ = (size_t)(T + 1) * L * 16;                                                                  \
         const int vec_ = (d % 4 == 0 && ldz % 4 == 0 && aligned(ZL, 16)) ? 1 : 0;                                        \
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S, L>),                                \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(spmm_tiled_local<T, S, L, F>),                             \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes_) != hipSuccess)                  \
             return CBM_ERR_LAUNCH;                                                                                       \
-        hipLaunchKernelGGL((spmm_tiled_local<T, S, L>), dim3(G * kXcds), dim3(kWave * kTiledWaves), bytes_, s,           \
-                           t->panel_ptr, t->blk_tile, t->seg, t->lidx, WL, ZL, t->row_scale, n, DL, SLABS, t->n_panels,  \
-                           ldz, relu, vec_);                                                                             \
+        hipLaunchKernelGGL((spmm_tiled_local<T, S, L, F>), dim3(G * kXcds), dim3(kWave * kTiledWaves), bytes_, s,        \
+                           t->panel_ptr, t->blk_tile, t->seg, t->lidx, t->rowptr_r, t->idx_r, WL, ZL, t->row_scale, n,   \
+                           DL, SLABS, t->n_panels, ldz, relu, vec_);                                                     \
+    } while (0)
+#define LAUNCH_TILED(T, S, L, WL, ZL, DL, SLABS)                                                                         \
+    do {                                                                                                                 \
+        if (fused) LAUNCH_TILED_F(T, S, L, true, WL, ZL, DL, SLABS);                                                     \
+        else LAUNCH_TILED_F(T, S, L, false, WL, ZL, DL, SLABS);                                                          \
     } while (0)
 #define LAUNCH_TILED_BOTH(T, S)                                                                                          \
     do {                                                                                                                 \
@@ -1726,6 +1838,7 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     else { if (t->has_negative) LAUNCH_TILED_BOTH(512, true); else LAUNCH_TILED_BOTH(512, false); }
 #undef LAUNCH_TILED_BOTH
 #undef LAUNCH_TILED
+#undef LAUNCH_TILED_F
     return check_launch();
 }
 

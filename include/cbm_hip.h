@@ -217,6 +217,13 @@ int cbm_set_spmm_kernel(int kind);
  * hook; no reference counterpart. */
 int cbm_set_spmm_occupancy(int waves_per_simd);
 
+/* Tiled multiply (cbm_spmm_tiled_f32) for later calls of this process: 1 (default) = when the plan
+ * cuts no rows, the kernel of the local blocks also gathers the remote entries, straight from the
+ * slab-major copy and strictly in entry order (one launch instead of two, no pass over Z in
+ * between); 0 = the remote entries always go through the slab kernel first (8 or 16 partial sums).
+ * A tuning hook; no reference counterpart. */
+int cbm_set_tiled_fused(int on);
+
 /* How many interleaved partial sums the SpMM keeps per output element for this shape (1 = the
  * entries of a row are accumulated strictly in order; g > 1 = entry k goes to partial sum
  * k mod g and the g sums are added as a balanced tree).  Lets a checker reproduce the fp32

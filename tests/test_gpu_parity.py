@@ -156,14 +156,19 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         return grouped_with_cuts(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
                                  mat.split_chunk, plan_groups, plan_tail)
     if mat.relayout and mat.is_tiled():
-        # tiled multiply: (remote entries, 8 interleaved partial sums) + (local entries in column order,
-        # one after the other), on the copy of X scaled by m
+        # tiled multiply: (remote entries) + (local entries in storage order, one after the other), on the
+        # copy of X scaled by m.  Remote entries: when no row is cut, the kernel of the local part gathers
+        # them itself, one after the other in column order; otherwise (or with that fusion switched off)
+        # the slab kernel sums them in 8 interleaved partial sums (16 in the half slab), pieces in order.
         local, row = tiled_split(mat)
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
         c, sg = col.numpy(), sign.numpy().astype(np.float32)
         rp = np.concatenate([[0], np.cumsum(np.bincount(row[~local], minlength=n))]).astype(np.int32)
-        remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs,
-                                   mat.split_chunk if mat.has_cut_rows() else 0, plan_groups, plan_tail)
+        if TILED_FUSED and not mat.has_cut_rows():
+            remote = orc.csr_spmm(rp, c[~local].astype(np.int32), sg[~local], xs, groups=1)
+        else:
+            remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs,
+                                       mat.split_chunk if mat.has_cut_rows() else 0, plan_groups, plan_tail)
         # local entries in storage order: by tile, then the columns of the row's own parity, then the others
         lr, lc, ls = row[local], c[local], sg[local]
         order = np.lexsort((lc, (lc + lr) % 2, lc // mat.tile_rows, lr))
@@ -177,6 +182,22 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
                             (m[:, None] * x).astype(np.float32), g, tail)
     val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
     return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, g, tail)
+
+
+TILED_FUSED = True            # state of cbm_set_tiled_fused (the library's default), for the oracle's order
+
+
+@pytest.fixture(params=[True, False], ids=["fused", "two-launch"])
+def tiled_fused(request):
+    """Run a test of the tiled multiply once with the remote entries gathered by the kernel of the local
+    part (default) and once with the slab kernel gathering them first."""
+    global TILED_FUSED
+    lib = _lib.hip_lib()
+    assert lib.cbm_set_tiled_fused(int(request.param)) == 0
+    TILED_FUSED = request.param
+    yield request.param
+    assert lib.cbm_set_tiled_fused(1) == 0
+    TILED_FUSED = True
 
 
 @pytest.fixture(params=["auto", "wave-per-row"])
@@ -991,10 +1012,11 @@ def test_gpu_built_format_counts_equal_the_oracle_build(orc):
 
 @pytest.mark.parametrize("normalized", [False, True])
 @pytest.mark.parametrize("alpha", [0, 10 ** 6])
-def test_tiled_multiply_against_oracle(orc, normalized, alpha):
-    """``tiling="on"``: local blocks gathered from LDS tiles, the rest by the slab kernel.  Bit for
-    bit against the oracle in the documented order -- (remote entries in 8 interleaved partial sums)
-    + (local entries one after the other in storage order) -- for signed deltas (alpha = 0) and a flat tree of
+def test_tiled_multiply_against_oracle(orc, normalized, alpha, tiled_fused):
+    """``tiling="on"``: local blocks gathered from LDS tiles, the rest from the slab-major copy by the same
+    kernel (in column order) or by the slab kernel first (8 interleaved partial sums).  Bit for
+    bit against the oracle in the documented order -- (remote entries) + (local entries one after the
+    other in storage order) -- for signed deltas (alpha = 0) and a flat tree of
     all-positive entries (alpha huge), widths on both store paths, with and without the ReLU, the
     SpMM alone, and the un-fused methods."""
     n = 3000
