@@ -305,9 +305,13 @@ def gcn_epoch(args, torch, workload="c4"):
         return TwoLayerGCN(CBMGCNLayer(w.d, hidden, op, fused=fused, relu=fused),
                            CBMGCNLayer(hidden, classes, op, fused=fused), relu_between=not fused).to(dev)
 
+    label_col = labels[:, None]
+
     def epoch(net):
         net.zero_grad(set_to_none=True)
-        loss = torch.nn.functional.cross_entropy(net(x), labels)
+        # mean cross entropy, written as log-softmax + gather: torch's nll_loss kernels reduce the 233k rows
+        # in one workgroup (0.34 ms forward + 0.21 ms backward per epoch, for all three models alike)
+        loss = -torch.log_softmax(net(x), dim=1).gather(1, label_col).mean()
         loss.backward()
         return loss
 
