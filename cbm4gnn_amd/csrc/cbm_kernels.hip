@@ -417,27 +417,15 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
     const int sub = lane / LPE, li = lane % LPE;
     if (threadIdx.x < LPE) tile_lds[TILE * LPE + threadIdx.x] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     constexpr uint32_t kPad = (uint32_t)(TILE * 8) | ((uint32_t)(TILE * 8) << 16);    // two entries of the zero row
-    // Workgroup b runs on XCD b % 8.  Slabs are pinned to XCDs as in the slab kernel, so that an
-    // XCD's L2 only ever sees its own slabs of the copy (tiles and remote rows alike):
-    //   n_slabs >= 8 (a multiple of 8): XCD x takes slabs x, x + 8, ... and every panel;
-    //   n_slabs < 8 (a divisor of 8): the 8 / n_slabs XCDs of a slab split the panels into
-    //     contiguous ranges.
-    // An XCD's items are dealt cyclically to its workgroups: they work on neighbouring panels of
-    // one slab at the same time, which share their tiles through the XCD's L2.
+    // Workgroup b runs on XCD b % 8.  Items (panel-major, slab-minor) are cut into 8 contiguous
+    // ranges, one per XCD, and dealt cyclically to the XCD's workgroups: the workgroups of an XCD
+    // work on neighbouring panels at the same time, which share their tiles through the XCD's L2.
     const int xcd = blockIdx.x % kXcds, j0 = blockIdx.x / kXcds, G = gridDim.x / kXcds;
-    int slab0, slab_step, panel0, panel_end;
-    if (n_slabs >= kXcds) {
-        slab0 = xcd; slab_step = kXcds; panel0 = 0; panel_end = n_panels;
-    } else {
-        const int share = kXcds / n_slabs, part = xcd / n_slabs;
-        const int chunk = (n_panels + share - 1) / share;
-        slab0 = xcd % n_slabs; slab_step = n_slabs;        // a single slab for this XCD
-        panel0 = part * chunk; panel_end = min(panel0 + chunk, n_panels);
-    }
-    const int my_panels = max(panel_end - panel0, 0);
-    const int items = my_panels * ((n_slabs - slab0 + slab_step - 1) / slab_step);
-    for (int item = j0; item < items; item += G) {
-        const int panel = panel0 + item % my_panels, slab = slab0 + (item / my_panels) * slab_step;
+    const int items = n_panels * n_slabs;
+    const int chunk = (items + kXcds - 1) / kXcds;
+    const int item_end = min((xcd + 1) * chunk, items);
+    for (int item = xcd * chunk + j0; item < item_end; item += G) {
+        const int panel = item / n_slabs, slab = item % n_slabs;
         float acc[kTiledSets][4];
 #pragma unroll
         for (int t = 0; t < kTiledSets; t++)
