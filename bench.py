@@ -23,6 +23,7 @@ feature width 256.  Prints ONE JSON line.  The default run also carries, in the 
 from __future__ import annotations
 
 import argparse
+import contextlib
 import glob
 import hashlib
 import json
@@ -275,7 +276,7 @@ def gcn_epoch(args, torch, workload="c4"):
     import numpy as np
 
     from cbm4gnn_amd import graphs
-    from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator
+    from cbm4gnn_amd.gcn import CBMGCNLayer, CSRGCNLayer, TwoLayerGCN, build_operator, csr_operator, tuned_gemms
 
     t0 = time.perf_counter()
     w = graphs.workload(workload, scale=args.scale)
@@ -328,7 +329,10 @@ def gcn_epoch(args, torch, workload="c4"):
         return a.elapsed_time(b) / args.steps, float(loss.detach())
 
     nets = {k: make(k) for k in ("cbm_fused", "cbm_unfused", "csr")}
-    res = {k: run(v) for k, v in nets.items()}
+    # the dense GEMMs of all three models alike run on the library solution torch's TunableOp measures
+    # fastest per shape (tuned during the warm-up epochs); --no-gemm-tuning leaves hipBLASLt's default pick
+    with (contextlib.nullcontext() if args.no_gemm_tuning else tuned_gemms()):
+        res = {k: run(v) for k, v in nets.items()}
     # aggregation alone: the 4 multiplies of an epoch (d = hidden and d = classes, forward and backward)
     agg = 0.0
     per_width = {}
@@ -351,6 +355,8 @@ def gcn_epoch(args, torch, workload="c4"):
         "aggregation_ms_per_epoch": agg, "aggregation_share": agg / ms, "multiply_ms_by_width": per_width,
         "loss": res["cbm_fused"][1], "loss_unfused_layers": res["cbm_unfused"][1], "loss_gpu_csr": res["csr"][1],
         "max_rel_weight_grad_diff_vs_gpu_csr": grad_err,
+        "dense_gemms": ("hipBLASLt default pick" if args.no_gemm_tuning else
+                        "library solution picked per shape by torch.cuda.tunable during warm-up (all three models)"),
         "host_s": {"generate": t_gen, "build_format": t_build, "build_phases": op.build_seconds},
     }
 
@@ -445,6 +451,9 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE), no timing, no JSON")
     ap.add_argument("--sweep", action="store_true",
                     help="alpha sweep (default workload c5): compression ratio and runtime per alpha")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="GCN epoch: leave the dense GEMMs on hipBLASLt's default pick instead of the solution "
+                         "torch's TunableOp measures fastest per shape (applies to all three models alike)")
     ap.add_argument("--gcn", action="store_true",
                     help="measure the 2-layer GCN forward+backward epoch (default workload c4) instead of the multiply")
     args = ap.parse_args()

@@ -31,13 +31,40 @@ the multiply:
 """
 from __future__ import annotations
 
+import contextlib
+import os
+import tempfile
+
 import torch
 from torch import nn
 
 from . import _lib
 from .cbm import CBMMatmul, _ld, _ptr, _wants_workspace, cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
 
-__all__ = ["CBMGCNLayer", "CSRGCNLayer", "TwoLayerGCN", "build_operator", "csr_operator", "CSRMatmul"]
+__all__ = ["CBMGCNLayer", "CSRGCNLayer", "TwoLayerGCN", "build_operator", "csr_operator", "CSRMatmul", "tuned_gemms"]
+
+
+@contextlib.contextmanager
+def tuned_gemms(max_ms_per_solution: int = 10, filename: str | None = None):
+    """Run the dense GEMMs inside the block on the library solution torch's TunableOp measures to be
+    fastest for each shape (first call of a shape inside the block tunes it, later calls reuse the pick).
+
+    The GEMMs around the aggregation are tall and skinny -- ``x W^T`` and the weight gradients
+    ``g^T x`` over N = 10^5..10^6 rows against 41..602 columns -- and hipBLASLt's default heuristic
+    serves the weight gradients badly (232,965 rows: 932 -> 484 us for 128 x N x 602, 435 -> 94 us for
+    41 x N x 128).  This is plumbing around the CBM multiply, not part of it; outside the block torch's
+    default choice is back.  The picks go to ``filename`` (default: a file in the temporary directory)."""
+    import torch.cuda.tunable as tunable
+    was_enabled, was_tuning = tunable.is_enabled(), tunable.tuning_is_enabled()
+    tunable.set_filename(filename or os.path.join(tempfile.gettempdir(), f"cbm4gnn_tunableop_{os.getpid()}.csv"))
+    tunable.set_max_tuning_duration(int(max_ms_per_solution))
+    tunable.enable(True)
+    tunable.tuning_enable(True)
+    try:
+        yield
+    finally:
+        tunable.tuning_enable(was_tuning)
+        tunable.enable(was_enabled)
 
 
 def build_operator(edge_index, alpha: int = 2, normalized: bool = True, builder: str = "auto") -> cbm_matrix:
