@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from cbm4gnn_amd import graphs
+from cbm4gnn_amd import _lib, graphs
 from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm
 
 pytestmark = pytest.mark.gpu
@@ -173,6 +173,14 @@ def test_gcn_graph_full_size_against_cpu_rows_and_gpu_csr(c4):
         assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
         ones = _mul(mat, torch.ones_like(xd))
         assert float(ones.min()) > 0.0 and torch.isfinite(ones).all()
+        # the two-launch plan (slab kernel on the remote entries first) sums the same entries in another order
+        assert mat.is_tiled() and not mat.has_cut_rows()
+        try:
+            assert _lib.hip_lib().cbm_set_tiled_fused(0) == 0
+            two = _mul(mat, xd)
+        finally:
+            assert _lib.hip_lib().cbm_set_tiled_fused(1) == 0
+        assert float((two - got).abs().max() / got.abs().max()) <= 1e-5 and not torch.equal(two, got)
 
 
 def test_gcn_epoch_full_size_anchored_rows(c4):
@@ -252,6 +260,11 @@ def test_duplication_graph_full_size():
         base = torch.empty_like(xd)
         csr_spmm(torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda(), val, xd, base)
         assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+        # the multiply walked the 11-level tree in one launch (every row down its own ancestor path): bit for
+        # bit what the level-by-level walk returns
+        assert mat._walks_paths(w.n, xd.size(1))
+        mat.path_walk_max_bytes = 0
+        assert torch.equal(_mul(mat, xd), got)
 
 
 def test_alpha_sweep_graph_same_format_for_every_alpha():
