@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes as C
+import os
 import warnings
 from collections import deque
 
@@ -231,6 +232,37 @@ def _build_staged(ei_cpu, n, alpha, threads, fmt, gpu, max_levels):
         host.cbm_builder_free(handle)
 
 
+def edge_fingerprint(edge_index, n=None) -> np.ndarray:
+    """Order-independent fingerprint of an edge list (uint64[4]: the number of edges, and three sums
+    modulo 2^64 over a 64-bit mix z of every edge key row * N + col: of z, of z * z and of a second
+    mix of z): equal for every ordering of the same edges, different -- for all practical purposes --
+    when an edge changes.  It keys the on-disk cache of the built format (no security claim: the
+    sums are additive)."""
+    ei = torch.as_tensor(edge_index).detach().to("cpu")
+    e = int(ei.size(1))
+    if n is None:
+        n = int(ei.max()) + 1 if e else 0
+
+    def s64(v):                                           # a 64-bit constant as torch's signed int64
+        return v - (1 << 64) if v >= (1 << 63) else v
+
+    def lsr(z, k):                                        # logical shift right (torch's >> is arithmetic)
+        return (z >> k) & ((1 << (64 - k)) - 1)
+
+    sums = [0, 0, 0]
+    for lo in range(0, e, 1 << 24):                       # int64 arithmetic wraps modulo 2^64
+        r = ei[0, lo:lo + (1 << 24)].to(torch.int64)
+        c = ei[1, lo:lo + (1 << 24)].to(torch.int64)
+        z = r * n + c + s64(0x9E3779B97F4A7C15)           # splitmix64 finaliser
+        z = (z ^ lsr(z, 30)) * s64(0xBF58476D1CE4E5B9)
+        z = (z ^ lsr(z, 27)) * s64(0x94D049BB133111EB)
+        z = z ^ lsr(z, 31)
+        y = (z ^ lsr(z, 33)) * s64(0xFF51AFD7ED558CCD)    # second mix (murmur3 finaliser step)
+        for i, t in enumerate((z, z * z, y ^ lsr(y, 29))):
+            sums[i] = (sums[i] + int(t.sum())) & ((1 << 64) - 1)
+    return np.array([e] + sums, np.uint64)
+
+
 class cbm_matrix:
 
     def __init__(self, edge_index, values, rows=None, cols=None, alpha=0, normalized=False,
@@ -308,10 +340,13 @@ class cbm_matrix:
         self.relayout = True                # False: gather from the caller's row-major X, no n*d scratch per call
         self._transposed = None
         self._edge_index_cpu = ei_cpu if not self.is_symmetric else None
+        self._edge_fingerprint, self._fingerprint_source = None, ei_cpu      # computed on first use (save, from_cache)
 
     # ------------------------------------------------------------------ on-disk cache --------
     _SAVED_ARRAYS = ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col")
-    FORMAT_VERSION = 2                  # 2 adds the depth limit (max_levels); version 1 files load with none
+    # 2 adds the depth limit (max_levels); 3 the fingerprint of the edge list the format was built from
+    # (what from_cache checks).  Older files load with no depth limit / no fingerprint.
+    FORMAT_VERSION = 3
 
     @staticmethod
     def _npz_path(path):
@@ -329,6 +364,8 @@ class cbm_matrix:
             arrays["edge_index"] = self._edge_index_cpu.numpy()
         meta = np.array([self.FORMAT_VERSION, self.num_rows, self.alpha, int(self.normalized), self.nnz, self.nnz_a,
                          self.n_candidates, self.n_levels, int(self.is_symmetric), self.max_levels or 0], np.int64)
+        if self.edge_fingerprint is not None:
+            arrays["edge_fingerprint"] = np.asarray(self.edge_fingerprint, np.uint64)
         np.savez(self._npz_path(path), meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
 
     @classmethod
@@ -337,7 +374,7 @@ class cbm_matrix:
         path = cls._npz_path(path)
         with np.load(path, allow_pickle=False) as z:
             meta = z["meta"].tolist()
-            if meta[0] not in (1, cls.FORMAT_VERSION):
+            if meta[0] not in (1, 2, cls.FORMAT_VERSION):
                 raise ValueError(f"unsupported CBM file version {meta[0]}")
             self = cls.__new__(cls)
             (_, self.num_rows, self.alpha, normalized, self.nnz, self.nnz_a, self.n_candidates, self.n_levels,
@@ -349,6 +386,8 @@ class cbm_matrix:
                 setattr(self, k, torch.from_numpy(z[k].copy()))
             self.col_multiplier = torch.from_numpy(z["col_multiplier"].copy()) if "col_multiplier" in z.files else None
             self._edge_index_cpu = torch.from_numpy(z["edge_index"].copy()) if "edge_index" in z.files else None
+            self._edge_fingerprint = z["edge_fingerprint"].copy() if "edge_fingerprint" in z.files else None
+            self._fingerprint_source = None
         n = self.num_rows
         ok = (self.rowptr.numel() == n + 1 and int(self.rowptr[-1]) == self.nnz == self.idx.numel()
               and self.parent.numel() == n and self.order.numel() == n and self.level_off.numel() == self.n_levels + 1
@@ -364,6 +403,39 @@ class cbm_matrix:
         self.relayout = True
         self._init_tiling("auto")
         return self
+
+    @property
+    def edge_fingerprint(self):
+        """``edge_fingerprint`` of the edge list this matrix was built from (None for a matrix loaded
+        from a file written before the fingerprint existed)."""
+        if self._edge_fingerprint is None and self._fingerprint_source is not None:
+            self._edge_fingerprint = edge_fingerprint(self._fingerprint_source, self.num_rows)
+            self._fingerprint_source = None
+        return self._edge_fingerprint
+
+    @classmethod
+    def from_cache(cls, path, edge_index, values=None, alpha=0, normalized=False, max_levels=None, **kwargs):
+        """The format of ``edge_index`` from the file at ``path`` when that file was built from the
+        same edges (``edge_fingerprint``) with the same ``alpha``, ``normalized`` and ``max_levels``;
+        otherwise build it (``cbm_matrix(edge_index, values, alpha=..., ...)``) and write the file.
+        The reference rebuilds on every run and caches only inside the process
+        (``cbm_message_passing.py:22-29``)."""
+        file = cls._npz_path(path)
+        if os.path.exists(file):
+            try:
+                got = cls.load(file)
+            except (ValueError, KeyError, OSError):
+                got = None
+            ei = torch.as_tensor(edge_index)
+            if (got is not None and got.edge_fingerprint is not None and got.alpha == int(alpha)
+                    and got.normalized == bool(normalized) and got.max_levels == (None if max_levels is None else int(max_levels))
+                    and np.array_equal(got.edge_fingerprint, edge_fingerprint(ei, got.num_rows))):
+                if "tiling" in kwargs:
+                    got._init_tiling(kwargs["tiling"])
+                return got
+        built = cls(edge_index, values, alpha=alpha, normalized=normalized, max_levels=max_levels, **kwargs)
+        built.save(file)
+        return built
 
     # ------------------------------------------------------------------ tiling --------------
     # Entries that cluster in (256-row panel, 1024-column tile) blocks -- graphs with community

@@ -159,3 +159,50 @@ def test_save_and_load_round_trip(tmp_path):
     np.savez(str(tmp_path / "bad.npz"), **bad)
     with pytest.raises(ValueError):
         cbm_matrix.load(str(tmp_path / "bad.npz"))
+
+
+def test_edge_fingerprint_and_cache_file(tmp_path):
+    """The cache file is keyed by an order-independent fingerprint of the edge list plus alpha, the
+    normalisation and the depth limit: same graph in another edge order -> loaded, anything else -> rebuilt."""
+    from cbm4gnn_amd.cbm import edge_fingerprint
+    ei = graphs.add_self_loops(graphs.sbm(300, 6, 0.5, 0.01, seed=2), 300)
+    perm = np.random.default_rng(0).permutation(ei.shape[1])
+    shuffled = np.ascontiguousarray(ei[:, perm])
+    assert np.array_equal(edge_fingerprint(ei), edge_fingerprint(shuffled))
+    assert edge_fingerprint(ei).dtype == np.uint64 and int(edge_fingerprint(ei)[0]) == ei.shape[1]
+    moved = ei.copy(); moved[1, 7] = (moved[1, 7] + 1) % 300               # one edge points elsewhere
+    assert not np.array_equal(edge_fingerprint(ei), edge_fingerprint(moved))
+    assert not np.array_equal(edge_fingerprint(ei), edge_fingerprint(ei[:, :-1]))
+    assert not np.array_equal(edge_fingerprint(ei, 300), edge_fingerprint(ei, 301))     # the key depends on N
+    swapped = np.ascontiguousarray(ei[::-1])                                # symmetric graph: the transpose is the same edge set
+    assert np.array_equal(edge_fingerprint(ei), edge_fingerprint(swapped))
+    directed = np.array([[0, 1, 2, 2], [1, 2, 0, 1]], np.int32)
+    assert not np.array_equal(edge_fingerprint(directed), edge_fingerprint(directed[::-1].copy()))
+
+    path = str(tmp_path / "cache")
+    first = cbm_matrix.from_cache(path, torch.from_numpy(ei), alpha=1, normalized=True)
+    assert first.builder is not None and first.build_seconds is not None           # built, file written
+    assert (tmp_path / "cache.npz").exists()
+    second = cbm_matrix.from_cache(path, torch.from_numpy(shuffled), alpha=1, normalized=True)
+    assert second.builder is None and second.build_seconds is None                  # loaded
+    for name in ("rowptr", "idx", "parent", "order", "level_off", "mst_row", "mst_col", "col_multiplier"):
+        assert torch.equal(getattr(first, name), getattr(second, name)), name
+    assert np.array_equal(second.edge_fingerprint, first.edge_fingerprint)
+    assert second.check_format(torch.from_numpy(ei))
+    # anything that changes the format rebuilds and overwrites the file
+    for kw in (dict(alpha=2, normalized=True), dict(alpha=1, normalized=False), dict(alpha=1, normalized=True, max_levels=2)):
+        again = cbm_matrix.from_cache(path, torch.from_numpy(ei), **kw)
+        assert again.builder is not None, kw
+        assert cbm_matrix.from_cache(path, torch.from_numpy(ei), **kw).builder is None, kw
+    other = cbm_matrix.from_cache(path, torch.from_numpy(moved), alpha=1, normalized=True, max_levels=2)
+    assert other.builder is not None and other.check_format(torch.from_numpy(moved))
+    # a file of an older version (no fingerprint) still loads, but never satisfies the cache
+    old = dict(np.load(str(tmp_path / "cache.npz")))
+    old.pop("edge_fingerprint"); old["meta"] = old["meta"].copy(); old["meta"][0] = 2
+    np.savez(str(tmp_path / "old.npz"), **old)
+    assert cbm_matrix.load(str(tmp_path / "old.npz")).edge_fingerprint is None
+    assert cbm_matrix.from_cache(str(tmp_path / "old"), torch.from_numpy(moved), alpha=1, normalized=True, max_levels=2).builder is not None
+    # a damaged file is rebuilt, not trusted
+    (tmp_path / "junk.npz").write_bytes(b"not a zip file")
+    assert cbm_matrix.from_cache(str(tmp_path / "junk"), torch.from_numpy(ei), alpha=0).builder is not None
+    assert cbm_matrix.from_cache(str(tmp_path / "junk"), torch.from_numpy(ei), alpha=0).builder is None

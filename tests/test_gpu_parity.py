@@ -976,18 +976,23 @@ def test_a_loaded_format_multiplies_like_the_built_one(tmp_path, symmetric):
     built.save(path)
     loaded = cbm_matrix.load(path)
     assert loaded.max_levels == 3
+    # the cache file keyed by the edge fingerprint: the same graph in another edge order is loaded, not rebuilt
+    perm = np.random.default_rng(1).permutation(ei.shape[1])
+    cached = cbm_matrix.from_cache(path, torch.from_numpy(np.ascontiguousarray(ei[:, perm])), alpha=1, normalized=True,
+                                   max_levels=3)
+    assert cached.builder is None and torch.equal(cached.idx, built.idx)
     say("loaded format", symmetric)
     x = torch.randn((n, d), generator=torch.Generator().manual_seed(31)).cuda()
     g = torch.randn((n, d), generator=torch.Generator().manual_seed(32)).cuda()
     out = []
-    for mat in (built, loaded):
+    for mat in (built, loaded, cached):
         y = torch.full_like(x, float("nan")); mat.omp_mkl_csr_fused_spmm_update(x, y)
         yp = torch.full_like(x, float("nan")); mat.omp_mkl_csr_spmm_update(x, yp)
         xg = x.clone().requires_grad_(True)
         (mat.matmul(xg) * g).sum().backward()
         out.append((y, yp, xg.grad))
-    for a, b in zip(*out):
-        assert torch.isfinite(a).all() and torch.equal(a, b)
+    for a, b, c in zip(*out):
+        assert torch.isfinite(a).all() and torch.equal(a, b) and torch.equal(a, c)
     if not symmetric:
         t_built, t_loaded = built.transposed(), loaded.transposed()
         assert t_loaded.max_levels == 3
