@@ -331,17 +331,14 @@ def gcn_epoch(args, torch, workload="c4"):
     nets = {k: make(k) for k in ("cbm_fused", "cbm_unfused", "csr")}
     # the dense GEMMs of all three models alike run on the library solution torch's TunableOp measures
     # fastest per shape (tuned during the warm-up epochs); --no-gemm-tuning leaves hipBLASLt's default pick
-    try:
-        tuning = contextlib.nullcontext() if args.no_gemm_tuning else tuned_gemms()
-        tuning.__enter__()
-    except Exception as exc:                               # a torch build without TunableOp: default picks
-        print(f"bench.py: GEMM tuning unavailable ({exc}); dense GEMMs on the default pick", file=sys.stderr)
-        tuning, args.no_gemm_tuning = contextlib.nullcontext(), True
-        tuning.__enter__()
-    try:
+    with contextlib.ExitStack() as stack:
+        if not args.no_gemm_tuning:
+            try:
+                stack.enter_context(tuned_gemms())
+            except Exception as exc:                       # a torch build without TunableOp: default picks
+                print(f"bench.py: GEMM tuning unavailable ({exc}); dense GEMMs on the default pick", file=sys.stderr)
+                args.no_gemm_tuning = True
         res = {k: run(v) for k, v in nets.items()}
-    finally:
-        tuning.__exit__(None, None, None)
     # aggregation alone: the 4 multiplies of an epoch (d = hidden and d = classes, forward and backward)
     agg = 0.0
     per_width = {}
