@@ -254,9 +254,12 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
         # first copies X slab-major, that copy is made once here and timed on its own
         zd = torch.empty_like(xd)
         scale = mat._device_arrays(xd.device)["m"] if w.normalized else None     # the step scales its copy by m
-        ws = relayout_slabs(xd, scale=scale) if (mat.relayout and _wants_workspace(xd, zd, nnz)) else None
+        ws = None
         relayout_ms = 0.0
-        if ws is not None:
+        if mat.relayout and _wants_workspace(xd, zd, nnz):
+            # room for the copy and, where the plan cuts rows into pieces, their sums behind it
+            ws = torch.empty(mat.workspace_floats(n, d, xd.device), dtype=torch.float32, device=xd.device)
+            relayout_slabs(xd, scale=scale, out=ws)
             _, relayout_ms, _ = time_gpu(lambda: relayout_slabs(xd, scale=scale, out=ws), args.steps, args.warmup, torch)
         spmm_only = lambda: mat._run_spmm(xd, zd, use_m=w.normalized, scale_roots=w.normalized, workspace=ws,
                                           workspace_ready=ws is not None,

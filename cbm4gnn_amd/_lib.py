@@ -76,6 +76,8 @@ HOST_SYMBOLS = {
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
     "cbm_schedule_split_count": (C.c_int64, [_P, _I32, _I32, C.POINTER(C.c_int32)]),
     "cbm_schedule_rows_split": (C.c_int, [_P, _P, _P, _I32, _I32, _P, _P]),
+    "cbm_schedule_blocks_count": (C.c_int64, [_P, _P, _I32, _I32, _I32, C.POINTER(C.c_int32)]),
+    "cbm_schedule_rows_blocks": (C.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _P]),
     "cbm_tile_rows": (C.c_int, [_P, _P, _I32, _I32, _I64, _I32, C.POINTER(CbmTiling)]),
     "cbm_tiling_free": (None, [C.POINTER(CbmTiling)]),
     "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),

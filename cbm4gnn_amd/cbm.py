@@ -456,6 +456,13 @@ class cbm_matrix:
         # wavefronts gather (``cbm_schedule_rows_split``); 0 = never cut.  A hub row of a power-law graph
         # would otherwise keep one wavefront per slab busy long after all others have finished.
         self.split_chunk = 2048
+        # Column blocks: every row is also cut where its columns pass from one B-th of X to the next and the
+        # pieces are scheduled block by block (``cbm_schedule_rows_blocks``), so that all wavefronts gather from
+        # the same part of X at about the same time.  "auto": 2 for matrices that are not tiled, have at least
+        # 100,000 rows and average at least 256 delta entries per row (long rows scattered over far more of X
+        # than the L2s hold: 5.9 -> 5.2 ms on the 132,534-node dense-community graph at d = 512; shorter rows
+        # lose more on the extra pieces than the L2 hits gain); an integer forces it (1 = off).
+        self.column_blocks = "auto"
         # Trees of 2 .. CBM_PATH_MAX_LEVELS levels are walked in ONE launch after the SpMM (every row sums down
         # its own ancestor path, ``cbm_spmm_update_paths_f32``) while the product is at most this many bytes:
         # there a launch per level costs more than the level's work.  0 = always walk level by level.
@@ -476,6 +483,10 @@ class cbm_matrix:
         if self.nnz == 0:
             return False
         cut = bool(self.split_chunk) and int((self.rowptr[1:] - self.rowptr[:-1]).max()) > int(self.split_chunk)
+        if self.column_blocks == "auto":
+            col_blocks = 2 if (n >= 100_000 and self.nnz >= 256 * n) else 1
+        else:
+            col_blocks = max(int(self.column_blocks), 1)
         tile = self.tiling != "off" and not (self.tiling == "auto" and (n < 16 * self.tile_rows or self.nnz < 32 * n))
         arrays = None
         if tile:                                            # "auto" on small matrices: tiles of 1024 rows cannot pay
@@ -505,13 +516,16 @@ class cbm_matrix:
                     }
             finally:
                 _lib.host_lib().cbm_tiling_free(C.byref(t))
-        if arrays is None and cut:                          # no local blocks: the whole matrix is "remote"
+        if arrays is not None:
+            col_blocks = 1                                  # the remote part of a tiled matrix has short rows
+        if arrays is None and (cut or col_blocks > 1):      # no local blocks: the whole matrix is "remote"
             arrays = {"n_panels": (n + 255) // 256, "n_blocks": 0, "tile_rows": self.tile_rows, "has_negative": 0,
                       "nnz_remote": self.nnz, "panel_ptr": torch.zeros((n + 255) // 256 + 1, dtype=torch.int32),
                       "rowptr_r": self.rowptr, "idx_r": self.idx}
         if arrays is not None:
-            arrays["cut"] = bool(self.split_chunk) and \
-                int((arrays["rowptr_r"][1:] - arrays["rowptr_r"][:-1]).max()) > int(self.split_chunk)
+            arrays["col_blocks"] = col_blocks
+            arrays["cut"] = col_blocks > 1 or (bool(self.split_chunk) and
+                                               int((arrays["rowptr_r"][1:] - arrays["rowptr_r"][:-1]).max()) > int(self.split_chunk))
             self._tiling_host = arrays
         return self._tiling_host
 
@@ -525,18 +539,19 @@ class cbm_matrix:
         th = self._host_tiling()
         return bool(th) and th["cut"]
 
-    def _split_schedule(self, rowptr, parent, m):
-        """(sched [count, 4], long_rows [n_long, 4], pieces) of ``cbm_schedule_rows_split``, CPU tensors."""
+    def _split_schedule(self, rowptr, idx, parent, m, col_blocks=1):
+        """(sched [count, 4], long_rows [n_long, 4], pieces) of ``cbm_schedule_rows_blocks``, CPU tensors."""
         n = rowptr.numel() - 1
         n_long = C.c_int32()
-        count = _lib.host_lib().cbm_schedule_split_count(_ptr(rowptr), n, int(self.split_chunk), C.byref(n_long))
+        chunk = int(self.split_chunk or 0)
+        count = _lib.host_lib().cbm_schedule_blocks_count(_ptr(rowptr), _ptr(idx), n, chunk, int(col_blocks), C.byref(n_long))
         if count < 0:
-            raise ValueError("cbm_schedule_split_count: bad row offsets or chunk size")
+            raise ValueError("cbm_schedule_blocks_count: bad row offsets, chunk size or block count")
         sched = torch.empty((count, 4), dtype=torch.int32)
         long_rows = torch.empty((max(n_long.value, 1), 4), dtype=torch.int32)
-        rc = _lib.host_lib().cbm_schedule_rows_split(_ptr(rowptr), _ptr(parent), _ptr(m), n, int(self.split_chunk), _ptr(sched),
-                                                     _ptr(long_rows))
-        _lib.check(rc, "cbm_schedule_rows_split")
+        rc = _lib.host_lib().cbm_schedule_rows_blocks(_ptr(rowptr), _ptr(idx), _ptr(parent), _ptr(m), n, chunk, int(col_blocks),
+                                                      _ptr(sched), _ptr(long_rows))
+        _lib.check(rc, "cbm_schedule_rows_blocks")
         long_rows = long_rows[:n_long.value]
         return sched, long_rows, int(long_rows[:, 2].sum()) if n_long.value else 0
 
@@ -665,7 +680,7 @@ class cbm_matrix:
                     if name == "scaled" and par is None:
                         continue
                     if th["cut"]:
-                        sched, long_rows, pieces = self._split_schedule(th["rowptr_r"], par, mm)
+                        sched, long_rows, pieces = self._split_schedule(th["rowptr_r"], th["idx_r"], par, mm, th["col_blocks"])
                         tensors["sched_" + name] = sched.to(device)
                         tensors["long_" + name] = long_rows.to(device)
                         tensors["n_long"], tensors["n_pieces"], tensors["n_sched"] = long_rows.size(0), pieces, sched.size(0)

@@ -587,6 +587,41 @@ struct cbm_builder {
     int32_t max_levels = 0;      // 0 = no limit
 };
 
+namespace {
+
+// Pieces of row r under a cut plan: the row's entries are cut where the column passes from one
+// column block to the next (col_blocks >= 2: blocks of ceil(n / col_blocks) consecutive columns; the
+// entries of a row are sorted by column, so a block's entries are contiguous), and a run longer than
+// `chunk` entries (chunk >= 64) is cut further into parts of `chunk`.  f(start, end, block) is called
+// for every non-empty piece in storage order; returns the number of pieces.
+template <class F>
+inline int32_t for_each_piece(const int32_t* rowptr, const uint32_t* idx, int32_t r, int32_t chunk, int32_t block_cols,
+                              F&& f) {
+    const int32_t b = rowptr[r], e = rowptr[r + 1];
+    int32_t pieces = 0, k = b;
+    while (k < e) {
+        int32_t run_end = e, block = 0;
+        if (block_cols > 0) {
+            block = (int32_t)((idx[k] & 0x7fffffffu) / (uint32_t)block_cols);
+            const uint32_t limit = (uint32_t)(block + 1) * (uint32_t)block_cols;       // first column of the next block
+            run_end = (int32_t)(std::lower_bound(idx + k, idx + e, limit,
+                                                 [](uint32_t v, uint32_t lim) { return (v & 0x7fffffffu) < lim; }) - idx);
+        }
+        for (int32_t q = k; q < run_end; q += (chunk > 0 ? chunk : run_end - k)) {
+            f(q, chunk > 0 ? std::min(q + chunk, run_end) : run_end, block);
+            pieces++;
+        }
+        k = run_end;
+    }
+    return pieces;
+}
+
+inline int32_t block_columns(int32_t n, int32_t col_blocks) {
+    return col_blocks >= 2 ? (int32_t)(((int64_t)n + col_blocks - 1) / col_blocks) : 0;
+}
+
+}  // namespace
+
 extern "C" {
 
 void cbm_build_host_timings(double* out4) {
@@ -631,50 +666,65 @@ int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float*
     }
 }
 
-int64_t cbm_schedule_split_count(const int32_t* rowptr, int32_t n, int32_t chunk, int32_t* n_long_out) {
-    if (!rowptr || n < 0 || chunk < 64) return -1;
+int64_t cbm_schedule_blocks_count(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t chunk, int32_t col_blocks,
+                                  int32_t* n_long_out) {
+    if (!rowptr || n < 0 || (chunk != 0 && chunk < 64) || col_blocks < 0 || (col_blocks >= 2 && !idx && n > 0 && rowptr[n] > 0))
+        return -1;
+    const int32_t bc = block_columns(n, col_blocks);
     int64_t count = 0;
     int32_t n_long = 0;
     for (int32_t r = 0; r < n; r++) {
-        const int64_t len = (int64_t)rowptr[r + 1] - rowptr[r];
-        if (len < 0) return -1;
-        if (len > chunk) { count += (len + chunk - 1) / chunk; n_long++; }
+        if (rowptr[r + 1] < rowptr[r]) return -1;
+        const int32_t pieces = for_each_piece(rowptr, idx, r, chunk, bc, [](int32_t, int32_t, int32_t) {});
+        if (pieces >= 2) { count += pieces; n_long++; }
         else count++;
     }
     if (n_long_out) *n_long_out = n_long;
     return count;
 }
 
-int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n, int32_t chunk,
-                            int32_t* sched_out, int32_t* long_rows_out) {
+int cbm_schedule_rows_blocks(const int32_t* rowptr, const uint32_t* idx, const int32_t* parent, const float* m, int32_t n,
+                             int32_t chunk, int32_t col_blocks, int32_t* sched_out, int32_t* long_rows_out) {
     if (!rowptr || !sched_out) return CBM_ERR_NULL;
     int32_t n_long = 0;
-    const int64_t count = cbm_schedule_split_count(rowptr, n, chunk, &n_long);
+    const int64_t count = cbm_schedule_blocks_count(rowptr, idx, n, chunk, col_blocks, &n_long);
     if (count < 0 || count > INT32_MAX) return CBM_ERR_SHAPE;
     if (n_long > 0 && !long_rows_out) return CBM_ERR_NULL;
+    const int32_t bc = block_columns(n, col_blocks);
     try {
-        // descriptors of rows and pieces, then the same stable counting sort by gather rounds as cbm_schedule_rows
-        struct Item { int32_t start, end, row; float scale; };
+        // descriptors of rows and pieces; then a stable counting sort by (column block, descending
+        // gather rounds): all wavefronts work on one column block at about the same time, longest first
+        struct Item { int32_t start, end, row, block; float scale; };
         std::vector<Item> items;
         items.reserve((size_t)count);
         int32_t slot = 0, at_long = 0;
+        std::vector<Item> mine;
         for (int32_t r = 0; r < n; r++) {
-            const int32_t b = rowptr[r], e = rowptr[r + 1];
             const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
-            if (e - b <= chunk) { items.push_back({b, e, r, scale}); continue; }
+            mine.clear();
+            for_each_piece(rowptr, idx, r, chunk, bc,
+                           [&](int32_t s, int32_t e, int32_t blk) { mine.push_back({s, e, 0, blk, 1.0f}); });
+            if (mine.size() <= 1) {                       // whole row (or an empty one): straight to Z, with its scale
+                if (mine.empty()) items.push_back({rowptr[r], rowptr[r + 1], r, 0, scale});
+                else items.push_back({mine[0].start, mine[0].end, r, mine[0].block, scale});
+                continue;
+            }
             int32_t* lr = long_rows_out + 4 * (size_t)at_long++;
-            lr[0] = r; lr[1] = slot;
-            for (int32_t k = b; k < e; k += chunk) items.push_back({k, std::min(k + chunk, e), (slot++) | CBM_SCHED_PIECE, 1.0f});
-            lr[2] = slot - lr[1];
+            lr[0] = r; lr[1] = slot; lr[2] = (int32_t)mine.size();
             std::memcpy(&lr[3], &scale, sizeof(float));
+            for (Item& it : mine) { it.row = (slot++) | CBM_SCHED_PIECE; items.push_back(it); }
         }
         int32_t max_rounds = 0;
         for (const Item& it : items) max_rounds = std::max(max_rounds, (it.end - it.start + 63) / 64);
-        std::vector<int64_t> first(max_rounds + 2, 0);
-        for (const Item& it : items) first[max_rounds - (it.end - it.start + 63) / 64 + 1]++;
-        for (int32_t b = 0; b <= max_rounds; b++) first[b + 1] += first[b];
+        const int64_t n_blocks = std::max(col_blocks, 1), buckets = n_blocks * (max_rounds + 1);
+        std::vector<int64_t> first((size_t)buckets + 1, 0);
+        auto bucket = [&](const Item& it) {
+            return (int64_t)it.block * (max_rounds + 1) + (max_rounds - (it.end - it.start + 63) / 64);
+        };
+        for (const Item& it : items) first[bucket(it) + 1]++;
+        for (int64_t b = 0; b < buckets; b++) first[b + 1] += first[b];
         for (const Item& it : items) {
-            int32_t* o = sched_out + 4 * first[max_rounds - (it.end - it.start + 63) / 64]++;
+            int32_t* o = sched_out + 4 * first[bucket(it)]++;
             o[0] = it.start; o[1] = it.end; o[2] = it.row;
             std::memcpy(&o[3], &it.scale, sizeof(float));
         }
@@ -682,6 +732,17 @@ int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const 
     } catch (const std::bad_alloc&) {
         return CBM_ERR_ALLOC;
     }
+}
+
+int64_t cbm_schedule_split_count(const int32_t* rowptr, int32_t n, int32_t chunk, int32_t* n_long_out) {
+    if (chunk < 64) return -1;
+    return cbm_schedule_blocks_count(rowptr, nullptr, n, chunk, 1, n_long_out);
+}
+
+int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n, int32_t chunk,
+                            int32_t* sched_out, int32_t* long_rows_out) {
+    if (chunk < 64) return CBM_ERR_SHAPE;
+    return cbm_schedule_rows_blocks(rowptr, nullptr, parent, m, n, chunk, 1, sched_out, long_rows_out);
 }
 
 void cbm_tiling_free(cbm_tiling* t) {

@@ -167,6 +167,21 @@ int64_t cbm_schedule_split_count(const int32_t* rowptr, int32_t n, int32_t chunk
 int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n, int32_t chunk,
                             int32_t* sched_out, int32_t* long_rows_out);
 
+/* cbm_schedule_rows_split that ALSO cuts every row where its (ascending) columns pass from one
+ * block of ceil(n / col_blocks) consecutive columns to the next (col_blocks >= 2; idx as in
+ * cbm_format), and orders the descriptors by column block first (then longest first): all
+ * wavefronts gather from the same col_blocks-th of X at about the same time, which keeps that part
+ * of the slab-major copy in the XCDs' L2s -- for matrices whose rows are long (hundreds of entries)
+ * and scattered over more of X than the L2s hold.  Runs longer than `chunk` are cut further
+ * (chunk = 0: never; else >= 64).  A row that ends up as one piece keeps an ordinary descriptor.
+ * col_blocks <= 1 is cbm_schedule_rows_split.  Same output formats; cbm_schedule_blocks_count
+ * returns the number of descriptors (and of cut rows), -1 on bad input.  HOST pointers.  No
+ * reference counterpart (MKL schedules rows internally). */
+int64_t cbm_schedule_blocks_count(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t chunk, int32_t col_blocks,
+                                  int32_t* n_long_out);
+int cbm_schedule_rows_blocks(const int32_t* rowptr, const uint32_t* idx, const int32_t* parent, const float* m, int32_t n,
+                             int32_t chunk, int32_t col_blocks, int32_t* sched_out, int32_t* long_rows_out);
+
 /* Split of a packed delta matrix (rowptr, idx as in cbm_format) into entries that cluster and the
  * rest, for cbm_spmm_tiled_f32.  Rows are cut into panels of CBM_TILING_PANEL_ROWS, columns into
  * tiles of tile_rows (1024); a (panel, tile) block that holds at least min_block_entries entries

@@ -107,37 +107,51 @@ def tiled_split(mat):
     return np.bincount(key)[key] >= mat.tile_min_block_entries, row
 
 
-def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8, tail=0):
-    """CSR product in ``groups`` interleaved partial sums per row, where a row with more than
-    ``chunk`` entries is cut into pieces of ``chunk`` entries: each piece is summed like a row of its
-    own and the piece sums are then added one after the other, starting from zero -- the order of
-    ``cbm_schedule_rows_split`` + ``combine_pieces``.  chunk = 0: nothing is cut."""
+def grouped_with_cuts(orc, rp, col, sgn, xs, chunk, groups=8, tail=0, col_blocks=1):
+    """CSR product in ``groups`` interleaved partial sums per row, where a row is cut into pieces --
+    where its columns pass from one block of ceil(n / col_blocks) columns to the next (col_blocks >= 2)
+    and, within such a run, every ``chunk`` entries (chunk = 0: never): each piece of a row with at
+    least two of them is summed like a row of its own and the piece sums are then added one after the
+    other, starting from zero -- the order of ``cbm_schedule_rows_blocks`` + ``combine_pieces``."""
     rp = np.asarray(rp, np.int64)
     n = rp.shape[0] - 1
+    block_cols = (n + col_blocks - 1) // col_blocks if col_blocks >= 2 else 0
     lens = np.diff(rp)
-    long_rows = np.nonzero(lens > chunk)[0] if chunk else np.empty(0, np.int64)
-    if long_rows.size == 0:
+    candidates = np.arange(n) if block_cols else (np.nonzero(lens > chunk)[0] if chunk else np.empty(0, np.int64))
+    starts, ends, owner, long_rows = [], [], [], []
+    for r in candidates:
+        pieces, k, e = [], int(rp[r]), int(rp[r + 1])
+        while k < e:
+            run_end = e
+            if block_cols:
+                run_end = k + int(np.searchsorted(col[k:e], (col[k] // block_cols + 1) * block_cols, side="left"))
+            step = chunk if chunk else run_end - k
+            pieces += [(q, min(q + step, run_end)) for q in range(k, run_end, step)]
+            k = run_end
+        if len(pieces) >= 2:
+            long_rows.append(r)
+            for a, b in pieces:
+                starts.append(a); ends.append(b); owner.append(r)
+    if not long_rows:
         return grouped_spmm(orc, rp.astype(np.int32), col, sgn, xs, groups, tail)
-    starts, ends, owner = [], [], []
-    for r in long_rows:
-        for k in range(rp[r], rp[r + 1], chunk):
-            starts.append(k); ends.append(min(k + chunk, rp[r + 1])); owner.append(r)
+    long_rows = np.array(long_rows)
+    is_long = np.zeros(n, bool); is_long[long_rows] = True
     # auxiliary matrix: the original rows (cut rows emptied) followed by one row per piece
-    keep = np.ones(col.shape[0], bool)
-    for r in long_rows:
-        keep[rp[r]:rp[r + 1]] = False
+    keep = ~np.repeat(is_long, lens)
     piece_idx = np.concatenate([np.arange(a, b) for a, b in zip(starts, ends)])
     aux_col = np.concatenate([col[keep], col[piece_idx]])
     aux_sgn = np.concatenate([sgn[keep], sgn[piece_idx]])
-    aux_len = np.concatenate([np.where(lens > chunk, 0, lens), np.array(ends) - np.array(starts)])
+    aux_len = np.concatenate([np.where(is_long, 0, lens), np.array(ends) - np.array(starts)])
     aux_rp = np.concatenate([[0], np.cumsum(aux_len)]).astype(np.int32)
     y = grouped_spmm(orc, aux_rp, aux_col.astype(np.int32), aux_sgn.astype(np.float32), xs, groups, tail)
     z = y[:n].copy()
-    for r in long_rows:
+    owner = np.array(owner)
+    first = np.concatenate([[0], np.flatnonzero(owner[1:] != owner[:-1]) + 1, [owner.shape[0]]])
+    for a, b in zip(first[:-1], first[1:]):                # pieces of a row are consecutive, in column order
         acc = np.zeros(xs.shape[1], np.float32)
-        for p in np.nonzero(np.array(owner) == r)[0]:
-            acc = acc + y[n + p]
-        z[r] = acc
+        for p in range(a, b):
+            acc = (acc + y[n + p]).astype(np.float32)
+        z[owner[a]] = acc
     return z
 
 
@@ -154,7 +168,7 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         # long rows cut into pieces; the plan-based multiply always gathers from the (scaled) copy
         xs = (orc.col_multiplier(ei, n)[:, None] * x).astype(np.float32) if normalized else x
         return grouped_with_cuts(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs,
-                                 mat.split_chunk, plan_groups, plan_tail)
+                                 int(mat.split_chunk or 0), plan_groups, plan_tail, mat._host_tiling()["col_blocks"])
     if mat.relayout and mat.is_tiled():
         # tiled multiply: (remote entries) + (local entries in storage order, one after the other), on the
         # copy of X scaled by m.  Remote entries: when no row is cut, the kernel of the local part gathers
@@ -1106,6 +1120,37 @@ def test_hub_row_is_cut_into_pieces(orc, normalized):
     whole.split_chunk = 0
     assert not whole.has_cut_rows()
     assert orc.max_rel_err(gpu_product(whole, x, normalized), got) <= 1e-5
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+def test_rows_cut_at_column_blocks(orc, normalized):
+    """``column_blocks = 3`` (with and without the chunk cut on top): every row is gathered in pieces, one
+    per third of X it touches, scheduled block by block; the piece sums are added in column order.  Bit for
+    bit against the oracle in that order, signed deltas and a deep tree included, both store paths, with
+    the ReLU, and the SpMM alone; the automatic choice leaves a matrix of this size alone."""
+    n = 3000
+    ei = graphs.add_self_loops(graphs.sbm(n, 30, 0.6, 0.05, seed=17), n)
+    auto = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized, tiling="off")
+    assert not auto.has_cut_rows() and auto._host_tiling() is False
+    for alpha, chunk in ((0, 2048), (10 ** 6, 64)):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=alpha, normalized=normalized, tiling="off")
+        mat.column_blocks, mat.split_chunk = 3, chunk
+        assert mat.has_cut_rows() and not mat.is_tiled() and mat._host_tiling()["col_blocks"] == 3
+        st = mat._device_arrays(torch.device("cuda", 0))["tiled"]
+        assert st["n_long"] > 0.9 * n and st["n_pieces"] >= 2 * st["n_long"]
+        for d in (41, 128):
+            say("column blocks", normalized, alpha, chunk, d)
+            x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+            got = gpu_product(mat, x, normalized)
+            want = oracle_product(orc, mat, ei, n, x, normalized)
+            assert np.array_equal(got, want)
+            assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CBM
+            assert orc.max_rel_err(got, gpu_product(auto, x, normalized)) <= 1e-5
+            xd = torch.from_numpy(x).cuda()
+            z = torch.full_like(xd, float("nan")); mat.omp_mkl_csr_spmm(xd, z)
+            assert np.array_equal(z.cpu().numpy(), oracle_delta_spmm(orc, mat, ei, n, x, normalized))
+            r_ = torch.full_like(xd, float("nan")); mat._run_spmm_update(xd, r_, use_m=normalized, relu=True)
+            assert np.array_equal(r_.cpu().numpy(), np.maximum(want, 0.0))
 
 
 def test_tiled_blocks_and_cut_rows_together(orc):

@@ -116,7 +116,7 @@ def test_split_schedule_covers_every_entry_once():
     m = torch.from_numpy(rng.random(n).astype(np.float32) + 0.5)
     mat = cbm_matrix.__new__(cbm_matrix)
     mat.split_chunk = 2048
-    sched, long_rows, pieces = mat._split_schedule(rowptr, parent, m)
+    sched, long_rows, pieces = mat._split_schedule(rowptr, None, parent, m)
     assert long_rows[:, 0].tolist() == [3, 77, 400] and long_rows[:, 2].tolist() == [5, 2, 2] and pieces == 9
     assert long_rows[:, 1].tolist() == [0, 5, 7]
     assert sched.shape[0] == n - 3 + 9
@@ -143,6 +143,65 @@ def test_split_schedule_covers_every_entry_once():
         assert np.array([w], np.int32).view(np.float32)[0] == (float(m[r]) if parent[r] < 0 else 1.0)
     # nothing to cut: the plain schedule
     mat.split_chunk = 1 << 20
-    s2, l2, p2 = mat._split_schedule(rowptr, parent, m)
+    s2, l2, p2 = mat._split_schedule(rowptr, None, parent, m)
     from cbm4gnn_amd.cbm import schedule_rows
     assert l2.shape[0] == 0 and p2 == 0 and torch.equal(s2, schedule_rows(rowptr, parent, m))
+
+
+def test_column_block_schedule():
+    """``cbm_schedule_rows_blocks``: every row is cut where its columns pass from one block of
+    ceil(n / B) columns to the next (and runs above the chunk size further), a row inside one block
+    keeps one descriptor, every entry is covered once, slots of a row are consecutive in column
+    order, and the descriptors are ordered by column block, longest first inside a block."""
+    rng = np.random.default_rng(1)
+    n, B, chunk = 1000, 4, 128
+    block_cols = (n + B - 1) // B
+    rows = []
+    for r in range(n):
+        k = int(rng.integers(0, 60))
+        if r == 10:
+            k = 900                                        # long row: cut by blocks and by chunk
+        lo, hi = (0, n) if r % 3 else (300, 340)            # every third row lives inside block 1
+        rows.append(np.sort(rng.choice(np.arange(lo, hi), size=min(k, hi - lo), replace=False)))
+    rowptr = torch.from_numpy(np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32))
+    col = np.concatenate(rows).astype(np.uint32)
+    idx = torch.from_numpy((col | (rng.random(col.shape[0]) < 0.3).astype(np.uint32) << 31).view(np.int32))
+    parent = torch.from_numpy(np.where(rng.random(n) < 0.5, -1, 0).astype(np.int32))
+    m = torch.from_numpy(rng.random(n).astype(np.float32) + 0.5)
+    mat = cbm_matrix.__new__(cbm_matrix)
+    mat.split_chunk = chunk
+    sched, long_rows, pieces = mat._split_schedule(rowptr, idx, parent, m, B)
+    PIECE = 0x40000000
+    owner_of = {}
+    for r, f, k, w in long_rows.tolist():
+        for q in range(k):
+            owner_of[f + q] = (r, q)
+        assert np.array([w], np.int32).view(np.float32)[0] == (float(m[r]) if parent[r] < 0 else 1.0)
+    assert sorted(owner_of) == list(range(pieces))
+    covered = np.zeros(col.shape[0], np.int32)
+    keys, starts_of = [], {}
+    for s0, s1, row, w in sched.tolist():
+        covered[s0:s1] += 1
+        blocks = set((col[s0:s1] // block_cols).tolist())
+        assert len(blocks) <= 1 and s1 - s0 <= chunk
+        blk = blocks.pop() if blocks else 0
+        keys.append((blk, -((s1 - s0 + 63) // 64)))
+        if row & PIECE:
+            r, q = owner_of[row & ~PIECE]
+            starts_of.setdefault(r, []).append((q, s0, s1))
+            assert np.array([w], np.int32).view(np.float32)[0] == 1.0
+        else:
+            assert s0 == rowptr[row] and s1 == rowptr[row + 1]
+            assert np.array([w], np.int32).view(np.float32)[0] == (float(m[row]) if parent[row] < 0 else 1.0)
+    assert (covered == 1).all() and keys == sorted(keys)
+    for r, lst in starts_of.items():                       # the pieces of a row tile it in slot order
+        lst.sort()
+        assert lst[0][1] == rowptr[r] and lst[-1][2] == rowptr[r + 1] and len(lst) >= 2
+        assert all(a[2] == b[1] for a, b in zip(lst, lst[1:]))
+    assert 10 in starts_of and len(starts_of[10]) == sum(-(-int(((rows[10] // block_cols) == b).sum()) // chunk) for b in range(B))
+    assert not any(r % 3 == 0 and r != 10 for r in starts_of)      # rows inside one block are not cut
+    # one block, no chunk: the plain schedule
+    mat.split_chunk = 0
+    s1_, l1_, p1_ = mat._split_schedule(rowptr, idx, parent, m, 1)
+    from cbm4gnn_amd.cbm import schedule_rows
+    assert p1_ == 0 and torch.equal(s1_, schedule_rows(rowptr, parent, m))
