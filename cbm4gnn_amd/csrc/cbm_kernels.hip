@@ -934,19 +934,33 @@ __global__ __launch_bounds__(256) void relu_rows(float* __restrict__ Y, int64_t 
 
 // Rows that the schedule cut into pieces: Z[row] = (piece sums added in order, from 0) * scale,
 // then the ReLU if asked.  long_rows = { row, first slot, pieces, bits(scale) } per cut row; a slot
-// holds slot_floats floats, Z and d are those of the column range the slots cover.  blockIdx.x =
-// cut row, threads along the columns.
-__global__ __launch_bounds__(256) void combine_pieces(const int4* __restrict__ long_rows, const float* __restrict__ partials,
-                                                      float* __restrict__ Z, int d, int64_t slot_floats, int64_t ldz,
-                                                      int apply_scale, int relu) {
-    const int4 lr = long_rows[blockIdx.x];
+// holds slot_floats floats, Z and d are those of the column range the slots cover.  One wavefront
+// per cut row, lanes along the columns (VEC floats each).
+template <int VEC>
+__global__ __launch_bounds__(kWave * kWavesPerBlock) void combine_pieces(
+    const int4* __restrict__ long_rows, const float* __restrict__ partials, float* __restrict__ Z, int n_long, int d,
+    int64_t slot_floats, int64_t ldz, int apply_scale, int relu) {
+    const int r = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (r >= n_long) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int4 lr = long_rows[r];
     const float scale = apply_scale ? __int_as_float(lr.w) : 1.0f;
-    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < d; j += gridDim.y * blockDim.x) {
-        float acc = 0.0f;
-        for (int k = 0; k < lr.z; k++) acc += partials[(int64_t)(lr.y + k) * slot_floats + j];
-        acc *= scale;
-        if (relu) acc = acc < 0.0f ? 0.0f : acc;
-        Z[(int64_t)lr.x * ldz + j] = acc;
+    for (int j = lane * VEC; j < d; j += kWave * VEC) {
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = 0.0f;
+        for (int k = 0; k < lr.z; k++) {
+            float v[VEC];
+            load_vec<VEC>(partials + (int64_t)(lr.y + k) * slot_floats + j, v);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc[e] += v[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            acc[e] *= scale;
+            if (relu) acc[e] = acc[e] < 0.0f ? 0.0f : acc[e];
+        }
+        store_vec<VEC>(Z + (int64_t)lr.x * ldz + j, acc);
     }
 }
 
@@ -1802,13 +1816,19 @@ int cbm_spmm_tiled_f32(const cbm_tiling_dev* t, const float* m, const float* X, 
     if (t->n_long > 0) {                                  // pieces of cut rows -> their rows of Z, per column range
         const int4* lr = reinterpret_cast<const int4*>(t->long_rows);
         const int scale_here = has_local ? 0 : 1, relu_here = (relu && !has_local) ? 1 : 0;
-        if (n_full > 0)
-            hipLaunchKernelGGL(combine_pieces, dim3((unsigned)t->n_long, (unsigned)std::min(8, (d_full + 255) / 256)), dim3(256),
-                               0, s, lr, partials, Z, d_full, (int64_t)n_full * 32, ldz, scale_here, relu_here);
+        const dim3 cgrid((unsigned)((t->n_long + kWavesPerBlock - 1) / kWavesPerBlock)), cblock(kWave * kWavesPerBlock);
+        if (n_full > 0) {
+            // slots are whole slabs (a multiple of 32 floats, 16-byte aligned): float4 where Z allows it
+            if (d_full % 4 == 0 && ldz % 4 == 0 && aligned(Z, 16))
+                hipLaunchKernelGGL(combine_pieces<4>, cgrid, cblock, 0, s, lr, partials, Z, t->n_long, d_full,
+                                   (int64_t)n_full * 32, ldz, scale_here, relu_here);
+            else
+                hipLaunchKernelGGL(combine_pieces<1>, cgrid, cblock, 0, s, lr, partials, Z, t->n_long, d_full,
+                                   (int64_t)n_full * 32, ldz, scale_here, relu_here);
+        }
         if (lay.tail)
-            hipLaunchKernelGGL(combine_pieces, dim3((unsigned)t->n_long, 1u), dim3(256), 0, s, lr,
-                               partials + (int64_t)t->n_pieces * n_full * 32, Z + n_full * 32, d_tail, (int64_t)lay.tail, ldz,
-                               scale_here, relu_here);
+            hipLaunchKernelGGL(combine_pieces<1>, cgrid, cblock, 0, s, lr, partials + (int64_t)t->n_pieces * n_full * 32,
+                               Z + n_full * 32, t->n_long, d_tail, (int64_t)lay.tail, ldz, scale_here, relu_here);
     }
     if (!has_local) return check_launch();
     // local entries: tiles of the copy staged in LDS; adds to Z, then scale and ReLU
