@@ -50,13 +50,23 @@ def _ptr(t):
 
 
 def _stream(device):
-    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """The current stream of ``device`` as a raw handle (what torch's own launches use; a small graph's
+    multiply is bound by the host cost of issuing it, and ``torch.cuda.current_stream`` alone is 4 us)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+
+
+_gpu_seen = False
 
 
 def _require_gpu():
+    global _gpu_seen
+    if _gpu_seen:
+        return
     if not torch.cuda.is_available():
         raise RuntimeError("cbm_matrix multiplies run on the GPU only and no HIP device is available "
                            "(there is no CPU fallback)")
+    _gpu_seen = True
 
 
 def _check_f32_matrix(t, name, n=None):
