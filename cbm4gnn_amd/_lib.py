@@ -105,6 +105,7 @@ HIP_SYMBOLS = {
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_paths_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
+    "cbm_spmm_update_single_f32": (C.c_int, [_P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_paths_scratch_floats": (C.c_int64, [_I32, _I32, _I32]),
     "cbm_spmm_update_static_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_tiled_workspace_floats": (C.c_int64, [C.POINTER(CbmTilingDev), _I32, _I32]),

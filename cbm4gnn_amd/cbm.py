@@ -477,6 +477,30 @@ class cbm_matrix:
         # its own ancestor path, ``cbm_spmm_update_paths_f32``) while the product is at most this many bytes:
         # there a launch per level costs more than the level's work.  0 = always walk level by level.
         self.path_walk_max_bytes = 64 << 20
+        # Products of at most this many bytes on shallow, sparse trees run as one launch (see _single_launch);
+        # 0 = never.
+        self.single_launch_max_bytes = 4 << 20
+
+    def _path_gather_ratio(self):
+        """(sum over rows of the delta entries on the row's ancestor path, itself included) / nnz: the extra
+        gather work of computing every row's ancestors anew (1.0 = flat tree).  Computed once."""
+        if getattr(self, "_path_ratio", None) is None:
+            lens = (self.rowptr[1:] - self.rowptr[:-1]).to(torch.int64)
+            cost = lens.clone()
+            order, lo, parent = self.order.long(), self.level_off.tolist(), self.parent.long()
+            for l in range(1, self.n_levels):                       # a level's parents are final before it
+                rows = order[lo[l]:lo[l + 1]]
+                cost[rows] = lens[rows] + cost[parent[rows]]
+            self._path_ratio = float(cost.sum()) / max(self.nnz, 1)
+        return self._path_ratio
+
+    def _single_launch(self, n, d):
+        """Whether ``*_spmm_update`` runs as ONE launch (``cbm_spmm_update_single_f32``: every row gathers its
+        own delta entries and those of its ancestors): small products, where a launch costs more than the
+        extra gathers -- at most ``single_launch_max_bytes`` of output, a tree of 2 .. 16 levels and at
+        most 1.5 x the gather work."""
+        return (1 < self.n_levels <= _lib.CBM_PATH_MAX_LEVELS and 0 < 4 * n * d <= int(self.single_launch_max_bytes)
+                and self._path_gather_ratio() <= 1.5)
 
     def _walks_paths(self, n, d):
         return (1 < self.n_levels <= _lib.CBM_PATH_MAX_LEVELS and 0 < 4 * n * d <= int(self.path_walk_max_bytes))
@@ -853,6 +877,16 @@ class cbm_matrix:
             raise ValueError("dst must not alias rhs")
         st = self._device_arrays(xd.device)
         tiled = st["tiled"] is not None and self.relayout and not (workspace_ready and use_m and not workspace_prescaled)
+        if not tiled and workspace is None and not workspace_ready and self._single_launch(n, x.size(1)):
+            with torch.cuda.device(xd.device):
+                rc = _lib.hip_lib().cbm_spmm_update_single_f32(
+                    _ptr(st["rowptr"]), _ptr(st["idx"]), _ptr(st["m"]) if use_m else None, None, _ptr(st["parent"]),
+                    self.n_levels, _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd),
+                    _lib.CBM_UPDATE_RELU if relu else 0, _stream(xd.device))
+            _lib.check(rc, "cbm_spmm_update_single_f32")
+            if yd is not y:
+                y.copy_(yd)
+            return
         if tiled:
             ws = self._tiled_workspace(xd, workspace)
         else:

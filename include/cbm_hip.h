@@ -364,6 +364,19 @@ int cbm_spmm_update_paths_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev
                               float* workspace_dev, float* z_scratch_dev, int32_t n, int32_t d, int64_t ldx,
                               int64_t ldy, int32_t flags, void* stream);
 
+/* Y = A_hat * X in ONE launch, for small matrices whose tree is shallow (n_levels <= CBM_PATH_MAX_LEVELS)
+ * and sparse (replaces the same reference functions as cbm_spmm_update_f32): the wavefront of row v
+ * computes the delta-row sums of v and of all its ancestors and combines them top-down.  Entries are
+ * accumulated strictly in order (as one wavefront per row does, cbm_spmm_summation_groups = 1) with
+ * the coefficient +-1 (m == NULL), +-m[col] gathered, or coef[k] streamed; the tree steps use the
+ * arithmetic of cbm_propagate_f32: Y is bit for bit what cbm_set_spmm_kernel(1) + cbm_spmm_update_f32
+ * return.  Work grows to the sum over rows of the delta entries on their ancestor paths, so this pays
+ * only where a launch costs more than those gathers (a few thousand rows, few rows with parents); the
+ * caller decides.  No workspace, no scratch.  flags: CBM_UPDATE_RELU. */
+int cbm_spmm_update_single_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, const float* m_dev, const float* coef_dev,
+                               const int32_t* parent_dev, int32_t n_levels, const float* X_dev, float* Y_dev, int32_t n,
+                               int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream);
+
 /* Floats of z_scratch that cbm_spmm_update_paths_f32 uses: n * ((d + 3) & ~3) for 2 <= n_levels <=
  * CBM_PATH_MAX_LEVELS, else 0 (the call then falls back to cbm_spmm_update_f32). */
 int64_t cbm_spmm_update_paths_scratch_floats(int32_t n, int32_t d, int32_t n_levels);

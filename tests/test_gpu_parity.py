@@ -59,13 +59,19 @@ def brings_workspace(relayout, nnz, n, d, ld=None):
     return bool(relayout) and n > 0 and (nnz >= 24 * n or groups_for(d, ld) == 1)
 
 
-def mat_groups(mat, d, ld=None):
-    """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough."""
+def mat_groups(mat, d, ld=None, update=False):
+    """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough.
+    ``update``: the whole product (``*_spmm_update``), which for small products on shallow, sparse trees is
+    one launch that sums every row strictly in order."""
     n = mat.num_rows
+    if update and not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(n, d):
+        return 1
     return groups_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, n, d, ld))
 
 
-def mat_tail(mat, d, ld=None):
+def mat_tail(mat, d, ld=None, update=False):
+    if update and not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(mat.num_rows, d):
+        return 0
     return tail_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, mat.num_rows, d, ld))
 
 
@@ -80,10 +86,11 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
         z = oracle_delta_spmm(orc, mat, ei, n, x, normalized)
         return (orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads) if normalized
                 else orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads))
-    g = mat_groups(mat, x.shape[1]) if groups is None else groups
-    tail = mat_tail(mat, x.shape[1]) if groups is None else 0
+    g = mat_groups(mat, x.shape[1], update=True) if groups is None else groups
+    tail = mat_tail(mat, x.shape[1], update=True) if groups is None else 0
     if prescaled is None:                                  # the copy is only made for the slab kernel (g > 1)
-        prescaled = normalized and brings_workspace(mat.relayout, mat.nnz, n, x.shape[1]) and mat_groups(mat, x.shape[1]) > 1
+        prescaled = (normalized and brings_workspace(mat.relayout, mat.nnz, n, x.shape[1])
+                     and mat_groups(mat, x.shape[1], update=True) > 1)
     if prescaled:
         xs = (m[:, None] * x).astype(np.float32)
         z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs, g, tail,
@@ -337,6 +344,7 @@ def test_update_only_entry_points(orc):
     for normalized in (False, True):
         say("update-only", normalized)
         mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+        mat.single_launch_max_bytes = 0                    # the product below is compared with SpMM + walk, step by step
         # spmm alone == Delta (diag m) X
         z = torch.empty((n, d), device="cuda")
         mat.omp_mkl_csr_spmm(torch.from_numpy(x).cuda(), z)
@@ -680,6 +688,61 @@ def test_path_walk_equals_the_level_by_level_walk(orc):
     assert torch.equal(y, want)
 
 
+def test_one_launch_product_for_small_shallow_trees(orc):
+    """``cbm_spmm_update_single_f32``: small products on shallow, sparse trees run as ONE launch in which
+    every row gathers its own delta entries and those of its ancestors.  Bit for bit what one wavefront per
+    row + the level-by-level walk return (entries in order, the reference's fma(+-m[c], x, acc)), with the
+    ReLU, widths with a scalar tail, a strided destination; the policy leaves large products, deep or
+    dense trees and flat trees alone; the C ABI refuses what it cannot do."""
+    from cbm4gnn_amd.cbm import _ptr
+    lib = _lib.hip_lib()
+    n = 1200
+    ei = graphs.add_self_loops(graphs.sbm(n, 40, 0.2, 0.002, seed=3), n)        # few rows find a parent
+    for normalized in (False, True):
+        mat = cbm_matrix(torch.from_numpy(ei), None, alpha=2, normalized=normalized)
+        say("one launch", normalized, "levels", mat.n_levels, "path ratio", round(mat._path_gather_ratio(), 3))
+        assert 2 <= mat.n_levels <= _lib.CBM_PATH_MAX_LEVELS and 1.0 < mat._path_gather_ratio() <= 1.5
+        for d in (10, 41, 64, 200):
+            assert mat._single_launch(n, d) and mat_groups(mat, d, update=True) == 1
+            x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+            got = gpu_product(mat, x, normalized)
+            assert np.array_equal(got, oracle_product(orc, mat, ei, n, x, normalized))
+            assert np.array_equal(got, oracle_product(orc, mat, ei, n, x, normalized, groups=1, prescaled=False))
+            assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CBM
+            xd = torch.from_numpy(x).cuda()
+            # the same through one wavefront per row + the level walk
+            mat.single_launch_max_bytes = 0
+            assert lib.cbm_set_spmm_kernel(1) == 0
+            try:
+                two = torch.empty_like(xd); mat._run_spmm_update(xd, two, use_m=normalized)
+            finally:
+                assert lib.cbm_set_spmm_kernel(0) == 0
+                mat.single_launch_max_bytes = 4 << 20
+            assert np.array_equal(two.cpu().numpy(), got)
+            r = torch.full((n, d + 8), float("nan"), device="cuda")[:, :d]
+            mat._run_spmm_update(xd, r, use_m=normalized, relu=True)
+            assert np.array_equal(r.cpu().numpy(), np.maximum(got, 0.0))
+        assert not mat._single_launch(n, 1024)              # 4.9 MB of output: the launches are no longer what costs
+    flat = cbm_matrix(torch.from_numpy(ei), None, alpha=10 ** 6)
+    assert flat.n_levels == 1 and not flat._single_launch(n, 64)
+    dense_tree = cbm_matrix(torch.from_numpy(graphs.add_self_loops(graphs.sbm(n, 6, 0.6, 0.01, seed=21), n)), None, alpha=0,
+                            max_levels=8)
+    assert dense_tree._path_gather_ratio() > 1.5 and not dense_tree._single_launch(n, 64)
+    # C ABI
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=2)
+    st = mat._device_arrays(torch.device("cuda", 0))
+    x = torch.randn((n, 64), device="cuda"); y = torch.full_like(x, 3.0)
+    call = lambda xx, yy, levels=mat.n_levels, flags=0: lib.cbm_spmm_update_single_f32(
+        _ptr(st["rowptr"]), _ptr(st["idx"]), None, None, _ptr(st["parent"]), levels, _ptr(xx), _ptr(yy), n, 64, 64, 64, flags, None)
+    assert call(x, x) == _lib.CBM_ERR_SHAPE and call(x, y, levels=_lib.CBM_PATH_MAX_LEVELS + 1) == 6 and call(x, y, flags=64) == 6
+    assert call(None, y) == _lib.CBM_ERR_NULL
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+    assert call(x, y) == 0
+    want = torch.empty_like(x); mat._run_spmm_update(x, want, use_m=False)
+    assert torch.equal(y, want)
+
+
 def test_degenerate_shapes(orc):
     # empty rows, a single-row matrix, d = 1, more slabs than rows
     ei = np.array([[0, 1, 2, 4, 2], [0, 2, 1, 2, 4]], np.int32)      # row 3 is empty
@@ -857,6 +920,7 @@ def test_alias_free_row_stride_needs_no_copy(orc):
     n, d = 700, 256
     ei = graphs.add_self_loops(graphs.sbm(n, 7, 0.3, 0.01, seed=9), n)
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+    mat.single_launch_max_bytes = 0                        # this test is about the slab kernel's gather, not the one-launch product
     assert mat.nnz >= 24 * n
     x = torch.randn((n, d), generator=torch.Generator().manual_seed(9)).cuda()
     xp = torch.zeros((n, d + 32), device="cuda")[:, :d]
@@ -962,6 +1026,7 @@ def test_changing_a_cached_setting_takes_effect():
     n, d = 500, 64
     ei = graphs.add_self_loops(graphs.sbm(n, 5, 0.3, 0.01, seed=8), n)
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=1, normalized=True)
+    mat.single_launch_max_bytes = 0                        # the one-launch product gathers m[col] and never expands coef
     x = torch.randn((n, d), generator=torch.Generator().manual_seed(8)).cuda()
     say("cached settings")
     mat.relayout = False                                    # gather in place: the entries' coefficients are used

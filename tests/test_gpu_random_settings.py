@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 def test_random_settings_against_oracle(orc, seed):
     """40 cases per seed: SBM / Erdos-Renyi / hub-row graphs of 7 .. 3,000 nodes, plain and normalised,
     alpha 0 .. huge, widths 1 .. 258, with and without the LDS tiling, the depth limit, rows cut by
-    length and at column-block boundaries, the one-launch path walk on and off."""
+    length and at column-block boundaries, the one-launch path walk and the one-launch product on and off."""
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     rng = np.random.default_rng(seed)
@@ -40,9 +40,11 @@ def test_random_settings_against_oracle(orc, seed):
         mat.split_chunk = int(rng.choice([0, 64, 2048]))
         mat.column_blocks = int(rng.choice([1, 1, 2, 3]))
         mat.path_walk_max_bytes = int(rng.choice([0, 64 << 20]))
+        mat.single_launch_max_bytes = int(rng.choice([0, 4 << 20]))
         x = rng.standard_normal((n, d)).astype(np.float32)
         parity.say("random settings", seed, case, kind, n, mat.nnz, mat.n_levels, normalized, alpha, d, tiling, mat.is_tiled(),
-                   mat.has_cut_rows(), mat.split_chunk, mat.column_blocks, max_levels, mat.path_walk_max_bytes)
+                   mat.has_cut_rows(), mat.split_chunk, mat.column_blocks, max_levels, mat.path_walk_max_bytes,
+                   mat.single_launch_max_bytes)
         got = parity.gpu_product(mat, x, normalized)
         assert np.array_equal(got, parity.oracle_product(orc, mat, ei, n, x, normalized)), (seed, case)
         assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= parity.TOL_CBM, (seed, case)
