@@ -130,7 +130,7 @@ def cpu_rows_fp64(rp, col, val, x, rows):
     return sub @ x.astype(np.float64)
 
 
-def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
+def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50, threads=0):
     """Reference-style CPU CBM and CPU CSR multiplies on this host (MKL SpMM + OpenMP walk), with
     all threads and with one thread."""
     import numpy as np
@@ -139,6 +139,9 @@ def cpu_baseline(w, mat, x, budget_s=20.0, max_iters=50):
 
     n, d = x.shape
     all_threads = orc.max_threads()
+    if threads > 0:                                           # --threads: the reference's num_threads knob
+        all_threads = min(int(threads), all_threads)
+        torch.set_num_threads(all_threads)
     ei = w.edge_index
     m = orc.col_multiplier(ei, n) if w.normalized else None
     col, sign = mat.columns()
@@ -449,6 +452,9 @@ def main():
     ap.add_argument("--d", type=int, default=None)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--threads", type=int, default=0,
+                    help="threads of the multi-threaded cpu_baseline leg (default: all host cores; the reference's "
+                         "benchmarks fix 16, benchmark/parallel/benchmark_spmm_cpu.py:2)")
     ap.add_argument("--only-multiply", action="store_true",
                     help="skip the gcn_epoch and other_workloads sections of the default run")
     ap.add_argument("--max-levels", type=int, default=None,
@@ -548,7 +554,7 @@ def main():
         "host_s": {"generate": t_gen, "build_format": ex["t_build"], "builder": mat.builder, "build_phases": mat.build_seconds},
     }
     if not args.no_cpu:
-        cpu, y_cpu = cpu_baseline(w, mat, ex["x"].numpy())
+        cpu, y_cpu = cpu_baseline(w, mat, ex["x"].numpy(), threads=args.threads)
         out["cpu_baseline"] = {
             "value": cpu["cbm_ms_mean"], "unit": "ms", "cores": cpu["threads"], "kind": "port",
             "sample": f"{cpu['iters'][0]} full multiplies of the same workload after 1 warm-up ({cpu['spmm']} + OpenMP tree walk); "
