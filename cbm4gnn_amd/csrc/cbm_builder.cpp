@@ -593,19 +593,21 @@ namespace {
 // column block to the next (col_blocks >= 2: blocks of ceil(n / col_blocks) consecutive columns; the
 // entries of a row are sorted by column, so a block's entries are contiguous), and a run longer than
 // `chunk` entries (chunk >= 64) is cut further into parts of `chunk`.  f(start, end, block) is called
-// for every non-empty piece in storage order; returns the number of pieces.
+// for every non-empty piece in storage order; returns the number of pieces.  Columns beyond the last
+// block (an index out of range) count as the last block.
 template <class F>
 inline int32_t for_each_piece(const int32_t* rowptr, const uint32_t* idx, int32_t r, int32_t chunk, int32_t block_cols,
-                              F&& f) {
+                              int32_t max_block, F&& f) {
     const int32_t b = rowptr[r], e = rowptr[r + 1];
     int32_t pieces = 0, k = b;
     while (k < e) {
         int32_t run_end = e, block = 0;
         if (block_cols > 0) {
-            block = (int32_t)((idx[k] & 0x7fffffffu) / (uint32_t)block_cols);
+            block = (int32_t)std::min<uint32_t>((idx[k] & 0x7fffffffu) / (uint32_t)block_cols, (uint32_t)max_block);
             const uint32_t limit = (uint32_t)(block + 1) * (uint32_t)block_cols;       // first column of the next block
             run_end = (int32_t)(std::lower_bound(idx + k, idx + e, limit,
                                                  [](uint32_t v, uint32_t lim) { return (v & 0x7fffffffu) < lim; }) - idx);
+            if (run_end <= k) run_end = e;                 // unsorted columns: never stall, keep the rest together
         }
         for (int32_t q = k; q < run_end; q += (chunk > 0 ? chunk : run_end - k)) {
             f(q, chunk > 0 ? std::min(q + chunk, run_end) : run_end, block);
@@ -675,7 +677,7 @@ int64_t cbm_schedule_blocks_count(const int32_t* rowptr, const uint32_t* idx, in
     int32_t n_long = 0;
     for (int32_t r = 0; r < n; r++) {
         if (rowptr[r + 1] < rowptr[r]) return -1;
-        const int32_t pieces = for_each_piece(rowptr, idx, r, chunk, bc, [](int32_t, int32_t, int32_t) {});
+        const int32_t pieces = for_each_piece(rowptr, idx, r, chunk, bc, std::max(col_blocks, 1) - 1, [](int32_t, int32_t, int32_t) {});
         if (pieces >= 2) { count += pieces; n_long++; }
         else count++;
     }
@@ -702,7 +704,7 @@ int cbm_schedule_rows_blocks(const int32_t* rowptr, const uint32_t* idx, const i
         for (int32_t r = 0; r < n; r++) {
             const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
             mine.clear();
-            for_each_piece(rowptr, idx, r, chunk, bc,
+            for_each_piece(rowptr, idx, r, chunk, bc, std::max(col_blocks, 1) - 1,
                            [&](int32_t s, int32_t e, int32_t blk) { mine.push_back({s, e, 0, blk, 1.0f}); });
             if (mine.size() <= 1) {                       // whole row (or an empty one): straight to Z, with its scale
                 if (mine.empty()) items.push_back({rowptr[r], rowptr[r + 1], r, 0, scale});
