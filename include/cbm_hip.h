@@ -227,9 +227,9 @@ const char* cbm_status_string(int status);
 int cbm_set_spmm_kernel(int kind);
 
 /* Resident wavefronts per SIMD of the slab SpMM kernel for later calls of this process: 0 =
- * automatic (default: 4 when rows average 128 entries or more, 6 from 32, else all the registers
- * allow), 1..8 = fixed.  A tuning
- * hook; no reference counterpart. */
+ * automatic (default: 4 when rows average 128 entries or more and a 128-byte slab of X exceeds an
+ * XCD's L2, 6 when it does not or rows average 32 or more, else all the registers allow), 1..8 =
+ * fixed.  A tuning hook; no reference counterpart. */
 int cbm_set_spmm_occupancy(int waves_per_simd);
 
 /* Tiled multiply (cbm_spmm_tiled_f32) for later calls of this process: 1 (default) = when the plan
