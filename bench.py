@@ -105,6 +105,21 @@ def time_gpu(fn, steps, warmup, torch):
     return wall_ms, span_ms, statistics.median(per_call)
 
 
+def time_gpu_back_to_back(fn, steps, torch):
+    """ms per call of ``steps`` calls issued back to back between ONE pair of events: what a caller's
+    loop sees.  The per-call events of ``time_gpu`` put two event records around every call, which
+    costs about as much as a whole multiply on the smallest workloads."""
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
 def csr_of(edge_index, n, m=None):
     """(rowptr int32, col int32, val fp32 or None, order) of the CSR of a COO list, NumPy."""
     import numpy as np
@@ -230,7 +245,11 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
     val_d = None if val is None else torch.from_numpy(val).cuda()
     ycsr = torch.empty_like(xd)
     csr_sched = schedule_rows(torch.from_numpy(rp)).to(xd.device)
-    _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp_d, col_d, val_d, xd, ycsr, csr_sched), args.steps, args.warmup, torch)
+    csr_step = lambda: csr_spmm(rp_d, col_d, val_d, xd, ycsr, csr_sched)
+    _, csr_ms, _ = time_gpu(csr_step, args.steps, args.warmup, torch)
+    # the same two calls without events between them (more of them where a call is short)
+    reps = args.steps * (10 if span_ms < 0.2 else 1)
+    loop_ms, csr_loop_ms = time_gpu_back_to_back(step, reps, torch), time_gpu_back_to_back(csr_step, reps, torch)
     step()
     torch.cuda.synchronize()
     err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
@@ -245,6 +264,8 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
         "workload": w.name, "alpha": alpha, "d": d, "nodes": n, "nnz_A": n_edges, "nnz_delta": nnz,
         "compression_ratio": mat.compression_ratio(), "tree_levels": mat.n_levels, "tree_edges": tree_edges,
         "cbm_ms": span_ms, "cbm_ms_median": med_ms, "gpu_csr_ms": csr_ms, "speedup_vs_gpu_csr": csr_ms / span_ms,
+        "cbm_ms_back_to_back": loop_ms, "gpu_csr_ms_back_to_back": csr_loop_ms,
+        "speedup_vs_gpu_csr_back_to_back": csr_loop_ms / loop_ms, "back_to_back_calls": reps,
         "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
         "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
         "max_rel_err_vs_gpu_csr": err_vs_csr, "max_rel_err_vs_cpu_fp64_rows": err_vs_cpu_rows,
@@ -528,6 +549,8 @@ def main():
                    "alpha": alpha, "normalized": bool(w.normalized), "tree_levels": mat.n_levels,
                    "tree_edges": ex["tree_edges"], "scale": args.scale},
         "ms_per_step_wall": ex["wall_ms"], "ms_per_step_median": ex["med_ms"],
+        "ms_per_step_back_to_back": row["cbm_ms_back_to_back"],
+        "gpu_csr_ms_back_to_back": row["gpu_csr_ms_back_to_back"],
         "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
         "cbm_frac_of_8TBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
