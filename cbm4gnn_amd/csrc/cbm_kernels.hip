@@ -493,7 +493,8 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 //   * A lane group reads its row's entries as one 16-byte vector per 8 entries; every (row, block)
 //     segment is padded to a multiple of 8 entries with the index of an all-zero row kept behind
 //     the tile in LDS, and a group whose segment is shorter than its neighbours' gathers that row:
-//     no coefficient, no masking -- per gather 1 unpack, 1 address op, 1 ds_read_b128, 4 adds.
+//     no coefficient, no masking -- per gather 1 address op (a 16-bit multiply-add on one half of
+//     the index word), 1 ds_read_b128, 4 adds.
 //   * lidx[k] = (row of X - first row of the tile) * 8 | sign << 15  (pre-multiplied so that the
 //     byte offset into LDS is (lidx + float4 index of the lane) << 4).
 // At the end the sums are added to what the slab kernel wrote for the remaining ("remote") entries
@@ -513,6 +514,23 @@ constexpr int kTiledWaves = 16;            // one 1024-thread workgroup
 // entries per row and set in flight, added strictly in order; nothing is read from Z and no launch
 // of the slab kernel is needed.  While one workgroup waits on the fabric in that phase, the
 // workgroups of other CUs are in their LDS phase: the two resources overlap across the chip.
+// LDS byte address of a tile row for one lane: half `hi` of `word` holds (row of the tile) x 8; the row
+// is LPE x 16 bytes long and `lane_lds` is the LDS address of the lane's float4 in row 0.
+typedef const __attribute__((address_space(3))) f32x4* lds_f32x4_ptr;
+template <int LPE>
+__device__ __forceinline__ uint32_t lds_row_address(uint32_t word, int hi, uint32_t lane_lds) {
+    static_assert(LPE == 8 || LPE == 4, "rows of 128 or 64 bytes");
+    uint32_t at;
+    if (LPE == 8) {
+        if (hi) asm("v_mad_u32_u16 %0, %1, 16, %2 op_sel:[1,0,0,0]" : "=v"(at) : "v"(word), "v"(lane_lds));
+        else asm("v_mad_u32_u16 %0, %1, 16, %2 op_sel:[0,0,0,0]" : "=v"(at) : "v"(word), "v"(lane_lds));
+    } else {
+        if (hi) asm("v_mad_u32_u16 %0, %1, 8, %2 op_sel:[1,0,0,0]" : "=v"(at) : "v"(word), "v"(lane_lds));
+        else asm("v_mad_u32_u16 %0, %1, 8, %2 op_sel:[0,0,0,0]" : "=v"(at) : "v"(word), "v"(lane_lds));
+    }
+    return at;
+}
+
 template <int TILE, bool SIGNED, int LPE, bool FUSED>
 __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_tiled_local(
     const int32_t* __restrict__ panel_ptr, const int32_t* __restrict__ blk_tile, const int32_t* __restrict__ seg,
@@ -528,6 +546,7 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
     const int sub = lane / LPE, li = lane % LPE;
     if (threadIdx.x < LPE) tile_lds[TILE * LPE + threadIdx.x] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     constexpr uint32_t kPad = (uint32_t)(TILE * 8) | ((uint32_t)(TILE * 8) << 16);    // two entries of the zero row
+    const uint32_t lane_lds = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float4*)tile_lds + li);
     // Workgroup b runs on XCD b % 8.  Items (panel-major, slab-minor) are cut into 8 contiguous
     // ranges, one per XCD, and dealt cyclically to the XCD's workgroups: the workgroups of an XCD
     // work on neighbouring panels at the same time, which share their tiles through the XCD's L2.
@@ -582,22 +601,23 @@ __global__ __launch_bounds__(kWave * kTiledWaves) __attribute__((amdgpu_waves_pe
                 // 8 entries = one 16-byte vector; gathers, then adds in entry order
                 auto gather8 = [&](const uint4& v) {
                     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-                    float4 x[8];
+                    f32x4 x[8];
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
-                        const uint32_t p = (u & 1) ? (w[u >> 1] >> 16) : (w[u >> 1] & 0xffffu);
-                        const uint32_t at = SIGNED ? (p & 0x7fffu) : p;      // row of the tile x 8
-                        x[u] = tile_lds[(LPE == 8 ? at : at >> 1) + li];
+                        // byte address in LDS = (row of the tile x 8) x (2 LPE) + 16 x lane of the group: one
+                        // 16-bit multiply-add on the selected half of the index word
+                        const uint32_t word = SIGNED ? (w[u >> 1] & 0x7fff7fffu) : w[u >> 1];
+                        x[u] = *reinterpret_cast<lds_f32x4_ptr>(lds_row_address<LPE>(word, u & 1, lane_lds));
                     }
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
                         if constexpr (SIGNED) {
                             const uint32_t p = (u & 1) ? (w[u >> 1] >> 16) : (w[u >> 1] & 0xffffu);
                             const float f = __uint_as_float(0x3f800000u | ((p & 0x8000u) << 16));
-                            acc[t][0] = fmaf(f, x[u].x, acc[t][0]); acc[t][1] = fmaf(f, x[u].y, acc[t][1]);
-                            acc[t][2] = fmaf(f, x[u].z, acc[t][2]); acc[t][3] = fmaf(f, x[u].w, acc[t][3]);
+                            acc[t][0] = fmaf(f, x[u][0], acc[t][0]); acc[t][1] = fmaf(f, x[u][1], acc[t][1]);
+                            acc[t][2] = fmaf(f, x[u][2], acc[t][2]); acc[t][3] = fmaf(f, x[u][3], acc[t][3]);
                         } else {
-                            acc[t][0] += x[u].x; acc[t][1] += x[u].y; acc[t][2] += x[u].z; acc[t][3] += x[u].w;
+                            acc[t][0] += x[u][0]; acc[t][1] += x[u][1]; acc[t][2] += x[u][2]; acc[t][3] += x[u][3];
                         }
                     }
                 };
