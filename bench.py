@@ -87,28 +87,37 @@ def compulsory_bytes(n, nnz, d):
 
 
 def time_gpu(fn, steps, warmup, torch):
-    """(wall ms per step, ms per step over the event-bracketed loop, median ms of per-call events)."""
+    """(wall ms per step, GPU ms per step, median ms of per-call events).  The first two come from ONE
+    loop of exactly ``steps`` calls issued back to back between two synchronisations (wall clock around
+    the synchronisations, one event pair inside them); the median from a second loop of the same
+    length with an event pair around every call (those records cost about 10 us per call, which is
+    why that loop is not the one the per-step figures come from)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    span_ms = a.elapsed_time(b) / steps
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
         fn()
         ends[i].record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     per_call = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    span_ms = starts[0].elapsed_time(ends[-1]) / steps
     return wall_ms, span_ms, statistics.median(per_call)
 
 
 def time_gpu_back_to_back(fn, steps, torch):
-    """ms per call of ``steps`` calls issued back to back between ONE pair of events: what a caller's
-    loop sees.  The per-call events of ``time_gpu`` put two event records around every call, which
-    costs about as much as a whole multiply on the smallest workloads."""
+    """GPU ms per call of ``steps`` calls between one pair of events (a longer loop than time_gpu's,
+    for the workloads whose multiply takes tens of microseconds)."""
     fn()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -247,9 +256,11 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
     csr_sched = schedule_rows(torch.from_numpy(rp)).to(xd.device)
     csr_step = lambda: csr_spmm(rp_d, col_d, val_d, xd, ycsr, csr_sched)
     _, csr_ms, _ = time_gpu(csr_step, args.steps, args.warmup, torch)
-    # the same two calls without events between them (more of them where a call is short)
-    reps = args.steps * (10 if span_ms < 0.2 else 1)
-    loop_ms, csr_loop_ms = time_gpu_back_to_back(step, reps, torch), time_gpu_back_to_back(csr_step, reps, torch)
+    # ten times as many calls where a call is short (launch gaps and clock ramps weigh on 20 calls of 20 us)
+    reps, loop_ms, csr_loop_ms = args.steps, span_ms, csr_ms
+    if span_ms < 0.2:
+        reps = 10 * args.steps
+        loop_ms, csr_loop_ms = time_gpu_back_to_back(step, reps, torch), time_gpu_back_to_back(csr_step, reps, torch)
     step()
     torch.cuda.synchronize()
     err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
@@ -549,8 +560,6 @@ def main():
                    "alpha": alpha, "normalized": bool(w.normalized), "tree_levels": mat.n_levels,
                    "tree_edges": ex["tree_edges"], "scale": args.scale},
         "ms_per_step_wall": ex["wall_ms"], "ms_per_step_median": ex["med_ms"],
-        "ms_per_step_back_to_back": row["cbm_ms_back_to_back"],
-        "gpu_csr_ms_back_to_back": row["gpu_csr_ms_back_to_back"],
         "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
         "cbm_frac_of_8TBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
