@@ -16,7 +16,9 @@ feature width 256.  Prints ONE JSON line.  The default run also carries, in the 
   * ``cpu_baseline``     the reference-style CPU path on the host cores of the same box, all
                          threads and one thread (``benchmark/sequential/benchmark_spmm_cpu.py:1-11``):
                          MKL ``mkl_sparse_s_mm`` (reached through torch's libtorch_cpu.so, handle
-                         re-created per call like the reference) + the OpenMP tree walk of the oracle.
+                         re-created per call like the reference) + the OpenMP tree walk of the oracle;
+  * ``gpu_vendor_csr``   the CSR product of the same matrix through ``torch.sparse.mm`` (hipSPARSE), an
+                         outside anchor for the hand-written GPU CSR baseline.
 
 ``--only-multiply`` skips the two extra sections; ``--gcn`` and ``--sweep`` run one of them alone.
 """
@@ -142,6 +144,22 @@ def csr_of(edge_index, n, m=None):
     return rp, col, val
 
 
+def vendor_csr_spmm(rp, col, val, xd, y_ref, steps, torch):
+    """The same CSR product through the vendor library: ``torch.sparse.mm`` on a CSR tensor, which
+    torch's ROCm build hands to hipSPARSE's SpMM.  An outside anchor for the hand-written GPU CSR
+    baseline; returns None where this torch build cannot run it."""
+    try:
+        n = rp.shape[0] - 1
+        values = torch.ones(col.shape[0], dtype=torch.float32) if val is None else torch.from_numpy(val)
+        a = torch.sparse_csr_tensor(torch.from_numpy(rp), torch.from_numpy(col), values, size=(n, n)).to(xd.device)
+        _, ms, med = time_gpu(lambda: torch.sparse.mm(a, xd), steps, 2, torch)
+        err = float((torch.sparse.mm(a, xd) - y_ref).abs().max() / y_ref.abs().max())
+        return {"what": "torch.sparse.mm(CSR, X) (hipSPARSE SpMM)", "ms": ms, "ms_median": med, "calls": steps,
+                "max_rel_err_vs_gpu_csr": err}
+    except Exception as e:          # noqa: BLE001 -- optional leg: report why it is absent
+        return {"what": "torch.sparse.mm(CSR, X)", "error": f"{type(e).__name__}: {e}"[:200]}
+
+
 def cpu_rows_fp64(rp, col, val, x, rows):
     """Rows ``rows`` of ``A_hat X`` in fp64 straight from the CSR arrays (SciPy): an anchor that
     shares no code with the kernels, cheap enough for every workload."""
@@ -264,6 +282,7 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
     step()
     torch.cuda.synchronize()
     err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
+    vendor = vendor_csr_spmm(rp, col, val, xd, ycsr, min(args.steps, 10), torch) if split_kernels else None
     # anchor that shares no code with the kernels: a sample of rows in fp64 from the edge list
     rows = np.sort(np.random.default_rng(0).choice(n, size=min(sample_rows, n), replace=False))
     want = cpu_rows_fp64(rp, col, val, x.numpy(), rows)
@@ -282,6 +301,8 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
         "max_rel_err_vs_gpu_csr": err_vs_csr, "max_rel_err_vs_cpu_fp64_rows": err_vs_cpu_rows,
         "cpu_rows_checked": int(rows.shape[0]), "build_s": t_build,
     }
+    if vendor is not None:
+        row["gpu_vendor_csr"] = vendor
     extra = {"mat": mat, "x": x, "xd": xd, "yd": yd, "wall_ms": wall_ms, "span_ms": span_ms, "med_ms": med_ms,
              "csr_ms": csr_ms, "b": (b_spmm, b_prop, b_csr), "t_build": t_build, "tree_edges": tree_edges}
     if split_kernels:
@@ -567,6 +588,7 @@ def main():
         "kernel_ms": {"relayout_slabs": ex["relayout_ms"], "delta_spmm": spmm_ms, "propagate": ex["prop_ms"]},
         "gpu_csr_ms": ex["csr_ms"], "gpu_csr_GBps": b_csr / (ex["csr_ms"] * 1e-3) / 1e9,
         "speedup_vs_gpu_csr": ex["csr_ms"] / span_ms,
+        "gpu_vendor_csr": row.get("gpu_vendor_csr"),
         "max_rel_err_vs_gpu_csr": row["max_rel_err_vs_gpu_csr"],
         "max_rel_err_vs_cpu_fp64_rows": row["max_rel_err_vs_cpu_fp64_rows"],
         # frac: algorithmic (gather-model, no reuse assumed) bytes over launch time -- it exceeds 1 where
