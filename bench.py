@@ -20,7 +20,7 @@ feature width 256.  Prints ONE JSON line.  The default run also carries, in the 
   * ``gpu_vendor_csr``   the CSR product of the same matrix through ``torch.sparse.mm`` (hipSPARSE), an
                          outside anchor for the hand-written GPU CSR baseline.
 
-``--only-multiply`` skips the two extra sections; ``--gcn`` and ``--sweep`` run one of them alone.
+``--only-multiply`` skips the extra sections (GCN epoch, other workloads, vendor CSR); ``--gcn`` and ``--sweep`` run one of them alone.
 """
 from __future__ import annotations
 
@@ -282,7 +282,7 @@ def measure_multiply(w, alpha, d, args, torch, split_kernels=False, sample_rows=
     step()
     torch.cuda.synchronize()
     err_vs_csr = float((yd - ycsr).abs().max() / ycsr.abs().max())
-    vendor = vendor_csr_spmm(rp, col, val, xd, ycsr, min(args.steps, 10), torch) if split_kernels else None
+    vendor = vendor_csr_spmm(rp, col, val, xd, ycsr, min(args.steps, 10), torch) if (split_kernels and not args.only_multiply) else None
     # anchor that shares no code with the kernels: a sample of rows in fp64 from the edge list
     rows = np.sort(np.random.default_rng(0).choice(n, size=min(sample_rows, n), replace=False))
     want = cpu_rows_fp64(rp, col, val, x.numpy(), rows)
@@ -509,7 +509,7 @@ def main():
                     help="threads of the multi-threaded cpu_baseline leg (default: all host cores; the reference's "
                          "benchmarks fix 16, benchmark/parallel/benchmark_spmm_cpu.py:2)")
     ap.add_argument("--only-multiply", action="store_true",
-                    help="skip the gcn_epoch and other_workloads sections of the default run")
+                    help="skip the gcn_epoch, other_workloads and gpu_vendor_csr sections of the default run")
     ap.add_argument("--max-levels", type=int, default=None,
                     help="depth limit of the arborescence (default: none, as the reference)")
     ap.add_argument("--builder", choices=("auto", "host", "gpu"), default="auto",
