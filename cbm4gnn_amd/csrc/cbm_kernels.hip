@@ -898,56 +898,94 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_narrow_levels(
 
 // A run of levels that all hold ONE row is a chain: row k's parent is row k - 1 of the run.  One
 // thread per feature column carries the running value in a register down the chain, so the only
-// dependency between levels is an add; the rows of Y it needs are independent loads and are
-// fetched kChainDepth levels ahead.  The 64 row ids (and their m) of a stretch come in with one
-// coalesced load and are broadcast with v_readlane.  Arithmetic per level is exactly that of
-// propagate_row.
-constexpr int kChainDepth = 64;
+// dependency between levels is an add; the rows of Y it needs are independent loads.  The chain is
+// walked in stretches of 64 levels -- the 64 row ids (and their m) of a stretch come in with one
+// coalesced load and are broadcast with v_readlane -- and every stretch in two halves: while one
+// half's 32 rows are added, the loads of the next half are in flight, and the ids of the stretch
+// after the next are already requested, so that no load is waited for right after it is issued.
+// All loads are unconditional (past the end of the chain: the chain's first row again) -- a load
+// that may or may not have been issued would force the wait in front of the next add down to
+// zero.  Arithmetic per level is exactly that of propagate_row.
+constexpr int kChainHalf = 32;
 constexpr int kMinChain = 4;               // shorter runs of single-row levels stay with the other kernels
 
 template <bool NORM>
 __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
     const int32_t* __restrict__ parent, const int32_t* __restrict__ order, int first, int count,
     const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy) {
+    static_assert(2 * kChainHalf == kWave, "a stretch is one row id per lane");
     const int lane = threadIdx.x & (kWave - 1);
     const int j = blockIdx.x * blockDim.x + threadIdx.x;          // feature column of this thread
     const bool live = j < d;                                      // whole waves beyond d were not launched
-    const int jj = live ? j : 0;                                  // dead lanes load column 0 and store nothing
+    const int jj = live ? j : 0;                                  // lanes past d (last wavefront only) load column 0 and store nothing
     const int v0 = order[first];
     const int u0 = parent[v0];
     float run = Y[(int64_t)u0 * ldy + jj];                         // final value of the row above the chain
     float mu = NORM ? m[u0] : 1.0f;
-    for (int base = 0; base < count; base += kWave) {
-        const int cnt = min(kWave, count - base);
-        int my_v = 0;
-        float my_m = 1.0f;
-        if (lane < cnt) {
-            my_v = order[first + base + lane];
-            if constexpr (NORM) my_m = m[my_v];
-        }
-        for (int k = 0; k < cnt; k += kChainDepth) {
-            float z[kChainDepth];
-            // unconditional loads (past the end of the stretch: its last row again), so that all
-            // kChainDepth of them are in flight before the first is needed
+    // ids of the stretch that starts at level `base`, one per lane; v0 past the end of the chain
+    auto ids = [&](int base) -> int {
+        const int g = min(base + lane, count - 1);
+        const int v = order[first + g];
+        return base + lane < count ? v : v0;
+    };
+    // A level's row of Y starts at Y + v * ldy: the lane that holds v computes the offset once per stretch, and a
+    // level gets it with two v_readlane into a scalar pair (the address of a load is then scalar base + lane column)
+    // instead of a 64-bit scalar multiply per load and per store.
+    auto row_of = [&](int64_t off_ids, int k) -> char* {         // off_ids: byte offsets v * ldy * 4, one per lane
+        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)off_ids, k);
+        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)((uint64_t)off_ids >> 32), k);
+        return reinterpret_cast<char*>(Y) + (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+    const uint32_t jj4 = (uint32_t)jj * 4u;                      // scalar row address + unsigned 32-bit byte offset of the lane
+    auto request = [&](float (&z)[kChainHalf], int64_t off_ids, int half) {
 #pragma unroll
-            for (int u = 0; u < kChainDepth; u++)
-                z[u] = Y[(int64_t)bcast_i(my_v, min(k + u, cnt - 1)) * ldy + jj];
+        for (int u = 0; u < kChainHalf; u++) z[u] = *reinterpret_cast<const float*>(row_of(off_ids, half * kChainHalf + u) + jj4);
+    };
+    // `full`: every level of this half exists (no test per level; the last stretches of a chain take the other path)
+    auto consume = [&](auto full, const float (&z)[kChainHalf], int64_t off_ids, float m_ids, int base, int half) {
 #pragma unroll
-            for (int u = 0; u < kChainDepth; u++) {
-                if (k + u < cnt) {
-                    const int v = bcast_i(my_v, k + u);
-                    if constexpr (NORM) {
-                        const float mv = bcast_f(my_m, k + u);
-                        const float inv_mu = 1.0f / mu;
-                        run = (j < dv) ? fmaf(run, inv_mu, z[u]) * mv : (z[u] + run / mu) * mv;
-                        mu = mv;
-                    } else {
-                        run = z[u] + run;
-                    }
-                    if (live) Y[(int64_t)v * ldy + j] = run;
+        for (int u = 0; u < kChainHalf; u++) {
+            const int k = half * kChainHalf + u;
+            if (decltype(full)::value || base + k < count) {
+                if constexpr (NORM) {
+                    const float mv = bcast_f(m_ids, k);
+                    const float inv_mu = 1.0f / mu;
+                    run = (jj < dv) ? fmaf(run, inv_mu, z[u]) * mv : (z[u] + run / mu) * mv;
+                    mu = mv;
+                } else {
+                    run = z[u] + run;
                 }
+                // lanes past d carry column 0 along but must not store it: the wavefront that owns column 0 may
+                // not have loaded this row yet
+                if (live) *reinterpret_cast<float*>(row_of(off_ids, k) + jj4) = run;
             }
         }
+    };
+    int v_cur = ids(0), v_nxt = ids(kWave);
+    int64_t o_cur = (int64_t)v_cur * ldy * 4, o_nxt = (int64_t)v_nxt * ldy * 4;
+    float m_cur = 1.0f;
+    if constexpr (NORM) m_cur = m[v_cur];
+    float za[kChainHalf], zb[kChainHalf];
+    request(za, o_cur, 0);
+    for (int base = 0; base < count; base += kWave) {
+        // requested first, needed last (by then older than every load still in flight): the ids of the stretch
+        // after the next, and the m of the next stretch's rows (their ids came in an iteration ago)
+        const int v_far = ids(base + 2 * kWave);
+        float m_nxt = 1.0f;
+        if constexpr (NORM) m_nxt = m[v_nxt];
+        request(zb, o_cur, 1);
+        if (base + kWave <= count) {
+            consume(std::true_type{}, za, o_cur, m_cur, base, 0);
+            request(za, o_nxt, 0);
+            consume(std::true_type{}, zb, o_cur, m_cur, base, 1);
+        } else {
+            consume(std::false_type{}, za, o_cur, m_cur, base, 0);
+            request(za, o_nxt, 0);
+            consume(std::false_type{}, zb, o_cur, m_cur, base, 1);
+        }
+        v_nxt = v_far;
+        o_cur = o_nxt; m_cur = m_nxt;
+        o_nxt = (int64_t)v_far * ldy * 4;
     }
 }
 

@@ -412,6 +412,27 @@ def test_deep_chain_uses_the_chain_kernel(orc):
         assert orc.max_rel_err(got, orc.dense_product(e2, n, x, normalized)) <= TOL_CSR
 
 
+def test_chain_lengths_around_the_stretch_size(orc):
+    # the chain kernel walks stretches of 64 levels in two halves of 32: runs of single-row levels that end
+    # inside the first half, around a half's end and around a stretch's end
+    n = 900
+    runs = set()
+    for chain in (12, 38, 39, 40, 41, 71, 72, 73, 74, 106):
+        ei = graphs.sbm_with_chain(n=n, blocks=16, p_in=1.0, mean_deg=60.0, chain=chain, base=40, seed=7)
+        for normalized, d in ((False, 96), (True, 41)):
+            e2 = graphs.add_self_loops(ei, n) if normalized else ei
+            mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
+            widths = np.diff(mat.level_off.numpy())
+            run = int(np.argmax(widths[::-1] != 1)) if (widths != 1).any() else len(widths)
+            runs.add(run)
+            say("chain of", chain, normalized, d, "levels", mat.n_levels, "single-row run", run)
+            x = np.random.default_rng(chain).standard_normal((n, d)).astype(np.float32)
+            got = gpu_product(mat, x, normalized)
+            want = oracle_product(orc, mat, e2, n, x, normalized)
+            assert np.array_equal(got, want)
+    assert {33, 64, 65} <= runs and min(runs) < 32 and max(runs) > 90, runs
+
+
 def test_strided_rows_and_cpu_staging(orc):
     n, d = 300, 48
     ei = graphs.erdos_renyi(n, 0.1, 5)
