@@ -25,6 +25,8 @@ import contextlib
 import ctypes as C
 import os
 import warnings
+import zipfile
+import zlib
 from collections import deque
 
 import numpy as np
@@ -376,36 +378,56 @@ class cbm_matrix:
                          self.n_candidates, self.n_levels, int(self.is_symmetric), self.max_levels or 0], np.int64)
         if self.edge_fingerprint is not None:
             arrays["edge_fingerprint"] = np.asarray(self.edge_fingerprint, np.uint64)
-        np.savez(self._npz_path(path), meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
+        # written under a temporary name in the same directory and renamed into place, so that a reader
+        # (another process's ``from_cache``) sees the old file or the new one, never half of one
+        final = self._npz_path(path)
+        tmp = f"{final}.{os.getpid()}.tmp.npz"
+        try:
+            np.savez(tmp, meta=meta, deltas_format=np.array(self.deltas_format), **arrays)
+            os.replace(tmp, final)
+        finally:
+            if os.path.exists(tmp):
+                os.remove(tmp)
 
     @classmethod
     def load(cls, path):
-        """Inverse of ``save``; runs no builder.  Consistency of the arrays is checked."""
+        """Inverse of ``save``; runs no builder.  Everything a kernel would index with is checked on the
+        host first (``_validate_loaded``): a stale, truncated or edited file raises ``ValueError`` here
+        instead of becoming an out-of-bounds gather on the GPU.  The reference's only guard on a format
+        is ``check_format`` (``cbm.py:69-115``), which needs the edge list; these checks need only the file."""
         path = cls._npz_path(path)
-        with np.load(path, allow_pickle=False) as z:
-            meta = z["meta"].tolist()
-            if meta[0] not in (1, 2, cls.FORMAT_VERSION):
-                raise ValueError(f"unsupported CBM file version {meta[0]}")
-            self = cls.__new__(cls)
-            (_, self.num_rows, self.alpha, normalized, self.nnz, self.nnz_a, self.n_candidates, self.n_levels,
-             symmetric) = meta[:9]
-            self.max_levels = (meta[9] or None) if meta[0] >= 2 else None
-            self.normalized, self.is_symmetric = bool(normalized), bool(symmetric)
-            self.deltas_format = str(z["deltas_format"])
-            for k in cls._SAVED_ARRAYS:
-                setattr(self, k, torch.from_numpy(z[k].copy()))
-            self.col_multiplier = torch.from_numpy(z["col_multiplier"].copy()) if "col_multiplier" in z.files else None
-            self._edge_index_cpu = torch.from_numpy(z["edge_index"].copy()) if "edge_index" in z.files else None
-            self._edge_fingerprint = z["edge_fingerprint"].copy() if "edge_fingerprint" in z.files else None
-            self._fingerprint_source = None
-        n = self.num_rows
-        ok = (self.rowptr.numel() == n + 1 and int(self.rowptr[-1]) == self.nnz == self.idx.numel()
-              and self.parent.numel() == n and self.order.numel() == n and self.level_off.numel() == self.n_levels + 1
-              and int(self.level_off[-1]) == n and self.mst_row.numel() == n + 2 and self.mst_col.numel() == n
-              and (self.col_multiplier is None) == (not self.normalized)
-              and (self.is_symmetric or self._edge_index_cpu is not None))
-        if not ok:
-            raise ValueError(f"{path} does not hold a consistent CBM format")
+        try:
+            z = np.load(path, allow_pickle=False)
+        except (zipfile.BadZipFile, EOFError) as e:
+            raise ValueError(f"{path} is not a readable .npz file: {e}") from None
+        with z:
+            try:
+                meta = np.asarray(z["meta"]).tolist()
+                if not isinstance(meta, list) or len(meta) < 9 or meta[0] not in (1, 2, cls.FORMAT_VERSION):
+                    raise ValueError(f"unsupported CBM file version {meta[0] if isinstance(meta, list) and meta else meta}")
+                self = cls.__new__(cls)
+                (_, self.num_rows, self.alpha, normalized, self.nnz, self.nnz_a, self.n_candidates, self.n_levels,
+                 symmetric) = [int(v) for v in meta[:9]]
+                self.max_levels = (int(meta[9]) or None) if (meta[0] >= 2 and len(meta) > 9) else None
+                self.normalized, self.is_symmetric = bool(normalized), bool(symmetric)
+                self.deltas_format = str(z["deltas_format"])
+                host = {k: z[k] for k in cls._SAVED_ARRAYS}
+                m = z["col_multiplier"] if "col_multiplier" in z.files else None
+                edges = z["edge_index"] if "edge_index" in z.files else None
+                fingerprint = z["edge_fingerprint"].copy() if "edge_fingerprint" in z.files else None
+            except (zipfile.BadZipFile, EOFError, zlib.error) as e:       # a member cut short or damaged
+                raise ValueError(f"{path} is damaged: {e}") from None
+            except KeyError as e:
+                raise ValueError(f"{path} lacks the array {e}") from None
+        problem = cls._validate_loaded(self, host, m, edges, fingerprint)
+        if problem:
+            raise ValueError(f"{path} does not hold a consistent CBM format: {problem}")
+        for k in cls._SAVED_ARRAYS:
+            setattr(self, k, torch.from_numpy(np.ascontiguousarray(host[k]).view(np.int32).copy()))
+        self._col_multiplier = None
+        self.col_multiplier = torch.from_numpy(m.copy()) if m is not None else None
+        self._edge_index_cpu = torch.from_numpy(edges.copy()) if edges is not None else None
+        self._edge_fingerprint, self._fingerprint_source = fingerprint, None
         self.build_seconds = None
         self.builder = None                                 # loaded, not built
         self._deltas, self._dev, self._transposed = None, {}, None
@@ -413,6 +435,69 @@ class cbm_matrix:
         self.relayout = True
         self._init_tiling("auto")
         return self
+
+    @staticmethod
+    def _validate_loaded(self, host, m, edges, fingerprint):
+        """Why the arrays read from a file are not a format the kernels may run on (a string), or None.
+        O(N + nnz) vectorised NumPy.  Checked: dtypes and lengths; row offsets start at 0, never decrease
+        and end at nnz; every delta column is below N and columns ascend inside a row (the tiler and the
+        column-block schedule rely on it); the tree arrays ``mst_row`` / ``mst_col`` describe a tree that
+        covers every row from the virtual root, and ``parent`` / ``order`` / ``level_off`` are exactly the
+        arrays that tree gives (so: parents in [-1, N), ``order`` a permutation sorted by (level, id), a
+        row one level below its parent, offsets monotone from 0 to N); the normalisation vector is finite
+        and positive; a directed matrix carries its edge list with ids below N."""
+        n, nnz, levels = self.num_rows, self.nnz, self.n_levels
+        if not (0 < n < 2 ** 31 and 0 <= nnz < 2 ** 31 and 0 < levels <= n and self.nnz_a >= 0 and self.n_candidates >= 0):
+            return "sizes in the header are out of range"
+        if self.max_levels is not None and not (0 < self.max_levels and levels <= self.max_levels):
+            return "more tree levels than the depth limit in the header"
+        if self.deltas_format not in ("csr", "coo"):
+            return "unknown deltas_format"
+        want_len = {"rowptr": n + 1, "idx": nnz, "parent": n, "order": n, "level_off": levels + 1, "mst_row": n + 2, "mst_col": n}
+        for k, length in want_len.items():
+            a = host[k]
+            if a.dtype not in (np.dtype(np.int32), np.dtype(np.uint32)) or a.ndim != 1:
+                return f"{k} is not a vector of 32-bit integers"
+            if a.shape[0] != length:
+                return f"{k} has {a.shape[0]} entries, expected {length}"
+        rowptr = host["rowptr"].astype(np.int64)
+        if rowptr[0] != 0 or rowptr[-1] != nnz or (np.diff(rowptr) < 0).any():
+            return "rowptr does not run monotonically from 0 to nnz"
+        col = (host["idx"].view(np.uint32) & np.uint32(0x7FFFFFFF)).astype(np.int64)
+        if nnz and int(col.max()) >= n:
+            return "a delta column is not below N"
+        if nnz > 1:
+            inside = np.ones(nnz - 1, bool)                 # pair (k, k+1) lies inside one row
+            starts = rowptr[1:-1]
+            inside[starts[(starts > 0) & (starts < nnz)] - 1] = False
+            if (np.diff(col)[inside] <= 0).any():
+                return "delta columns do not ascend inside a row"
+        mst_row, mst_col = host["mst_row"].astype(np.int64), host["mst_col"].astype(np.int64)
+        if mst_row[0] != 0 or mst_row[-1] != n or (np.diff(mst_row) < 0).any():
+            return "mst_row does not run monotonically from 0 to N"
+        if mst_col.min() < 0 or mst_col.max() >= n or np.bincount(mst_col, minlength=n).max() != 1:
+            return "mst_col is not a permutation of the rows"
+        try:
+            parent, order, level_off = tree_levels(mst_row, mst_col)
+        except ValueError as e:
+            return f"mst_row / mst_col: {e}"
+        for k, derived in (("parent", parent), ("order", order), ("level_off", level_off)):
+            if derived.shape[0] != host[k].shape[0] or not np.array_equal(derived, host[k].view(np.int32)):
+                return f"{k} is not what the tree in mst_row / mst_col gives"
+        if (m is None) == self.normalized:
+            return "normalisation flag and col_multiplier disagree"
+        if m is not None and not (m.dtype == np.float32 and m.shape == (n,) and np.isfinite(m).all() and (m > 0).all()):
+            return "col_multiplier is not a finite positive float32 vector of N entries"
+        if not self.is_symmetric and edges is None:
+            return "a directed matrix without its edge list"
+        if edges is not None:
+            if edges.dtype != np.int32 or edges.ndim != 2 or edges.shape[0] != 2 or edges.shape[1] == 0:
+                return "edge_index is not an int32 [2, E] array"
+            if edges.min() < 0 or edges.max() >= n:
+                return "edge_index names a row that is not below N"
+        if fingerprint is not None and not (fingerprint.dtype == np.uint64 and fingerprint.shape == (4,)):
+            return "edge_fingerprint is not uint64[4]"
+        return None
 
     @property
     def edge_fingerprint(self):
@@ -434,7 +519,7 @@ class cbm_matrix:
         if os.path.exists(file):
             try:
                 got = cls.load(file)
-            except (ValueError, KeyError, OSError):
+            except (ValueError, KeyError, OSError, zipfile.BadZipFile):
                 got = None
             ei = torch.as_tensor(edge_index)
             if (got is not None and got.edge_fingerprint is not None and got.alpha == int(alpha)

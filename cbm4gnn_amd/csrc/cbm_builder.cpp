@@ -768,28 +768,44 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
     try {
         // pass 1: per panel, the tiles that hold at least min_block_entries of its entries
         std::vector<std::vector<int32_t>> tiles_of(n_panels);
-        int bad = 0;
+        // (a std::bad_alloc must not leave a parallel region: caught inside, flagged, rethrown after it)
+        int bad = 0, no_memory = 0;
 #pragma omp parallel num_threads(threads)
         {
-            std::vector<int64_t> cnt(n_tiles, 0);
-            std::vector<int32_t> touched;
+            try {
+                std::vector<int64_t> cnt(n_tiles, 0);
+                std::vector<int32_t> touched;
 #pragma omp for schedule(dynamic, 4)
-            for (int32_t p = 0; p < n_panels; p++) {
-                touched.clear();
-                const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
-                for (int64_t k = rowptr[(int64_t)p * P]; k < rowptr[r_end]; k++) {
-                    const uint32_t c = idx[k] & 0x7fffffffu;
-                    if (c >= (uint32_t)n) { bad = 1; continue; }
-                    const int32_t t = (int32_t)(c / (uint32_t)T);
-                    if (cnt[t]++ == 0) touched.push_back(t);
+                for (int32_t p = 0; p < n_panels; p++) {
+                    touched.clear();
+                    const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
+                    int wrong = 0;
+                    for (int32_t r = p * P; r < r_end; r++) {
+                        int64_t before = -1;                // columns must ascend inside a row: the fill below
+                        for (int64_t k = rowptr[r]; k < rowptr[r + 1]; k++) {   // takes a block's entries as one run
+                            const uint32_t c = idx[k] & 0x7fffffffu;
+                            if (c >= (uint32_t)n || (int64_t)c <= before) { wrong = 1; continue; }
+                            before = c;
+                            const int32_t t = (int32_t)(c / (uint32_t)T);
+                            if (cnt[t]++ == 0) touched.push_back(t);
+                        }
+                    }
+                    if (wrong) {
+#pragma omp atomic write
+                        bad = 1;
+                    }
+                    std::sort(touched.begin(), touched.end());
+                    for (int32_t t : touched) {
+                        if (cnt[t] >= min_block_entries) tiles_of[p].push_back(t);
+                        cnt[t] = 0;
+                    }
                 }
-                std::sort(touched.begin(), touched.end());
-                for (int32_t t : touched) {
-                    if (cnt[t] >= min_block_entries) tiles_of[p].push_back(t);
-                    cnt[t] = 0;
-                }
+            } catch (const std::bad_alloc&) {
+#pragma omp atomic write
+                no_memory = 1;
             }
         }
+        if (no_memory) throw std::bad_alloc();
         if (bad) return CBM_ERR_SHAPE;
         out->n = n; out->tile_rows = T; out->panel_rows = P; out->n_panels = n_panels;
         out->panel_ptr = (int32_t*)malloc(sizeof(int32_t) * ((size_t)n_panels + 1));
@@ -809,10 +825,16 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
         int any_negative = 0;
 #pragma omp parallel num_threads(threads)
         {
-            std::vector<int32_t> block_of(n_tiles, -1);
+            std::vector<int32_t> block_of;
+            try { block_of.assign(n_tiles, -1); } catch (const std::bad_alloc&) {
+#pragma omp atomic write
+                no_memory = 1;
+            }
             int neg = 0;
+            const bool usable = (int32_t)block_of.size() == n_tiles;
 #pragma omp for schedule(dynamic, 4)
             for (int32_t p = 0; p < n_panels; p++) {
+                if (!usable) continue;
                 const int32_t b0 = out->panel_ptr[p];
                 for (size_t i = 0; i < tiles_of[p].size(); i++) block_of[tiles_of[p][i]] = b0 + (int32_t)i;
                 const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
@@ -832,6 +854,7 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                 any_negative = 1;
             }
         }
+        if (no_memory) throw std::bad_alloc();
         // counts -> offsets: segments padded to multiples of 8 entries, seg[] in units of 8 entries
         int64_t at8 = 0, real = 0;
         for (int32_t b = 0; b < B; b++) {
@@ -859,10 +882,15 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
         const uint16_t pad = (uint16_t)(T * 8);
 #pragma omp parallel num_threads(threads)
         {
-            std::vector<int32_t> block_of(n_tiles, -1);
-            std::vector<int32_t> fill(P > 0 ? P : 1);
+            std::vector<int32_t> block_of;
+            try { block_of.assign(n_tiles, -1); } catch (const std::bad_alloc&) {
+#pragma omp atomic write
+                no_memory = 1;
+            }
+            const bool usable = (int32_t)block_of.size() == n_tiles;
 #pragma omp for schedule(dynamic, 4)
             for (int32_t p = 0; p < n_panels; p++) {
+                if (!usable) continue;
                 const int32_t b0 = out->panel_ptr[p];
                 for (size_t i = 0; i < tiles_of[p].size(); i++) block_of[tiles_of[p][i]] = b0 + (int32_t)i;
                 const int32_t r_end = std::min<int64_t>((int64_t)(p + 1) * P, n);
@@ -901,6 +929,7 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                 for (int32_t t : tiles_of[p]) block_of[t] = -1;
             }
         }
+        if (no_memory) throw std::bad_alloc();
         return CBM_OK;
     } catch (const std::bad_alloc&) {
         cbm_tiling_free(out);

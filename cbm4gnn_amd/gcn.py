@@ -27,7 +27,9 @@ the multiply:
 * the Linear output, the layer output, the workspace and the gradient buffer are allocated once
   per layer and reused by every call, as the reference caches its output
   (``cbm_message_passing.py:26-29``).  As there, the tensor a call returns is overwritten by the
-  next call of the same layer.
+  next call of the same layer.  A backward that would read an overwritten buffer raises: the layer
+  counts its forward calls and bumps the buffer's autograd version, so ``forward, forward, backward
+  of the first`` is an error, never a wrong gradient (``fused=False`` allocates per call instead).
 """
 from __future__ import annotations
 
@@ -90,6 +92,14 @@ class _FusedGCNLayer(torch.autograd.Function):
         torch.mm(xd, weight.detach().t(), out=b["h"])
         op._run_spmm_update(b["h"], b["y"], use_m=op.col_multiplier is not None,
                             workspace=b["ws"] if b["copy_h"] else None, relu=layer.relu)
+        # The kernels wrote y through a raw pointer, which autograd cannot see: say so, so that a tensor
+        # saved on this storage by an earlier call (the next layer keeps its input for its weight gradient)
+        # fails its version check in backward instead of silently holding this call's values ...
+        torch.autograd.graph.increment_version(b["y"])
+        # ... and count the calls: this layer's own backward reads y as the ReLU mask and must see the
+        # y of the forward it belongs to.
+        layer._generation += 1
+        ctx.generation = layer._generation
         ctx.layer = layer
         ctx.save_for_backward(xd, weight)
         return b["y"].detach()                              # a fresh tensor object on the cached storage
@@ -97,6 +107,10 @@ class _FusedGCNLayer(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         layer = ctx.layer
+        if layer._generation != ctx.generation:
+            raise RuntimeError("CBMGCNLayer(fused=True) keeps one output buffer per layer: this layer ran forward again "
+                               "before the backward of an earlier call, which overwrote the output that backward needs. "
+                               "Run backward before the next forward, or build the layer with fused=False.")
         x, weight = ctx.saved_tensors
         op_t = layer.cached_a_t.transposed()
         n, d = g.shape
@@ -131,6 +145,7 @@ class CBMGCNLayer(nn.Module):
         self.cached_a_t = operator
         self.fused, self.relu = bool(fused), bool(relu)
         self._cache = None
+        self._generation = 0                                # forward calls of the fused path so far
 
     def _layer_buffers(self, n, d, device):
         """Device buffers of the layer for n rows of width d, allocated at the first call."""

@@ -198,6 +198,8 @@ int cbm_schedule_rows_blocks(const int32_t* rowptr, const uint32_t* idx, const i
  *   lidx[nnz_local_padded]    (row of X - first row of the tile) * 8 | (negative ? 1 << 15 : 0);
  *                             padding = tile_rows * 8, the all-zero row behind the tile
  *   rowptr_r / idx_r          the remote entries, packed like idx, columns ascending
+ * The columns of every row must ascend strictly and lie below n (the fill takes a block's entries of
+ * a row as one run): anything else is CBM_ERR_SHAPE, running out of memory CBM_ERR_ALLOC.
  * threads <= 0 means all OpenMP threads.  HOST pointers; release with cbm_tiling_free.  No reference
  * counterpart: the reference hands its delta matrix to mkl_sparse_s_mm as it is
  * (cbm_extensions.cpp:1133-1159). */

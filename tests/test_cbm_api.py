@@ -1,5 +1,7 @@
 """Host-side surface of cbm_matrix (no GPU): constructor, attributes, the reference's method
 names, error behaviour, and the loud failure when no HIP device exists."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -206,3 +208,96 @@ def test_edge_fingerprint_and_cache_file(tmp_path):
     (tmp_path / "junk.npz").write_bytes(b"not a zip file")
     assert cbm_matrix.from_cache(str(tmp_path / "junk"), torch.from_numpy(ei), alpha=0).builder is not None
     assert cbm_matrix.from_cache(str(tmp_path / "junk"), torch.from_numpy(ei), alpha=0).builder is None
+
+
+def _corruptions(z, n):
+    """(name, changed arrays) pairs: one damaged copy of a saved file per array a kernel indexes with."""
+    def with_(**kw):
+        out = {k: v.copy() for k, v in z.items()}
+        out.update(kw)
+        return out
+
+    idx, rowptr, parent, order = z["idx"], z["rowptr"], z["parent"], z["order"]
+    level_off, mst_row, mst_col = z["level_off"], z["mst_row"], z["mst_col"]
+    k = int(np.argmax(np.diff(rowptr) >= 2))                 # a row with at least two entries
+    lo = int(rowptr[k])
+    swapped = idx.copy(); swapped[[lo, lo + 1]] = swapped[[lo + 1, lo]]
+    big = idx.copy(); big[3] = 10 ** 6
+    neg_big = idx.copy(); neg_big[3] = np.int32(-(2 ** 31) + n)          # sign bit set, column N
+    far = parent.copy(); far[5] = 4000
+    root = int(np.argmax(parent >= 0))                       # a row that has a parent: claim it hangs off the root
+    orphan = parent.copy(); orphan[root] = -1
+    other = parent.copy(); other[root] = (other[root] + 1) % n
+    dup = order.copy(); dup[1] = dup[0]
+    rev = order.copy(); rev[:2] = rev[:2][::-1]
+    hump = rowptr.copy(); hump[k + 1] = hump[k] - 1 if hump[k] > 0 else hump[k + 2] + 1
+    short_end = rowptr.copy(); short_end[-1] -= 1
+    lv = level_off.copy(); lv[1] = lv[1] - 1 if lv.shape[0] > 2 else lv[1]
+    mr = mst_row.copy(); mr[1:-1] = mr[1:-1][::-1] if not np.array_equal(mr[1:-1], mr[1:-1][::-1]) else mr[1:-1] + 1
+    mc = mst_col.copy(); mc[0] = mc[1]
+    mc_swap = mst_col.copy(); mc_swap[[0, n - 1]] = mc_swap[[n - 1, 0]]
+    meta = z["meta"].copy(); meta[1] += 1
+    meta_nnz = z["meta"].copy(); meta_nnz[4] += 1
+    cases = [("idx out of range", with_(idx=big)), ("idx out of range under the sign bit", with_(idx=neg_big)),
+             ("idx unsorted", with_(idx=swapped)), ("idx truncated", with_(idx=idx[:-1])),
+             ("idx dtype", with_(idx=idx.astype(np.int64))),
+             ("parent out of range", with_(parent=far)), ("parent says root", with_(parent=orphan)),
+             ("parent names another row", with_(parent=other)),
+             ("order not a permutation", with_(order=dup)), ("order not sorted", with_(order=rev)),
+             ("rowptr not monotone", with_(rowptr=hump)), ("rowptr end", with_(rowptr=short_end)),
+             ("level_off", with_(level_off=lv)), ("level_off truncated", with_(level_off=level_off[:-1])),
+             ("mst_row", with_(mst_row=mr)), ("mst_col not a permutation", with_(mst_col=mc)),
+             ("mst_col another tree", with_(mst_col=mc_swap)),
+             ("N in the header", with_(meta=meta)), ("nnz in the header", with_(meta=meta_nnz))]
+    if "col_multiplier" in z:
+        nan = z["col_multiplier"].copy(); nan[2] = np.nan
+        cases += [("m not finite", with_(col_multiplier=nan)), ("m truncated", with_(col_multiplier=z["col_multiplier"][:-1])),
+                  ("m missing", {k_: v for k_, v in z.items() if k_ != "col_multiplier"})]
+    if "edge_index" in z:
+        e = z["edge_index"].copy(); e[0, 0] = n + 7
+        cases += [("edge_index out of range", with_(edge_index=e)),
+                  ("edge_index missing", {k_: v for k_, v in z.items() if k_ != "edge_index"})]
+    return cases
+
+
+@pytest.mark.parametrize("kind", ["undirected", "directed"])
+def test_load_rejects_every_damaged_array(tmp_path, kind):
+    """A file whose arrays would send a kernel out of bounds (or to a wrong product) never loads: every
+    check of ``load`` is exercised on the host with one damaged copy of a good file per array.  None of
+    these files goes anywhere near a GPU."""
+    n = 50
+    if kind == "undirected":
+        ei = torch.from_numpy(graphs.add_self_loops(graphs.sbm(n, 5, 0.7, 0.05, seed=4), n))
+    else:
+        rng = np.random.default_rng(3)
+        dense = rng.random((n, n)) < 0.25
+        dense[np.arange(n), (np.arange(n) + 1) % n] = True              # every row and column used
+        dense[10:20] = dense[10]                                         # rows that share everything: a tree
+        dense[10:20, 30:40] ^= np.eye(10, dtype=bool)
+        ei = torch.from_numpy(np.stack(np.nonzero(dense)).astype(np.int32))
+    a = cbm_matrix(ei, None, alpha=0, normalized=True)
+    assert a.n_levels >= 2 and (kind == "undirected") == a.is_symmetric
+    good = str(tmp_path / "good.npz")
+    a.save(good)
+    assert not [f for f in os.listdir(tmp_path) if ".tmp" in f]          # written under a temporary name, renamed
+    z = dict(np.load(good))
+    assert cbm_matrix.load(good).check_format(ei)
+    seen = set()
+    for name, arrays in _corruptions(z, n):
+        path = str(tmp_path / "damaged.npz")
+        np.savez(path, **arrays)
+        with pytest.raises(ValueError) as err:
+            cbm_matrix.load(path)
+        seen.add(str(err.value).split(": ", 1)[-1])
+        # ... and the cache rebuilds instead of trusting it
+        rebuilt = cbm_matrix.from_cache(path, ei, alpha=0, normalized=True)
+        assert rebuilt.builder is not None and torch.equal(rebuilt.idx, a.idx), name
+        assert cbm_matrix.from_cache(path, ei, alpha=0, normalized=True).builder is None, name
+    assert len(seen) >= 12                                               # the cases trip different checks
+    # a file cut short (a writer that died, a partial copy)
+    blob = open(good, "rb").read()
+    for cut in (len(blob) // 2, len(blob) - 7, 10):
+        (tmp_path / "cut.npz").write_bytes(blob[:cut])
+        with pytest.raises(ValueError):
+            cbm_matrix.load(str(tmp_path / "cut.npz"))
+        assert cbm_matrix.from_cache(str(tmp_path / "cut"), ei, alpha=0, normalized=True).builder is not None

@@ -613,6 +613,56 @@ def test_two_layer_gcn_forward_backward_matches_dense(orc, fused, alpha, directe
     assert abs(float(base_loss.detach()) - float(loss.detach())) <= 1e-5 * abs(float(loss.detach()))
 
 
+def test_fused_gcn_layer_refuses_a_backward_whose_buffers_were_overwritten(orc):
+    """The fused layer keeps one output buffer per layer (as the reference caches its output,
+    cbm_message_passing.py:26-29): backward of a call whose output a later forward has overwritten must
+    raise -- for the layer's own ReLU mask (call counter) and for the next layer's saved input (autograd
+    version of the buffer) -- while the ordinary forward/backward sequence gives the dense gradient."""
+    from cbm4gnn_amd.gcn import CBMGCNLayer, TwoLayerGCN, build_operator
+    n, f_in, hidden, classes = 200, 19, 64, 7
+    ei_np = graphs.add_self_loops(graphs.sbm(n, 4, 0.3, 0.02, seed=12), n)
+    op = build_operator(torch.from_numpy(ei_np), alpha=1, normalized=True)
+    torch.manual_seed(3)
+    model = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op, relu=True), CBMGCNLayer(hidden, classes, op), relu_between=False).cuda()
+    x1 = torch.randn((n, f_in), generator=torch.Generator().manual_seed(4)).cuda()
+    x2 = torch.randn((n, f_in), generator=torch.Generator().manual_seed(5)).cuda()
+    say("fused gcn layer: second forward before backward")
+    first = model(x1).square().sum()
+    with torch.no_grad():
+        model(x2)                                           # e.g. an evaluation pass in between
+    with pytest.raises(RuntimeError):
+        first.backward()
+    # only the FIRST layer runs again: the second layer's saved input lives in the first layer's buffer
+    model.zero_grad(set_to_none=True)
+    second = model(x1).square().sum()
+    with torch.no_grad():
+        model.first_layer(x2)
+    with pytest.raises(RuntimeError):
+        second.backward()
+    # forward -> backward, twice on different inputs: gradients of the dense fp64 model each time
+    a = torch.from_numpy(orc.dense_adjacency(np.stack([ei_np[1], ei_np[0]]), n)).double().cuda()
+    m = a.sum(dim=1).pow(-0.5)
+    a_hat = m[:, None] * a * m[None, :]
+    for x in (x1, x2):
+        model.zero_grad(set_to_none=True)
+        model(x).square().sum().backward()
+        w1 = model.first_layer.lin.weight.detach().double().requires_grad_(True)
+        w2 = model.last_layer.lin.weight.detach().double().requires_grad_(True)
+        (a_hat @ ((a_hat @ (x.double() @ w1.t())).relu() @ w2.t())).square().sum().backward()
+        for got, want in ((model.first_layer.lin.weight.grad, w1.grad), (model.last_layer.lin.weight.grad, w2.grad)):
+            assert float((got.double() - want).abs().max() / want.abs().max()) <= 1e-3
+    # the un-fused composition allocates per call and may interleave
+    torch.manual_seed(3)
+    loose = TwoLayerGCN(CBMGCNLayer(f_in, hidden, op, fused=False), CBMGCNLayer(hidden, classes, op, fused=False)).cuda()
+    out1 = loose(x1).square().sum()
+    loose(x2)
+    out1.backward()
+    w1 = loose.first_layer.lin.weight.detach().double().requires_grad_(True)
+    w2 = loose.last_layer.lin.weight.detach().double().requires_grad_(True)
+    (a_hat @ ((a_hat @ (x1.double() @ w1.t())).relu() @ w2.t())).square().sum().backward()
+    assert float((loose.first_layer.lin.weight.grad.double() - w1.grad).abs().max() / w1.grad.abs().max()) <= 1e-3
+
+
 def test_relu_epilogue_and_masked_copy_through_the_c_abi(orc):
     """CBM_UPDATE_RELU on a flat and on a deeper tree equals max(multiply, 0) bit for bit, for
     widths on both SpMM kernels; cbm_relayout_slabs_masked_f32 holds x where the mask is positive."""
@@ -789,18 +839,53 @@ def test_degenerate_shapes(orc):
         one.omp_mkl_csr_spmm_update(x, x)                             # in place is refused
 
 
-def test_alpha_tuner_reports_every_alpha_and_picks_the_fastest():
+def _oracle_levels(parent):
+    """Number of tree levels from the oracle's parent array (-1 or N = child of the virtual root)."""
+    parent = np.asarray(parent, np.int64)
+    n = parent.shape[0]
+    level = np.where((parent < 0) | (parent >= n), 0, -1)
+    while (level < 0).any():
+        known = (level < 0) & (level[np.clip(parent, 0, n - 1)] >= 0)
+        assert known.any()
+        level[known] = level[parent[known]] + 1
+    return int(level.max()) + 1
+
+
+def test_alpha_tuner_reports_every_alpha_and_picks_the_fastest(orc):
+    """Every candidate alpha is held against the ORACLE, not only against this library's own CSR kernel
+    (the reference's searcher asserts each candidate against an independent product,
+    alpha_searcher/spmm_cpu_parallel.py:116-124): delta entries = the oracle builder's arborescence weight,
+    candidate count and compression ratio = the oracle's, and the product the tuner timed = dense fp64."""
     from cbm4gnn_amd.tuner import tune_alpha
     w = graphs.workload("c2", scale=0.25)
+    n, d = w.n, 64
     say("alpha tuner")
-    best, rows = tune_alpha(w.edge_index, 64, alphas=(0, 4, 10_000), normalized=True, iters=10, warmup=2)
+    x = np.random.default_rng(5).standard_normal((n, d)).astype(np.float32)
+    dense = orc.dense_product(w.edge_index, n, x, True)
+    best, rows = tune_alpha(w.edge_index, d, alphas=(0, 4, 10_000), normalized=True, iters=10, warmup=2,
+                            x=x, reference=dense, reference_tolerance=TOL_CBM)
     assert [r["alpha"] for r in rows] == [0, 4, 10_000]
+    for r in rows:
+        o = orc.build_format(w.edge_index, n, r["alpha"])
+        assert r["nnz_delta"] == o["nnz"] == o["msa_weight"] and r["n_candidates"] == o["n_candidates"]
+        assert r["compression_ratio"] == pytest.approx(orc.compression_ratio(n, w.edge_index.shape[1], o["nnz"]))
+        # equal-weight arborescences may differ in depth between two algorithms; flat is flat for both
+        assert (r["tree_levels"] == 1) == (_oracle_levels(o["parent"]) == 1)
+        assert r["max_rel_err_vs_reference"] is not None and r["max_rel_err_vs_reference"] <= TOL_CBM
+        assert r["max_rel_err_vs_gpu_csr"] <= TOL_CSR
     assert rows[-1]["tree_levels"] == 1 and rows[-1]["compression_ratio"] < 1.0      # flat tree: delta = A
     assert rows[0]["compression_ratio"] > 1.2
-    assert all(r["max_rel_err_vs_gpu_csr"] <= 1e-3 for r in rows)
     assert best in (0, 4, 10_000)
     fastest = min(r["cbm_ms"] for r in rows)
     assert next(r for r in rows if r["alpha"] == best)["cbm_ms"] <= 1.02 * fastest
+    # the chosen alpha, multiplied once more outside the tuner: in the oracle's order bit for bit, dense at 1e-4
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=best, normalized=True)
+    got = gpu_product(mat, x, True)
+    assert np.array_equal(got, oracle_product(orc, mat, w.edge_index, n, x, True))
+    assert orc.max_rel_err(got, dense) <= TOL_CBM
+    # a reference that is NOT the product is refused (the check can fail)
+    with pytest.raises(AssertionError):
+        tune_alpha(w.edge_index, d, alphas=(10_000,), normalized=True, iters=2, warmup=1, x=x, reference=dense * 1.01)
 
 
 def test_shared_slab_major_copy(orc):
@@ -986,14 +1071,25 @@ def test_depth_limited_trees_multiply_like_the_oracle(orc, normalized):
     assert levels[0] > 8 and levels[1:] == [8, 3, 1]
 
 
-def test_tuner_sweeps_depth_limits():
+def test_tuner_sweeps_depth_limits(orc):
     from cbm4gnn_amd.tuner import tune_alpha
     w = graphs.workload("c2", scale=0.25)
     say("tuner with depth limits")
-    best, rows = tune_alpha(w.edge_index, 64, alphas=(0, 10_000), normalized=True, iters=10, warmup=2, max_levels=(None, 3))
+    x = np.random.default_rng(6).standard_normal((w.n, 64)).astype(np.float32)
+    dense = orc.dense_product(w.edge_index, w.n, x, True)
+    best, rows = tune_alpha(w.edge_index, 64, alphas=(0, 10_000), normalized=True, iters=10, warmup=2, max_levels=(None, 3),
+                            x=x, reference=dense, reference_tolerance=TOL_CBM)
     assert [(r["alpha"], r["max_levels"]) for r in rows] == [(0, None), (0, 3), (10_000, None), (10_000, 3)]
     assert rows[1]["tree_levels"] <= 3 < rows[0]["tree_levels"] and rows[1]["nnz_delta"] >= rows[0]["nnz_delta"]
     assert sum(r["best"] for r in rows) == 1 and next(r for r in rows if r["best"])["alpha"] == best
+    assert all(r["max_rel_err_vs_reference"] <= TOL_CBM for r in rows)
+    o = orc.build_format(w.edge_index, w.n, 0)
+    assert rows[0]["nnz_delta"] == o["msa_weight"] and rows[2]["nnz_delta"] == w.edge_index.shape[1]
+    # a depth-limited format is heavier than the optimum but still the same matrix: every row rebuilt from it
+    limited = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=0, normalized=True, max_levels=3)
+    assert limited.nnz == rows[1]["nnz_delta"]
+    assert orc.check_format(w.edge_index, w.n, limited.rowptr.numpy(), limited.idx.numpy().view(np.uint32),
+                            limited.mst_row.numpy(), limited.mst_col.numpy())
 
 
 def test_plain_methods_on_a_normalised_matrix_apply_the_right_scaling_only(orc):

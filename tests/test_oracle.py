@@ -192,6 +192,23 @@ def test_golden_products_normalised(orc, golden, case):
         np.testing.assert_allclose(y, golden[f"case{case}_ax_normalized"], rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("case", range(5))
+def test_dense_product_closed_form_against_golden(orc, golden, case):
+    """``dense_product`` is the fp64 closed form the GPU tests lean on; the golden products were written by
+    a script that imports neither kernels nor oracle (tests/golden/make_fixtures.py)."""
+    ei, x = golden[f"case{case}_edge_index"], golden[f"case{case}_x"]
+    n = x.shape[0]
+    assert np.array_equal(orc.dense_product(ei, n, x, False), golden[f"case{case}_ax"])         # integers: exact
+    np.testing.assert_allclose(orc.dense_product(ei, n, x, True), golden[f"case{case}_ax_normalized"], rtol=1e-13, atol=0)
+    # a directed list must not be symmetrised, and the row (not the column) degree normalises
+    tri = np.array([[0, 0, 1], [1, 2, 2]], np.int32)
+    got = orc.dense_product(np.concatenate([tri, np.array([[2], [2]], np.int32)], axis=1), 3, np.eye(3, dtype=np.float32), False)
+    assert np.array_equal(got, np.array([[0, 1, 1], [0, 0, 1], [0, 0, 1]], np.float64))
+    loops = np.array([[0, 0, 1, 2], [0, 1, 1, 2]], np.int32)                                   # row degrees 2, 1, 1
+    got = orc.dense_product(loops, 3, np.eye(3, dtype=np.float32), True)
+    assert np.allclose(got, np.array([[0.5, 2 ** -0.5, 0], [0, 1, 0], [0, 0, 1]]), rtol=1e-15)
+
+
 def test_fused_walk_formula_by_hand(orc):
     # chain root -> 0 -> 1 -> 2, d = 10: columns 0..7 take the FMA form, 8..9 the division
     # form (cbm_extensions.cpp:966-990); recompute both in NumPy fp32 step by step

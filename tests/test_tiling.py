@@ -205,3 +205,38 @@ def test_column_block_schedule():
     s1_, l1_, p1_ = mat._split_schedule(rowptr, idx, parent, m, 1)
     from cbm4gnn_amd.cbm import schedule_rows
     assert p1_ == 0 and torch.equal(s1_, schedule_rows(rowptr, parent, m))
+
+
+def test_tiling_rejects_unsorted_and_out_of_range_columns():
+    """The fill takes the entries of one row inside one block as a single ascending run; a row whose
+    columns do not ascend strictly (or leave the matrix) is refused, not tiled wrongly."""
+    import ctypes as C
+    from cbm4gnn_amd import _lib
+    host = _lib.host_lib()
+    n = 2048
+    rp = np.arange(0, 4 * (n + 1), 4, dtype=np.int32)
+    # row r holds the columns r % 1000 + {0, 7, 14, 21}
+    good = (np.arange(4, dtype=np.uint32)[None, :] * 7 + (np.arange(n, dtype=np.uint32)[:, None] % 1000)).ravel()
+
+    def run(idx):
+        t = _lib.CbmTiling()
+        rc = host.cbm_tile_rows(C.c_void_p(rp.ctypes.data), C.c_void_p(idx.ctypes.data), n, 1024, 1, 0, C.byref(t))
+        blocks = int(t.n_blocks)
+        host.cbm_tiling_free(C.byref(t))
+        return rc, blocks
+
+    rc, blocks = run(good)
+    assert rc == 0 and blocks > 0
+    for damage in ("swap", "repeat", "range", "sign"):
+        bad = good.copy()
+        if damage == "swap":
+            bad[[4 * 700, 4 * 700 + 1]] = bad[[4 * 700 + 1, 4 * 700]]
+        elif damage == "repeat":
+            bad[4 * 701 + 2] = bad[4 * 701 + 1]
+        elif damage == "range":
+            bad[4 * 702 + 3] = n
+        else:
+            bad[4 * 703 + 3] = np.uint32(0x80000000) | np.uint32(n + 5)      # out of range under the sign bit
+        assert run(bad)[0] == _lib.CBM_ERR_SHAPE, damage
+    signed = good.copy(); signed[4 * 9 + 1] |= np.uint32(0x80000000)         # a negative entry in range is fine
+    assert run(signed)[0] == 0
