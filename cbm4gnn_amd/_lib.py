@@ -64,6 +64,26 @@ class CbmTilingDev(C.Structure):
     ]
 
 
+class CbmWalkPlan(C.Structure):
+    """Mirror of ``struct cbm_walk_plan`` (host arrays made by ``cbm_walk_plan_build``)."""
+    _fields_ = [
+        ("n", C.c_int32), ("cut", C.c_int32), ("n_entries", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32),
+        ("reserved", C.c_int32), ("longest_bin", C.c_int64),
+        ("entries", C.POINTER(C.c_int32)), ("bin_off", C.POINTER(C.c_int32)),
+    ]
+
+
+class CbmWalkDev(C.Structure):
+    """Mirror of ``struct cbm_walk_dev`` (the same arrays in device memory)."""
+    _fields_ = [
+        ("cut", C.c_int32), ("n_entries", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32),
+        ("entries", C.c_void_p), ("bin_off", C.c_void_p),
+    ]
+
+
+CBM_WALK_LOAD_ONLY = 63
+CBM_WALK_MAX_SLOTS = 31
+
 _P = C.c_void_p
 _I32, _I64 = C.c_int32, C.c_int64
 
@@ -80,6 +100,8 @@ HOST_SYMBOLS = {
     "cbm_schedule_rows_blocks": (C.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _P]),
     "cbm_tile_rows": (C.c_int, [_P, _P, _I32, _I32, _I64, _I32, C.POINTER(CbmTiling)]),
     "cbm_tiling_free": (None, [C.POINTER(CbmTiling)]),
+    "cbm_walk_plan_build": (C.c_int, [_P, _P, _P, _I32, _I32, _I32, _I32, C.POINTER(CbmWalkPlan)]),
+    "cbm_walk_plan_free": (None, [C.POINTER(CbmWalkPlan)]),
     "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),
     "cbm_builder_arrays": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
                                      C.POINTER(_P), C.POINTER(_I64)]),
@@ -103,6 +125,7 @@ HIP_SYMBOLS = {
     "cbm_relayout_slabs_masked_f32": (C.c_int, [_P, _P, _P, _P, _I32, _I32, _I64, _I64, _P]),
     "cbm_relayout_slabs_scaled_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
+    "cbm_propagate_subtrees_f32": (C.c_int, [C.POINTER(CbmWalkDev), _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_paths_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_single_f32": (C.c_int, [_P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),

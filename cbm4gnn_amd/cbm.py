@@ -565,6 +565,11 @@ class cbm_matrix:
         # Products of at most this many bytes on shallow, sparse trees run as one launch (see _single_launch);
         # 0 = never.
         self.single_launch_max_bytes = 4 << 20
+        # Trees deeper than the path walk takes: "auto" walks the rows below some level by SUBTREES in one launch
+        # (``cbm_propagate_subtrees_f32``) when a cost estimate from the tree's shape says that beats one launch
+        # per level; "on" / "off" force it; an integer forces it with that cut level.
+        self.subtree_walk = "auto"
+        self._walk_plans = {}
 
     def _path_gather_ratio(self):
         """(sum over rows of the delta entries on the row's ancestor path, itself included) / nnz: the extra
@@ -673,6 +678,110 @@ class cbm_matrix:
         _lib.check(rc, "cbm_schedule_rows_blocks")
         long_rows = long_rows[:n_long.value]
         return sched, long_rows, int(long_rows[:, 2].sum()) if n_long.value else 0
+
+    # ------------------------------------------------------------------ walk by subtrees -----
+    # Rough costs of the two ways to walk a deep tree, in microseconds (measured on MI355X: a dependent launch
+    # of a small kernel, one level of the register-carried chain, one row of a subtree sequence, and the rate
+    # at which wide levels stream rows).  They only rank the plans of one tree against each other.
+    _WALK_US_PER_LAUNCH = 4.0
+    _WALK_US_PER_NARROW_LEVEL = 2.0
+    _WALK_US_PER_CHAIN_LEVEL = 0.085
+    _WALK_US_PER_ENTRY = 0.14
+    _WALK_BYTES_PER_US = 4.0e6
+
+    def _level_plan_cost_us(self, d, first_level=1, last_level=None):
+        """Estimated time of the level-by-level launches for levels first_level .. last_level - 1."""
+        lo = self.level_off.tolist()
+        levels = self.n_levels if last_level is None else last_level
+        width = lambda l: lo[l + 1] - lo[l]
+
+        def chain_end(l):
+            while l < levels and width(l) == 1:
+                l += 1
+            return l
+
+        cost, l = 0.0, first_level
+        while l < levels:
+            if width(l) == 1 and chain_end(l) - l >= 4:
+                e = chain_end(l)
+                cost += self._WALK_US_PER_LAUNCH + (e - l) * self._WALK_US_PER_CHAIN_LEVEL
+                l = e
+            elif width(l) <= 64:
+                e = l + 1
+                while e < levels and width(e) <= 64 and chain_end(e) - e < 4:
+                    e += 1
+                cost += self._WALK_US_PER_LAUNCH + (e - l) * self._WALK_US_PER_NARROW_LEVEL
+                l = e
+            else:
+                cost += max(self._WALK_US_PER_LAUNCH, width(l) * d * 12 / self._WALK_BYTES_PER_US)
+                l += 1
+        return cost
+
+    def _host_walk_plan(self, cut, d):
+        """``cbm_walk_plan_build`` for this tree at ``cut`` (CPU tensors + stats), cached.  The bins are sized so
+        that (bins x 64-column slices) wavefronts fill the GPU a few times over."""
+        slices = (d + 63) // 64
+        target_bins = max(64, 8192 // slices)
+        key = (int(cut), target_bins)
+        plan = self._walk_plans.get(key)
+        if plan is None:
+            p = _lib.CbmWalkPlan()
+            rc = _lib.host_lib().cbm_walk_plan_build(_ptr(self.parent), _ptr(self.order), _ptr(self.level_off), self.num_rows,
+                                                     self.n_levels, int(cut), target_bins, C.byref(p))
+            try:
+                if rc == 6:                                 # more live slots than the kernel has: not for this tree
+                    plan = False
+                else:
+                    _lib.check(rc, "cbm_walk_plan_build")
+                    take = lambda ptr, count: torch.from_numpy(
+                        np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(np.int32, copy=True))
+                    plan = {"cut": int(p.cut), "n_entries": int(p.n_entries), "n_bins": int(p.n_bins), "n_slots": int(p.n_slots),
+                            "longest_bin": int(p.longest_bin),
+                            "entries": take(p.entries, 2 * p.n_entries).view(-1, 2), "bin_off": take(p.bin_off, p.n_bins + 1)}
+            finally:
+                _lib.host_lib().cbm_walk_plan_free(C.byref(p))
+            self._walk_plans[key] = plan
+        return plan
+
+    def _subtree_plan_cost_us(self, plan, d):
+        return (self._level_plan_cost_us(d, 1, plan["cut"] + 1) + self._WALK_US_PER_LAUNCH +
+                max(plan["longest_bin"] * self._WALK_US_PER_ENTRY, plan["n_entries"] * d * 8 / self._WALK_BYTES_PER_US))
+
+    def walk_plan(self, d):
+        """The subtree-walk plan a multiply of width ``d`` uses, or None when it walks level by level: by
+        ``subtree_walk`` -- "off": None; an integer: that cut; "on": the cheapest cut by the estimate; "auto":
+        the cheapest cut if the estimate beats the level-by-level launches by a fifth.  (A multiply that the
+        one-launch path walk takes -- a shallow tree, a small product -- does not ask.)"""
+        policy = self.subtree_walk
+        if policy == "off" or self.n_levels < 2:
+            return None
+        if isinstance(policy, int) and not isinstance(policy, bool):
+            return self._host_walk_plan(min(max(policy, 0), self.n_levels - 2), d) or None
+        if policy not in ("auto", "on"):
+            raise ValueError('subtree_walk must be "auto", "on", "off" or a cut level')
+        key = ("choice", policy, (d + 63) // 64)
+        if key not in self._walk_plans:
+            best, best_cost = None, None
+            for cut in range(0, min(self.n_levels - 1, 4)):           # deeper cuts: the levels above cost launches again
+                plan = self._host_walk_plan(cut, d)
+                if not plan or plan["n_entries"] == 0:
+                    continue
+                cost = self._subtree_plan_cost_us(plan, d)
+                if best is None or cost < best_cost:
+                    best, best_cost = plan, cost
+            if best is not None and policy == "auto" and best_cost > 0.8 * self._level_plan_cost_us(d):
+                best = None
+            self._walk_plans[key] = best
+        return self._walk_plans[key]
+
+    def _walk_struct(self, st, plan):
+        """``struct cbm_walk_dev`` over the device copy of ``plan`` (uploaded once per device and cut)."""
+        key = ("walk", plan["cut"], plan["n_bins"])
+        dev = st.get(key)
+        if dev is None:
+            device = st["rowptr"].device
+            dev = st[key] = (plan["entries"].contiguous().to(device), plan["bin_off"].to(device))
+        return _lib.CbmWalkDev(plan["cut"], plan["n_entries"], plan["n_bins"], plan["n_slots"], dev[0].data_ptr(), dev[1].data_ptr())
 
     # Settings the cached device arrays depend on: changing one drops the cache, so that a later
     # multiply never runs on coefficients or schedules derived from the old value.
@@ -921,7 +1030,7 @@ class cbm_matrix:
         if yd is not y:
             y.copy_(yd)
 
-    def _run_propagate(self, y, use_m, flags=0):
+    def _run_propagate(self, y, use_m, flags=0, scale_roots=True):
         n = self.num_rows
         _check_f32_matrix(y, "dst", n)
         if use_m and self.col_multiplier is None:
@@ -929,14 +1038,21 @@ class cbm_matrix:
         _require_gpu()
         yd, back = self._stage(y)
         st = self._device_arrays(yd.device)
-        if use_m:
+        if use_m and scale_roots:
             flags |= _lib.CBM_PROP_SCALE_ROOTS
+        plan = self.walk_plan(y.size(1)) if n and y.size(1) else None
         with torch.cuda.device(yd.device):
-            rc = _lib.hip_lib().cbm_propagate_f32(
-                _ptr(st["parent"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off),
-                self.n_levels, _ptr(st["m"]) if use_m else None, _ptr(yd), n, y.size(1), _ld(yd),
-                flags, _stream(yd.device))
-        _lib.check(rc, "cbm_propagate_f32")
+            if plan is not None:
+                rc = _lib.hip_lib().cbm_propagate_subtrees_f32(
+                    C.byref(self._walk_struct(st, plan)), _ptr(st["parent"]), _ptr(st["order"]), _ptr(st["level_off"]),
+                    _ptr(self.level_off), self.n_levels, _ptr(st["m"]) if use_m else None, _ptr(yd), n, y.size(1), _ld(yd),
+                    flags, _stream(yd.device))
+            else:
+                rc = _lib.hip_lib().cbm_propagate_f32(
+                    _ptr(st["parent"]), _ptr(st["order"]), _ptr(st["level_off"]), _ptr(self.level_off),
+                    self.n_levels, _ptr(st["m"]) if use_m else None, _ptr(yd), n, y.size(1), _ld(yd),
+                    flags & _lib.CBM_PROP_SCALE_ROOTS, _stream(yd.device))
+        _lib.check(rc, "cbm_propagate_subtrees_f32" if plan is not None else "cbm_propagate_f32")
         if back:
             y.copy_(yd)
 
@@ -969,6 +1085,14 @@ class cbm_matrix:
                     self.n_levels, _ptr(xd), _ptr(yd), n, x.size(1), _ld(xd), _ld(yd),
                     _lib.CBM_UPDATE_RELU if relu else 0, _stream(xd.device))
             _lib.check(rc, "cbm_spmm_update_single_f32")
+            if yd is not y:
+                y.copy_(yd)
+            return
+        if (tiled or not self._walks_paths(n, x.size(1))) and self.walk_plan(x.size(1)) is not None:
+            # a deep tree: the SpMM (root children scaled in its epilogue), then the walk by subtrees
+            self._run_spmm(xd, yd, use_m, scale_roots=use_m, workspace=workspace, workspace_ready=workspace_ready,
+                           workspace_prescaled=workspace_prescaled)
+            self._run_propagate(yd, use_m, flags=_lib.CBM_UPDATE_RELU if relu else 0, scale_roots=False)
             if yd is not y:
                 y.copy_(yd)
             return

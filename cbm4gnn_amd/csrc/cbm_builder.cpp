@@ -747,6 +747,127 @@ int cbm_schedule_rows_split(const int32_t* rowptr, const int32_t* parent, const 
     return cbm_schedule_rows_blocks(rowptr, nullptr, parent, m, n, chunk, 1, sched_out, long_rows_out);
 }
 
+void cbm_walk_plan_free(cbm_walk_plan* p) {
+    if (!p) return;
+    free(p->entries); free(p->bin_off);
+    std::memset(p, 0, sizeof(*p));
+}
+
+int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32_t* level_off, int32_t n,
+                        int32_t n_levels, int32_t cut, int32_t target_bins, cbm_walk_plan* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if (!parent || !order || !level_off) return CBM_ERR_NULL;
+    if (n <= 0 || n_levels < 1 || cut < 0 || cut >= n_levels || target_bins < 1) return CBM_ERR_SHAPE;
+    if (level_off[0] != 0 || level_off[n_levels] != n) return CBM_ERR_SHAPE;
+    for (int32_t l = 0; l < n_levels; l++)
+        if (level_off[l + 1] < level_off[l]) return CBM_ERR_SHAPE;
+    try {
+        // level of every row; order must be a permutation whose rows sit one level below their parents
+        std::vector<int32_t> level(n, -1);
+        for (int32_t l = 0; l < n_levels; l++)
+            for (int32_t i = level_off[l]; i < level_off[l + 1]; i++) {
+                const int32_t v = order[i];
+                if (v < 0 || v >= n || level[v] >= 0) return CBM_ERR_SHAPE;
+                level[v] = l;
+            }
+        for (int32_t v = 0; v < n; v++) {
+            const int32_t u = parent[v];
+            if (u >= n || u == v) return CBM_ERR_SHAPE;
+            if (u < 0 ? level[v] != 0 : level[u] + 1 != level[v]) return CBM_ERR_SHAPE;
+        }
+        // children lists (CSR by parent) and subtree sizes (leaves first: order[] backwards)
+        std::vector<int32_t> child_ptr(n + 1, 0), child(n > 0 ? n : 1), size(n, 1);
+        for (int32_t v = 0; v < n; v++)
+            if (parent[v] >= 0) child_ptr[parent[v] + 1]++;
+        for (int32_t v = 0; v < n; v++) child_ptr[v + 1] += child_ptr[v];
+        {
+            std::vector<int32_t> at(child_ptr.begin(), child_ptr.end() - 1);
+            for (int32_t v = 0; v < n; v++)
+                if (parent[v] >= 0) child[at[parent[v]]++] = v;
+        }
+        for (int32_t i = n - 1; i >= 0; i--) {
+            const int32_t v = order[i];
+            if (parent[v] >= 0) size[parent[v]] += size[v];
+        }
+        // lightest child first, heaviest last (ties by id): the value of a row then has to be kept only while
+        // the walk is inside one of its lighter children, which bounds the kept values by log2(subtree size)
+        for (int32_t v = 0; v < n; v++)
+            std::sort(child.begin() + child_ptr[v], child.begin() + child_ptr[v + 1],
+                      [&](int32_t a, int32_t b) { return size[a] != size[b] ? size[a] < size[b] : a < b; });
+        // tasks: the rows of level `cut` that have children, longest subtree first (ties by id)
+        std::vector<int32_t> roots;
+        for (int32_t i = level_off[cut]; i < level_off[cut + 1]; i++)
+            if (size[order[i]] > 1) roots.push_back(order[i]);
+        std::sort(roots.begin(), roots.end(),
+                  [&](int32_t a, int32_t b) { return size[a] != size[b] ? size[a] > size[b] : a < b; });
+        int64_t total = 0;
+        for (int32_t r : roots) total += size[r];
+        if (total > INT32_MAX) return CBM_ERR_SHAPE;
+        out->n = n; out->cut = cut; out->n_entries = (int32_t)total;
+        out->entries = (int32_t*)malloc(sizeof(int32_t) * 2 * std::max<size_t>((size_t)total, 1));
+        if (!out->entries) throw std::bad_alloc();
+        // bins: consecutive tasks of the sorted list until a bin holds `target` entries
+        const int64_t target = std::max<int64_t>((total + target_bins - 1) / target_bins, CBM_WALK_MIN_BIN);
+        std::vector<int32_t> bin_off(1, 0);
+        int64_t at = 0, in_bin = 0, longest = 0;
+        int32_t max_slots = 0;
+        std::vector<std::pair<int32_t, int32_t>> stack;    // (row, next child to visit)
+        for (int32_t r : roots) {
+            if (in_bin >= target) { bin_off.push_back((int32_t)at); longest = std::max(longest, in_bin); in_bin = 0; }
+            in_bin += size[r];
+            // iterative pre-order walk; `kept` = rows on the current path whose value sits in a slot
+            int32_t kept = 0;
+            out->entries[2 * at] = r; out->entries[2 * at + 1] = CBM_WALK_LOAD_ONLY; 
+            {
+                const int32_t k = child_ptr[r + 1] - child_ptr[r];
+                if (k >= 2) { kept++; out->entries[2 * at + 1] |= kept << 8; }
+            }
+            at++;
+            stack.clear();
+            stack.emplace_back(r, 0);
+            std::vector<int32_t> slot_of_depth;            // slot of the stack's rows (0 = none)
+            slot_of_depth.push_back(kept);
+            max_slots = std::max(max_slots, kept);
+            while (!stack.empty()) {
+                const int32_t u = stack.back().first;
+                const int32_t i = stack.back().second;
+                const int32_t k = child_ptr[u + 1] - child_ptr[u];
+                if (i == k) { stack.pop_back(); slot_of_depth.pop_back(); continue; }
+                stack.back().second = i + 1;
+                const int32_t v = child[child_ptr[u] + i];
+                // source of the parent's value: the row visited just before (first child), else the parent's slot;
+                // the last child frees that slot before taking one of its own
+                int32_t ctl = (i == 0) ? 0 : slot_of_depth.back();
+                if (i == k - 1 && k >= 2) kept--;
+                const int32_t kv = child_ptr[v + 1] - child_ptr[v];
+                int32_t mine = 0;
+                if (kv >= 2) {
+                    mine = ++kept;
+                    if (mine > CBM_WALK_MAX_SLOTS) return (cbm_walk_plan_free(out), CBM_ERR_UNSUPPORTED);
+                    max_slots = std::max(max_slots, mine);
+                    ctl |= mine << 8;
+                }
+                out->entries[2 * at] = v; out->entries[2 * at + 1] = ctl;
+                at++;
+                if (kv > 0) { stack.emplace_back(v, 0); slot_of_depth.push_back(mine); }
+            }
+        }
+        if (at != total) return (cbm_walk_plan_free(out), CBM_ERR_INTERNAL);
+        if (total > 0) { bin_off.push_back((int32_t)at); longest = std::max(longest, in_bin); }
+        out->n_bins = (int32_t)bin_off.size() - 1;
+        out->n_slots = max_slots;
+        out->longest_bin = longest;
+        out->bin_off = (int32_t*)malloc(sizeof(int32_t) * bin_off.size());
+        if (!out->bin_off) throw std::bad_alloc();
+        std::copy(bin_off.begin(), bin_off.end(), out->bin_off);
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        cbm_walk_plan_free(out);
+        return CBM_ERR_ALLOC;
+    }
+}
+
 void cbm_tiling_free(cbm_tiling* t) {
     if (!t) return;
     free(t->panel_ptr); free(t->blk_tile); free(t->seg); free(t->lidx); free(t->rowptr_r); free(t->idx_r);

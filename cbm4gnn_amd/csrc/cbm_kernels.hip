@@ -989,6 +989,107 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
     }
 }
 
+// The walk of all subtrees below a level in ONE launch (plan: cbm_walk_plan_build).  A wavefront takes a bin
+// of the plan -- whole subtrees, each a sequence of rows in depth-first pre-order -- and 64 feature columns
+// (one per lane), and carries the value of the row it has just finished in a register: the next row of the
+// sequence is usually that row's first child.  A row with two or more children also leaves its value (and
+// its m) in an LDS slot of the wavefront, where the later children find it; children are ordered lightest
+// subtree first, so few slots are live at once.  Global memory is touched twice per row -- its SpMM result is
+// read, its final value written -- and no load depends on an earlier store, so, as in propagate_chain, the
+// rows of a stretch of 64 entries are requested half a stretch ahead and every load is unconditional (past
+// the end of the bin: the bin's first row again).  The head of a subtree is final already (a child of the
+// root after the SpMM, or a row of a level walked before this launch): it is loaded, not stored.
+// Arithmetic per row is exactly that of propagate_row, so Y is bit-identical to the level-by-level walk.
+constexpr int kSubWaves = 4;               // wavefronts per workgroup (each owns its LDS slots)
+
+template <bool NORM>
+__global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
+    const int2* __restrict__ entries, const int32_t* __restrict__ bin_off, int n_bins, int slices,
+    const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy, int n_slots) {
+    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int w = blockIdx.x * kSubWaves + (threadIdx.x >> 6);
+    const int bin = w / slices;
+    if (bin >= n_bins) return;
+    const int j = (w % slices) * kWave + lane;                    // feature column of this thread
+    const bool live = j < d;
+    const int jj = live ? j : 0;                                  // lanes past d load column 0 and store nothing
+    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
+    const int first = bin_off[bin], count = bin_off[bin + 1] - first;
+    const int2 e0 = entries[first];
+    auto ids = [&](int base) -> int2 {                            // entry base + lane; past the end: the first one
+        const int2 e = entries[first + min(base + lane, count - 1)];
+        return base + lane < count ? e : e0;
+    };
+    auto row_of = [&](int64_t off_ids, int k) -> char* {          // off_ids: byte offsets row * ldy * 4, one per lane
+        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)off_ids, k);
+        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)((uint64_t)off_ids >> 32), k);
+        return reinterpret_cast<char*>(Y) + (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+    const uint32_t jj4 = (uint32_t)jj * 4u;
+    auto request = [&](float (&z)[kChainHalf], int64_t off_ids, int half) {
+#pragma unroll
+        for (int u = 0; u < kChainHalf; u++) z[u] = *reinterpret_cast<const float*>(row_of(off_ids, half * kChainHalf + u) + jj4);
+    };
+    float run = 0.0f, mu = 1.0f;
+    auto consume = [&](auto full, const float (&z)[kChainHalf], int64_t off_ids, int c_ids, float m_ids, int base, int half) {
+#pragma unroll
+        for (int u = 0; u < kChainHalf; u++) {
+            const int k = half * kChainHalf + u;
+            if (decltype(full)::value || base + k < count) {
+                const int ctl = bcast_i(c_ids, k);                // wave-uniform: the branches below are scalar
+                const int src = ctl & 63, dst = (ctl >> 8) & 63;
+                const float mv = NORM ? bcast_f(m_ids, k) : 1.0f;
+                if (src == CBM_WALK_LOAD_ONLY) {
+                    run = z[u];
+                } else {
+                    float a = run, ma = mu;
+                    if (src) {
+                        a = st[(src - 1) * 2 * kWave];
+                        if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
+                    }
+                    if constexpr (NORM) {
+                        const float inv_mu = 1.0f / ma;
+                        run = (jj < dv) ? fmaf(a, inv_mu, z[u]) * mv : (z[u] + a / ma) * mv;
+                    } else {
+                        run = z[u] + a;
+                    }
+                    if (live) *reinterpret_cast<float*>(row_of(off_ids, k) + jj4) = run;
+                }
+                mu = mv;
+                if (dst) {
+                    st[(dst - 1) * 2 * kWave] = run;
+                    if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
+                }
+            }
+        }
+    };
+    int2 e_cur = ids(0), e_nxt = ids(kWave);
+    int64_t o_cur = (int64_t)e_cur.x * ldy * 4, o_nxt = (int64_t)e_nxt.x * ldy * 4;
+    float m_cur = 1.0f;
+    if constexpr (NORM) m_cur = m[e_cur.x];
+    float za[kChainHalf], zb[kChainHalf];
+    request(za, o_cur, 0);
+    for (int base = 0; base < count; base += kWave) {
+        const int2 e_far = ids(base + 2 * kWave);
+        float m_nxt = 1.0f;
+        if constexpr (NORM) m_nxt = m[e_nxt.x];
+        request(zb, o_cur, 1);
+        if (base + kWave <= count) {
+            consume(std::true_type{}, za, o_cur, e_cur.y, m_cur, base, 0);
+            request(za, o_nxt, 0);
+            consume(std::true_type{}, zb, o_cur, e_cur.y, m_cur, base, 1);
+        } else {
+            consume(std::false_type{}, za, o_cur, e_cur.y, m_cur, base, 0);
+            request(za, o_nxt, 0);
+            consume(std::false_type{}, zb, o_cur, e_cur.y, m_cur, base, 1);
+        }
+        e_cur = e_nxt; e_nxt = e_far;
+        o_cur = o_nxt; m_cur = m_nxt;
+        o_nxt = (int64_t)e_far.x * ldy * 4;
+    }
+}
+
 // The walk of a SHALLOW tree in one launch, out of place: the wavefront of row v follows parent[]
 // up to the child of the root above it (at most kMaxPathLevels - 1 steps, the ids kept one per
 // lane), then adds the rows of Z down that path with exactly the arithmetic of propagate_row, so
@@ -1585,6 +1686,7 @@ template <bool NORM>
 int launch_propagate(const int32_t* parent, const int32_t* order, const int32_t* level_off_dev,
                      const int32_t* lo, int32_t n_levels, const float* m, float* Y, int32_t n, int32_t d,
                      int64_t ldy, int32_t flags, hipStream_t s) {
+    // n_levels may be a prefix of the tree's levels: the subtree walk takes over below it
     const Tiling t = pick_tiling(d, ldy, ldy, Y, Y);
     const int dv = d - d % 8;
     const dim3 block(kWave * kWavesPerBlock);
@@ -1682,6 +1784,20 @@ int static_scratch(float** out) {
     }
     *out = g_scratch_ptr[dev];
     return CBM_OK;
+}
+
+template <bool NORM>
+int launch_subtrees(const cbm_walk_dev* w, const float* m, float* Y, int32_t d, int64_t ldy, hipStream_t s) {
+    if (w->n_bins == 0) return CBM_OK;
+    const int slices = (d + kWave - 1) / kWave;
+    const int64_t waves = (int64_t)w->n_bins * slices;
+    const int64_t blocks = (waves + kSubWaves - 1) / kSubWaves;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    const size_t lds = (size_t)kSubWaves * w->n_slots * 2 * kWave * sizeof(float);       // at most 62 KB
+    hipLaunchKernelGGL((propagate_subtrees<NORM>), dim3((unsigned)blocks), dim3(kWave * kSubWaves), lds, s,
+                       reinterpret_cast<const int2*>(w->entries), w->bin_off, w->n_bins, slices, m, Y, d, d - d % 8, ldy,
+                       w->n_slots);
+    return check_launch();
 }
 
 }  // namespace
@@ -1849,6 +1965,33 @@ int cbm_propagate_f32(const int32_t* parent, const int32_t* order, const int32_t
     hipStream_t s = static_cast<hipStream_t>(stream);
     return m ? launch_propagate<true>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s)
              : launch_propagate<false>(parent, order, level_off_dev, level_off_host, n_levels, m, Y, n, d, ldy, flags, s);
+}
+
+int cbm_propagate_subtrees_f32(const cbm_walk_dev* walk, const int32_t* parent, const int32_t* order,
+                               const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels, const float* m,
+                               float* Y, int32_t n, int32_t d, int64_t ldy, int32_t flags, void* stream) {
+    if (!walk || !parent || !order || !level_off_dev || !level_off_host || !Y) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldy)) return rc;
+    if (int rc = validate_levels(level_off_host, n_levels, n)) return rc;
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU)) return CBM_ERR_UNSUPPORTED;
+    if (n == 0 || d == 0) return CBM_OK;
+    if (walk->cut < 0 || walk->cut >= n_levels || walk->n_bins < 0 || walk->n_entries < 0 || walk->n_slots < 0 ||
+        walk->n_slots > CBM_WALK_MAX_SLOTS)
+        return CBM_ERR_SHAPE;
+    if (walk->n_bins > 0 && (!walk->entries || !walk->bin_off || !aligned(walk->entries, 8))) return CBM_ERR_NULL;
+    if ((int64_t)n * ldy * 4 > ((int64_t)1 << 46)) return CBM_ERR_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // levels 1 .. cut level by level (and the scale of the root's children, if asked), then every subtree below
+    const int32_t prop_flags = flags & CBM_PROP_SCALE_ROOTS;
+    int rc = m ? launch_propagate<true>(parent, order, level_off_dev, level_off_host, walk->cut + 1, m, Y, n, d, ldy, prop_flags, s)
+               : launch_propagate<false>(parent, order, level_off_dev, level_off_host, walk->cut + 1, m, Y, n, d, ldy, prop_flags, s);
+    if (rc) return rc;
+    rc = m ? launch_subtrees<true>(walk, m, Y, d, ldy, s) : launch_subtrees<false>(walk, m, Y, d, ldy, s);
+    if (rc || !(flags & CBM_UPDATE_RELU)) return rc;
+    const int64_t total = (int64_t)n * d, blocks = (total + 255) / 256;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    hipLaunchKernelGGL(relu_rows, dim3((unsigned)blocks), dim3(256), 0, s, Y, total, d, ldy);
+    return check_launch();
 }
 
 int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m, const float* coef,

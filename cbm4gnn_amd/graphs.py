@@ -6,7 +6,8 @@ by (row, col)) whose ids are contiguous from 0 and in which every node has at le
 edge -- the four preconditions the reference states in ``cbm/utility.py:4-29``.
 
 The five named workloads (``workload("c1") .. workload("c5")``) are the graphs the
-reference-style benchmarks of this repository run on; the reference itself downloads
+reference-style benchmarks of this repository run on (plus ``"c2b"``, the second workload held to
+its configured size, and ``"c6"``, a deep and wide tree outside the five); the reference itself downloads
 SNAP / DIMACS graphs (``benchmark/utility.py:23-42``), which is impossible offline.
 """
 from __future__ import annotations
@@ -18,7 +19,7 @@ import numpy as np
 
 __all__ = [
     "Workload", "workload", "coalesce_undirected", "add_self_loops", "edge_hash",
-    "erdos_renyi", "sbm", "duplication", "chung_lu_cliques", "sbm_with_chain",
+    "erdos_renyi", "sbm", "duplication", "chung_lu_cliques", "sbm_with_chain", "staircases",
 ]
 
 
@@ -149,18 +150,24 @@ def sbm(n: int, blocks: int, p_in: float, p_out: float, seed: int = 0, patch: bo
     return _patch_isolated(rng, ei, n) if patch else ei
 
 
-def duplication(n: int, keep: float = 0.7, extra: int = 3, seed_clique: int = 8, seed: int = 0) -> np.ndarray:
+def duplication(n: int, keep: float = 0.7, extra: int = 3, seed_clique: int = 8, seed: int = 0,
+                copy_cap: int | None = None) -> np.ndarray:
     """Duplication model: node t picks a uniform earlier node, copies that node's CURRENT
     neighbour list keeping each entry with probability ``keep``, and adds ``extra`` uniform
     random earlier nodes.  A node's row overlaps its template's by ~``keep``, which is what
     CBM compresses.  Copying current lists makes the edge count grow like t^(2*keep): with
-    keep=0.7 and n=12000 the graph has ~1.8M undirected edges."""
+    keep=0.7 and n=12000 the graph has ~1.8M undirected edges.  ``copy_cap``: copy from at most
+    this many entries of the template's list (a uniform sample of it), which bounds a new node's
+    degree and with it the growth: keep=0.7, n=12000, copy_cap=26 gives ~240k undirected edges.
+    (``copy_cap=None`` draws exactly the random numbers it always drew.)"""
     rng = np.random.default_rng(seed)
     nb = [set(s for s in range(seed_clique) if s != t) for t in range(seed_clique)] + [None] * (n - seed_clique)
     for t in range(seed_clique, n):
         proto = int(rng.integers(0, t))
         src = np.fromiter(nb[proto], np.int64, len(nb[proto]))
         src.sort()
+        if copy_cap is not None and src.size > copy_cap:
+            src = np.sort(rng.choice(src, size=copy_cap, replace=False))
         kept = src[rng.random(src.size) < keep]
         mine = set(kept.tolist()) | set(rng.integers(0, t, size=extra).tolist())
         nb[t] = mine
@@ -237,6 +244,30 @@ def sbm_with_chain(n: int = 132_534, blocks: int = 300, p_in: float = 1.0, mean_
     return coalesce_undirected(u, v, n)
 
 
+def staircases(n_chains: int = 800, depth: int = 100, base: int = 28, noise_deg: float = 2.0, seed: int = 0) -> np.ndarray:
+    """``n_chains`` disjoint half-graphs ("staircases") plus a sparse random background: a graph whose
+    minimum arborescence is DEEP AND WIDE at once.  Staircase w has ``depth`` chain nodes c_0 .. c_{depth-1}
+    and ``base + depth`` anchors; c_k is adjacent to the anchors a_0 .. a_{base+k}, so row(c_k) =
+    row(c_{k-1}) + one column, and on the other side row(a_{base+j}) = row(a_{base+j+1}) + one column: both
+    sides are chains of Hamming distance 1, ``depth`` levels deep, and every tree level holds about
+    2 * n_chains rows.  On top, ``noise_deg * n / 2`` uniform random edges, so that consecutive rows
+    differ in a handful of columns rather than one.  Node ids are shuffled: neither the kernels nor the
+    builder get the chains as contiguous id ranges.  n = n_chains * (2 * depth + base)."""
+    rng = np.random.default_rng(seed)
+    per = 2 * depth + base
+    n = n_chains * per
+    k = np.repeat(np.arange(depth, dtype=np.int64), base + 1 + np.arange(depth))      # chain node of every stair edge
+    j = np.concatenate([np.arange(base + 1 + q, dtype=np.int64) for q in range(depth)])  # its anchor
+    off = (np.arange(n_chains, dtype=np.int64) * per)[:, None]
+    u = (off + k[None, :]).ravel()                                                      # chain nodes: first `depth` ids of a staircase
+    v = (off + depth + j[None, :]).ravel()                                              # anchors: the rest
+    m = int(round(noise_deg * n / 2))
+    nu, nv = rng.integers(0, n, size=m), rng.integers(0, n, size=m)
+    perm = rng.permutation(n)
+    u, v = perm[np.concatenate([u, nu])], perm[np.concatenate([v, nv])]
+    return _patch_isolated(rng, coalesce_undirected(u, v, n), n)
+
+
 # ----------------------------------------------------------------------------------------
 # the five named workloads
 # ----------------------------------------------------------------------------------------
@@ -274,7 +305,17 @@ def workload(name: str, seed: int = 0, scale: float = 1.0) -> Workload:
         n = max(64, int(12_000 * scale))
         ei = add_self_loops(duplication(n, 0.7, 3, 8, seed), n)
         return Workload("c2", ei, n, 128, True, (0, 8), "normal",
-                        "duplication model keep=0.7 +3 random, A+I normalised")
+                        "duplication model keep=0.7 +3 random, A+I normalised [the stated process, taken literally, yields "
+                        "1.82 M undirected edges at N = 12 000, not the ~240 k the configuration names; c2b is the same "
+                        "process held to that size]")
+    if name == "c2b":
+        # the same process held to the SIZE the configuration names (~240k undirected edges at N = 12 000): a new
+        # node copies from at most 26 entries of its template's list
+        n = max(64, int(12_000 * scale))
+        ei = add_self_loops(duplication(n, 0.7, 3, 8, seed, copy_cap=26), n)
+        return Workload("c2b", ei, n, 128, True, (0, 8), "normal",
+                        "duplication model keep=0.7 +3 random, copying from at most 26 entries of the template's list "
+                        "(~240k undirected edges), A+I normalised")
     if name == "c3":
         n = max(256, int(100_000 * scale))
         ei = add_self_loops(chung_lu_cliques(n, 2.1, 32.0, max(1, int(20_000 * scale)), 4, 12, seed), n)
@@ -295,4 +336,14 @@ def workload(name: str, seed: int = 0, scale: float = 1.0) -> Workload:
         ei = sbm_with_chain(n, blocks, 1.0, 600.0 * min(1.0, scale), chain, 48, seed)
         return Workload("c5", ei, n, 512, False, (0, 2, 4, 8, 16, 32), "normal",
                         "SBM 300 clique blocks (p_in=1) + p_out to mean degree ~600, + 2000-deep staircase chain, plain A")
+    if name == "c6":
+        # outside the five configured workloads: a deep AND wide arborescence with a high compression ratio, the
+        # regime of the reference's best datasets (plot_results_alpha_vs_runtime.py:55,63: ratios 5.9 .. 9.8),
+        # where its tree walk -- serial inside a subtree, cbm_extensions.cpp:1166-1218 -- is the bottleneck
+        chains = max(4, int(800 * scale))
+        ei = add_self_loops(staircases(chains, 100, 28, 2.0, seed))
+        n = chains * 228
+        return Workload("c6", ei, n, 256, True, (0,), "normal",
+                        "800 disjoint staircases (half-graphs) of depth 100 + random edges of mean degree 2, ids shuffled, "
+                        "A+I normalised: ~100 tree levels of ~1 600 rows each")
     raise ValueError(f"unknown workload {name!r}")

@@ -218,6 +218,38 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                   int32_t threads, cbm_tiling* out);
 void cbm_tiling_free(cbm_tiling* t);
 
+/* Plan of the tree walk by SUBTREES (cbm_propagate_subtrees_f32): the rows below level `cut` of the
+ * arborescence, as one sequence per subtree in depth-first pre-order, so that ONE launch walks all of
+ * them -- a wavefront per (bin of subtrees, 64 feature columns) carries a row's value down to its
+ * children in registers and LDS and touches global memory only to read the row's own SpMM result and to
+ * write its final value (two row accesses per tree edge instead of three, none of them dependent on the
+ * previous one).  The reference's walk has the same shape -- parallel over the children of the root,
+ * depth-first with a stack inside a subtree (cbm_extensions.cpp:1166-1218) -- on CPU threads.
+ *   cut        rows of levels 0 .. cut are final before the launch (level 0 after the SpMM, levels 1 .. cut
+ *              by the level-by-level launches); every row of level `cut` that has children heads a task
+ *   entries    [n_entries][2] int32 { row, ctl }: ctl & 63 = where the parent's value is: 0 = the row just
+ *              before this one, 1 .. CBM_WALK_MAX_SLOTS = that LDS slot, CBM_WALK_LOAD_ONLY = this row is a
+ *              task's head: final already, only loaded; (ctl >> 8) & 63 = slot to keep this row's value in
+ *              (0 = none; rows with two or more children).  Children are visited lightest subtree first,
+ *              so at most log2(subtree size) + 1 slots are live at once
+ *   bin_off    [n_bins + 1] offsets into entries: a bin is what one wavefront walks (whole tasks, longest
+ *              first, small ones packed together up to about n_entries / target_bins entries)
+ *   n_slots    most slots any task uses;  longest_bin  entries of the longest bin (the critical path)
+ * HOST pointers; release with cbm_walk_plan_free.  CBM_ERR_UNSUPPORTED if a task needs more than
+ * CBM_WALK_MAX_SLOTS slots (a tree of more than 2^31 rows would). */
+#define CBM_WALK_LOAD_ONLY 63
+#define CBM_WALK_MAX_SLOTS 31
+#define CBM_WALK_MIN_BIN 32
+typedef struct cbm_walk_plan {
+    int32_t n, cut, n_entries, n_bins, n_slots, reserved;
+    int64_t longest_bin;
+    int32_t* entries;
+    int32_t* bin_off;
+} cbm_walk_plan;
+int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32_t* level_off, int32_t n,
+                        int32_t n_levels, int32_t cut, int32_t target_bins, cbm_walk_plan* out);
+void cbm_walk_plan_free(cbm_walk_plan* p);
+
 /* ------------------------------------------------------------------ libcbm_hip.so ----------- */
 
 const char* cbm_version(void);
@@ -335,6 +367,27 @@ int cbm_relayout_slabs_scaled_f32(const float* X_dev, const float* scale_dev, fl
 int cbm_propagate_f32(const int32_t* parent_dev, const int32_t* order_dev, const int32_t* level_off_dev,
                       const int32_t* level_off_host, int32_t n_levels, const float* m_dev, float* Y_dev,
                       int32_t n, int32_t d, int64_t ldy, int32_t flags, void* stream);
+
+/* A walk plan (cbm_walk_plan_build) in DEVICE memory.  The struct itself lives in HOST memory. */
+typedef struct cbm_walk_dev {
+    int32_t cut, n_entries, n_bins, n_slots;
+    const int32_t* entries;     /* [n_entries][2], 8-byte aligned */
+    const int32_t* bin_off;     /* [n_bins + 1] */
+} cbm_walk_dev;
+
+/* cbm_propagate_f32 with the rows below level walk->cut walked by subtrees in one launch: levels
+ * 1 .. cut run level by level as in cbm_propagate_f32, then one wavefront per (bin of the plan, 64 feature
+ * columns) walks its subtrees depth-first.  Per row the arithmetic is that of cbm_propagate_f32, so Y is
+ * bit-identical to it; what changes is the number of dependent launches (cut + 1 instead of one per tree
+ * level) and the traffic (a row's parent value comes from a register or LDS, not from Y).  The plan must
+ * have been built from the same parent / order / level_off.  flags: CBM_PROP_SCALE_ROOTS as in
+ * cbm_propagate_f32; CBM_UPDATE_RELU = one pass Y = max(Y, 0) after the walk.
+ * Replaces the same walks as cbm_propagate_f32 (cbm_extensions.cpp:1166-1218, :1285-1373), whose
+ * parallelisation -- threads over the children of the root, a stack inside each subtree -- it mirrors. */
+int cbm_propagate_subtrees_f32(const cbm_walk_dev* walk, const int32_t* parent_dev, const int32_t* order_dev,
+                               const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
+                               const float* m_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldy, int32_t flags,
+                               void* stream);
 
 /* Y = A_hat * X in one call: cbm_spmm_f32 followed by cbm_propagate_f32 on the same stream.
  * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);

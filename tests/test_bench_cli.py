@@ -44,6 +44,36 @@ def test_traffic_record_lookup():
     assert bench.measured_traffic("no-such-workload", 0, 1) == (None, None, False)
 
 
+def test_launch_count_follows_the_walk_plan():
+    """Copy of X + SpMM, then the walk: one launch per wide level, one per run of narrow levels, one per
+    chain of at least four single-row levels; one launch in all for a small product on a shallow tree; one
+    more than the SpMM's two for a tree the path walk finishes in one launch."""
+    import types
+    import torch
+
+    def fake(widths, tiled=False, cut=False, single=False, paths=False, subtrees=None):
+        lo = torch.tensor([0] + list(__import__("itertools").accumulate(widths)), dtype=torch.int32)
+        return types.SimpleNamespace(level_off=lo, n_levels=len(widths), is_tiled=lambda: tiled, has_cut_rows=lambda: cut,
+                                     _single_launch=lambda n, d: single, _walks_paths=lambda n, d: paths,
+                                     walk_plan=lambda d: ({"cut": subtrees} if subtrees is not None else None))
+
+    assert bench.launches_per_multiply(fake([500]), 500, 64) == 2                         # flat tree
+    assert bench.launches_per_multiply(fake([500], cut=True), 500, 64) == 3               # + adding the pieces
+    assert bench.launches_per_multiply(fake([500, 300, 200]), 1000, 64) == 4              # two wide levels
+    assert bench.launches_per_multiply(fake([500, 300, 200], single=True), 1000, 64) == 1
+    assert bench.launches_per_multiply(fake([500, 300, 200], paths=True), 1000, 64) == 3
+    assert bench.launches_per_multiply(fake([500, 300, 200], paths=True, tiled=True), 1000, 64) == 4
+    # wide, wide, narrow run of three, chain of five, narrow pair (a chain of two is not a chain)
+    assert bench.launches_per_multiply(fake([900, 100, 70, 30, 20, 10, 1, 1, 1, 1, 1, 9, 1, 1]), 2000, 64) == 2 + 2 + 1 + 1 + 1
+    # the walk by subtrees: the levels above its cut level by level, then one launch
+    deep = [900, 100, 70, 30, 20, 10, 1, 1, 1, 1, 1, 9, 1, 1]
+    assert bench.launches_per_multiply(fake(deep, subtrees=0), 2000, 64) == 2 + 1
+    assert bench.launches_per_multiply(fake(deep, subtrees=2), 2000, 64) == 2 + 2 + 1
+    assert bench.launches_per_multiply(fake(deep, subtrees=0, paths=True), 2000, 64) == 2 + 1      # the path walk asks first
+    # a lone narrow level between wide ones is a launch of its own
+    assert bench.launches_per_multiply(fake([900, 100, 7, 100]), 2000, 64) == 2 + 3
+
+
 def test_more_than_one_gpu_is_refused():
     p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120)

@@ -166,13 +166,15 @@ def test_graph_generators_are_pinned():
     import json, os
     with open(os.path.join(os.path.dirname(__file__), "golden", "graph_hashes.json")) as f:
         want = json.load(f)
-    for name in ("c1", "c2", "c3"):
+    for name in ("c1", "c2", "c2b", "c3", "c6"):
         w = graphs.workload(name)
-        assert w.edge_index.shape[1] == want[name]["edges"]
+        assert w.edge_index.shape[1] == want[name]["edges"] and w.n == want[name]["n"]
         assert graphs.edge_hash(w.edge_index) == want[name]["sha256"], name
         if name == "c1":
             from cbm4gnn_amd.utility import check_edge_index
             check_edge_index(torch.from_numpy(w.edge_index).long())
+        if name == "c2b":                       # the size the configuration names: about 240k undirected edges
+            assert abs((w.edge_index.shape[1] - w.n) // 2 - 240_000) < 5_000
 
 
 def test_row_schedule_properties():

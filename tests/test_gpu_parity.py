@@ -401,6 +401,7 @@ def test_deep_chain_uses_the_chain_kernel(orc):
     for normalized, d in ((False, 512), (True, 96), (True, 41), (False, 10), (True, 1100)):
         e2 = graphs.add_self_loops(ei, n) if normalized else ei
         mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
+        mat.subtree_walk = "off"                           # this test is about the level plan's chain kernel
         assert mat.n_levels >= 151
         widths = np.diff(mat.level_off.numpy())
         assert (widths[-120:] == 1).all()
@@ -422,6 +423,7 @@ def test_chain_lengths_around_the_stretch_size(orc):
         for normalized, d in ((False, 96), (True, 41)):
             e2 = graphs.add_self_loops(ei, n) if normalized else ei
             mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
+            mat.subtree_walk = "off"                       # the level plan's chain kernel
             widths = np.diff(mat.level_off.numpy())
             run = int(np.argmax(widths[::-1] != 1)) if (widths != 1).any() else len(widths)
             runs.add(run)
@@ -431,6 +433,157 @@ def test_chain_lengths_around_the_stretch_size(orc):
             want = oracle_product(orc, mat, e2, n, x, normalized)
             assert np.array_equal(got, want)
     assert {33, 64, 65} <= runs and min(runs) < 32 and max(runs) > 90, runs
+
+
+def _walk_graph(kind):
+    if kind == "bushy":
+        n = 900
+        return graphs.sbm(n, 9, 0.4, 0.01, seed=3), n
+    if kind == "chain":
+        n = 1500
+        return graphs.sbm_with_chain(n=n, blocks=24, p_in=1.0, mean_deg=80.0, chain=150, base=48, seed=0), n
+    if kind == "staircases":
+        ei = graphs.staircases(30, 70, 6, 2.0, seed=1)
+        return ei, int(ei.max()) + 1
+    n = 1200
+    return graphs.duplication(n, 0.7, 3, 8, seed=2), n
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+@pytest.mark.parametrize("kind", ["bushy", "chain", "staircases", "duplication"])
+def test_subtree_walk_equals_the_level_walk_and_the_oracle(orc, kind, normalized):
+    """cbm_propagate_subtrees_f32: the rows below a level walked by subtrees in one launch (a wavefront per bin
+    of subtrees and 64 columns, parent values carried in a register / LDS slots).  Per row the arithmetic is
+    that of the level-by-level walk, so the product must be bit-identical to it -- and to the oracle on the
+    product's tree -- for every cut level, width (one to eighteen 64-column slices, ragged last slice,
+    d % 8 != 0 for the division tail) and for trees that are bushy (slots in use), one long chain (bins of
+    more than two stretches), many chains (deep and wide) and a duplication graph."""
+    ei, n = _walk_graph(kind)
+    if normalized:
+        ei = graphs.add_self_loops(ei, n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+    mat.single_launch_max_bytes = 0
+    mat.path_walk_max_bytes = 0
+    assert mat.n_levels >= 3
+    slots = mat._host_walk_plan(0, 64)["n_slots"]
+    assert (slots >= 2) if kind in ("bushy", "duplication") else True
+    mul = mat.omp_mkl_csr_fused_spmm_update if normalized else mat.omp_mkl_csr_spmm_update
+    upd = mat.omp_mkl_csr_fused_update if normalized else mat.omp_mkl_csr_update
+    for d in (1, 19, 64, 100, 256, 1100):
+        x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+        xd = torch.from_numpy(x).cuda()
+        mat.subtree_walk = "off"
+        want = torch.full_like(xd, float("nan")); mul(xd, want)
+        z = torch.empty_like(xd); mat.omp_mkl_csr_spmm(xd, z)            # the SpMM alone, for the update-only calls
+        want_upd = z.clone(); upd(want_upd)
+        if d in (19, 256):
+            assert np.array_equal(want.cpu().numpy(), oracle_product(orc, mat, ei, n, x, normalized))
+        for cut in ("on", 0, 1, mat.n_levels - 2):
+            say("subtree walk", kind, normalized, "d", d, "cut", cut, "levels", mat.n_levels, "slots", slots)
+            mat.subtree_walk = cut
+            plan = mat.walk_plan(d)
+            assert plan is not None and (cut == "on" or plan["cut"] == cut)
+            got = torch.full_like(xd, float("nan")); mul(xd, got)
+            assert torch.equal(got, want)
+            # update-only entry point, in place on a matrix whose rows are further apart than d
+            wide = torch.full((n, d + 5), 3.0, device="cuda")
+            wide[:, :d] = z
+            upd(wide[:, :d])
+            assert torch.equal(wide[:, :d], want_upd) and bool((wide[:, d:] == 3.0).all())
+        if d == 100:                                                     # the ReLU is a pass after the walk
+            relu = torch.full_like(xd, float("nan"))
+            mat._run_spmm_update(xd, relu, use_m=normalized, relu=True)
+            assert float(want.min()) < 0 and torch.equal(relu, want.clamp_min(0.0))
+    # the automatic choice follows the cost estimate; deep trees take the subtree walk
+    mat.subtree_walk = "auto"
+    auto = mat.walk_plan(256)
+    if mat.n_levels > 16:
+        assert auto is not None
+    if auto is not None:
+        assert mat._subtree_plan_cost_us(auto, 256) <= 0.8 * mat._level_plan_cost_us(256)
+
+
+def test_subtree_walk_on_hand_made_trees(orc):
+    """Trees the builder rarely produces, through the C ABI alone: a complete binary tree (a slot per level of
+    the path), a random recursive tree (bushy, ~20 levels) and a caterpillar (a long spine with a leaf at
+    every row: every row keeps its value for one child) -- plan from cbm_walk_plan_build, walk by
+    cbm_propagate_subtrees_f32, against cbm_propagate_f32 on the same arrays and the oracle's walk."""
+    from cbm4gnn_amd.cbm import tree_levels
+    lib, host = _lib.hip_lib(), _lib.host_lib()
+    rng = np.random.default_rng(5)
+    trees = {}
+    n = 2047
+    trees["binary"] = np.concatenate([[-1], (np.arange(1, n) - 1) // 2])
+    n = 5000
+    par = np.full(n, -1, np.int64)
+    par[40:] = (rng.random(n - 40) * np.arange(40, n)).astype(np.int64)          # 40 children of the root
+    trees["recursive"] = par
+    n = 1201
+    par = np.full(n, -1, np.int64)
+    par[1:601] = np.arange(0, 600)                                                # spine 0 .. 600
+    par[601:] = np.arange(0, 600)                                                 # a leaf at every spine row
+    trees["caterpillar"] = par
+    p = lambda t: C.c_void_p(t.data_ptr())
+    for name, par in trees.items():
+        n = par.shape[0]
+        kids = [[] for _ in range(n + 1)]
+        for v in range(n):
+            kids[n if par[v] < 0 else par[v]].append(v)
+        mst_col = np.array(sum(kids, []), np.int32)
+        mst_row = np.concatenate([[0], np.cumsum([len(k) for k in kids])]).astype(np.int32)
+        parent, order, level_off = (torch.from_numpy(a) for a in tree_levels(mst_row, mst_col))
+        levels = level_off.numel() - 1
+        m = (rng.random(n).astype(np.float32) + 0.5)
+        for d, norm in ((72, True), (130, False)):
+            z = rng.standard_normal((n, d)).astype(np.float32)
+            want = (orc.update_fused(mst_row, mst_col, m, z.copy()) if norm else orc.update_plain(mst_row, mst_col, z.copy()))
+            md = torch.from_numpy(m).cuda() if norm else None
+            dev = [t.cuda() for t in (parent, order, level_off)]
+            flags = _lib.CBM_PROP_SCALE_ROOTS if norm else 0
+            y0 = torch.from_numpy(z).cuda()
+            assert lib.cbm_propagate_f32(p(dev[0]), p(dev[1]), p(dev[2]), p(level_off), levels, p(md) if norm else None, p(y0),
+                                         n, d, d, flags, None) == 0
+            assert np.array_equal(y0.cpu().numpy(), want)
+            for cut in (0, 2):
+                plan = _lib.CbmWalkPlan()
+                assert host.cbm_walk_plan_build(p(parent), p(order), p(level_off), n, levels, cut, 64, C.byref(plan)) == 0
+                say("hand-made tree", name, "d", d, norm, "cut", cut, "levels", levels, "slots", plan.n_slots, "bins", plan.n_bins)
+                if name == "binary":
+                    assert plan.n_slots >= levels - 2 - cut
+                ent = torch.from_numpy(np.ctypeslib.as_array(plan.entries, shape=(2 * plan.n_entries,)).copy()).cuda()
+                off = torch.from_numpy(np.ctypeslib.as_array(plan.bin_off, shape=(plan.n_bins + 1,)).copy()).cuda()
+                w = _lib.CbmWalkDev(plan.cut, plan.n_entries, plan.n_bins, plan.n_slots, ent.data_ptr(), off.data_ptr())
+                host.cbm_walk_plan_free(C.byref(plan))
+                y = torch.from_numpy(z).cuda()
+                assert lib.cbm_propagate_subtrees_f32(C.byref(w), p(dev[0]), p(dev[1]), p(dev[2]), p(level_off), levels,
+                                                      p(md) if norm else None, p(y), n, d, d, flags, None) == 0
+                assert torch.equal(y, y0), (name, d, norm, cut)
+
+
+def test_subtree_walk_status_codes():
+    lib = _lib.hip_lib()
+    ei = graphs.add_self_loops(graphs.staircases(8, 20, 6, 2.0, seed=4))
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=True)
+    n, d = mat.num_rows, 64
+    y = torch.zeros((n, d), device="cuda")
+    st = mat._device_arrays(y.device)
+    plan = mat._host_walk_plan(0, d)
+    good = mat._walk_struct(st, plan)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    call = lambda w, flags=0, levels=mat.n_levels: lib.cbm_propagate_subtrees_f32(
+        C.byref(w) if w is not None else None, p(st["parent"]), p(st["order"]), p(st["level_off"]), p(mat.level_off), levels,
+        p(st["m"]), p(y), n, d, d, flags, None)
+    say("subtree walk status codes")
+    assert call(good) == 0
+    assert call(None) == _lib.CBM_ERR_NULL
+    assert call(good, flags=64) == 6                                     # unknown flag
+    bad = _lib.CbmWalkDev(mat.n_levels, good.n_entries, good.n_bins, good.n_slots, good.entries, good.bin_off)
+    assert call(bad) == _lib.CBM_ERR_SHAPE                               # cut beyond the last level
+    bad = _lib.CbmWalkDev(0, good.n_entries, good.n_bins, 40, good.entries, good.bin_off)
+    assert call(bad) == _lib.CBM_ERR_SHAPE                               # more slots than a wavefront has
+    bad = _lib.CbmWalkDev(0, good.n_entries, good.n_bins, good.n_slots, None, good.bin_off)
+    assert call(bad) == _lib.CBM_ERR_NULL
+    torch.cuda.synchronize()
 
 
 def test_strided_rows_and_cpu_staging(orc):
