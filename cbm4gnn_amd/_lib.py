@@ -19,6 +19,8 @@ CBM_UPDATE_RELU = 2
 CBM_UPDATE_WORKSPACE_READY = 4
 CBM_SPMM_WORKSPACE_PRESCALED = 4
 CBM_UPDATE_WORKSPACE_PRESCALED = 8
+CBM_SPMM_SCHED_BATCHED = 8
+CBM_UPDATE_SCHED_BATCHED = 16
 CBM_ERR_NULL = 1
 CBM_ERR_SHAPE = 3
 CBM_ERR_SCRATCH = 7
@@ -94,6 +96,7 @@ HOST_SYMBOLS = {
     "cbm_format_free": (None, [C.POINTER(CbmFormat)]),
     "cbm_build_host_timings": (None, [C.POINTER(C.c_double)]),
     "cbm_schedule_rows": (C.c_int, [_P, _P, _P, _I32, _P]),
+    "cbm_schedule_rows_batched": (C.c_int, [_P, _P, _P, _I32, _I32, _P]),
     "cbm_schedule_split_count": (C.c_int64, [_P, _I32, _I32, C.POINTER(C.c_int32)]),
     "cbm_schedule_rows_split": (C.c_int, [_P, _P, _P, _I32, _I32, _P, _P]),
     "cbm_schedule_blocks_count": (C.c_int64, [_P, _P, _I32, _I32, _I32, C.POINTER(C.c_int32)]),

@@ -120,13 +120,25 @@ def _ld(t):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
 
 
-def schedule_rows(rowptr, parent=None, m=None):
+# Rows of at most this many delta entries are summed a batch at a time by the slab kernel (8 rows per
+# wavefront, each lane group a row of its own, entries in order): ``cbm_schedule_rows_batched``.  0 = never.
+DEFAULT_BATCH_ROWS = 16
+
+
+def schedule_rows(rowptr, parent=None, m=None, batch=0):
     """Row schedule of the SpMM kernels (``cbm_schedule_rows``): int32 tensor [n, 4] holding
-    {start, end, row, bits(left scale)} per row, longest rows first."""
+    {start, end, row, bits(left scale)} per row, longest rows first.  ``batch`` > 0: the schedule of
+    ``cbm_schedule_rows_batched`` -- rows of at most ``batch`` entries last, to be summed a batch at a time --
+    as an [n + 1, 4] tensor whose last descriptor is the trailer (pass it with ``CBM_SPMM_SCHED_BATCHED``)."""
     rowptr = rowptr.to("cpu", torch.int32).contiguous()
     n = rowptr.numel() - 1
     parent = None if parent is None else parent.to("cpu", torch.int32).contiguous()
     m = None if m is None else m.to("cpu", torch.float32).contiguous()
+    if batch:
+        out = torch.empty((n + 1, 4), dtype=torch.int32)
+        rc = _lib.host_lib().cbm_schedule_rows_batched(_ptr(rowptr), _ptr(parent), _ptr(m), n, int(batch), _ptr(out))
+        _lib.check(rc, "cbm_schedule_rows_batched")
+        return out
     out = torch.empty((n, 4), dtype=torch.int32)
     rc = _lib.host_lib().cbm_schedule_rows(_ptr(rowptr), _ptr(parent), _ptr(m), n, _ptr(out))
     _lib.check(rc, "cbm_schedule_rows")
@@ -570,6 +582,7 @@ class cbm_matrix:
         # per level; "on" / "off" force it; an integer forces it with that cut level.
         self.subtree_walk = "auto"
         self._walk_plans = {}
+        self._batch_rows = DEFAULT_BATCH_ROWS
 
     def _path_gather_ratio(self):
         """(sum over rows of the delta entries on the row's ancestor path, itself included) / nnz: the extra
@@ -798,6 +811,21 @@ class cbm_matrix:
         self._stream_coefficients = bool(value)
 
     @property
+    def batch_rows(self):
+        """Rows of at most this many delta entries are summed a batch at a time by the slab kernel, each lane
+        group a row of its own, entries strictly in order (``cbm_schedule_rows_batched``); 0 = every row is
+        summed by a whole wavefront."""
+        return self._batch_rows
+
+    @batch_rows.setter
+    def batch_rows(self, value):
+        if not 0 <= int(value) <= 64:
+            raise ValueError("batch_rows must be 0 .. 64")
+        if int(value) != self._batch_rows:
+            self._dev = {}
+        self._batch_rows = int(value)
+
+    @property
     def col_multiplier(self):
         return self._col_multiplier
 
@@ -889,8 +917,8 @@ class cbm_matrix:
                 "m": self.col_multiplier.to(device) if self.col_multiplier is not None else None,
                 "coef": None,
                 # row schedules (longest rows first): without and with the left scale of root children
-                "sched": schedule_rows(self.rowptr, None, None).to(device),
-                "sched_scaled": (schedule_rows(self.rowptr, self.parent, self.col_multiplier).to(device)
+                "sched": schedule_rows(self.rowptr, None, None, self.batch_rows).to(device),
+                "sched_scaled": (schedule_rows(self.rowptr, self.parent, self.col_multiplier, self.batch_rows).to(device)
                                  if self.col_multiplier is not None else None),
             }
             th = self._host_tiling()
@@ -1017,7 +1045,8 @@ class cbm_matrix:
         # per-entry coefficients are only read when the multiply does not scale its own copy of X
         coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
         flags = (_lib.CBM_SPMM_WORKSPACE_READY if workspace_ready else 0) | \
-                (_lib.CBM_SPMM_WORKSPACE_PRESCALED if workspace_prescaled else 0)
+                (_lib.CBM_SPMM_WORKSPACE_PRESCALED if workspace_prescaled else 0) | \
+                (_lib.CBM_SPMM_SCHED_BATCHED if self.batch_rows else 0)
         with torch.cuda.device(xd.device):
             rc = _lib.hip_lib().cbm_spmm_f32(
                 _ptr(st["rowptr"]), _ptr(st["idx"]), self.nnz, _ptr(st["m"]) if use_m else None,
@@ -1120,6 +1149,8 @@ class cbm_matrix:
                 y.copy_(yd)
             return
         coef = self._coef(st, xd.device) if (use_m and (ws is None or (workspace_ready and not workspace_prescaled))) else None
+        if self.batch_rows:
+            flags |= _lib.CBM_UPDATE_SCHED_BATCHED
         if self._walks_paths(n, x.size(1)):
             zs = torch.empty(_lib.hip_lib().cbm_spmm_update_paths_scratch_floats(n, x.size(1), self.n_levels),
                              dtype=torch.float32, device=xd.device)
@@ -1301,7 +1332,8 @@ def csr_spmm(rowptr, col, val, x, y, sched=None):
     """Plain CSR SpMM ``y = A @ x`` on the GPU: the hand-written baseline the CBM multiply is
     measured against (role of ``omp_s_spmm_csr_int32``, ``cbm_extensions.cpp:1707-1755``).
     ``rowptr`` [N+1] / ``col`` int32 device tensors, ``val`` fp32 or None (all ones); ``sched``:
-    optional device copy of ``schedule_rows(rowptr)`` (same scheduling as the CBM kernels)."""
+    optional device copy of ``schedule_rows(rowptr)`` or ``schedule_rows(rowptr, batch=...)`` (same
+    scheduling as the CBM kernels, short rows in batches included)."""
     n = rowptr.numel() - 1
     _check_f32_matrix(x, "rhs")
     _check_f32_matrix(y, "dst", n)
@@ -1312,7 +1344,13 @@ def csr_spmm(rowptr, col, val, x, y, sched=None):
     if not (x.is_cuda and y.is_cuda and rowptr.is_cuda and col.is_cuda):
         raise ValueError("csr_spmm expects device tensors")
     ws = _workspace(x, y, col.numel())
+    flags = 0
+    if sched is not None:
+        if tuple(sched.shape) == (n + 1, 4):
+            flags = _lib.CBM_SPMM_SCHED_BATCHED
+        elif tuple(sched.shape) != (n, 4):
+            raise ValueError("sched must be schedule_rows(rowptr) ([n, 4]) or its batched form ([n + 1, 4])")
     with torch.cuda.device(x.device):
         rc = _lib.hip_lib().csr_spmm_f32(_ptr(rowptr), _ptr(col), col.numel(), _ptr(val), _ptr(sched), _ptr(x), _ptr(y), _ptr(ws),
-                                         0, n, x.size(1), _ld(x), _ld(y), _stream(x.device))
+                                         flags, n, x.size(1), _ld(x), _ld(y), _stream(x.device))
     _lib.check(rc, "csr_spmm_f32")

@@ -668,6 +668,41 @@ int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float*
     }
 }
 
+int cbm_schedule_rows_batched(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
+                              int32_t batch_max_entries, int32_t* sched_out) {
+    if (!rowptr || !sched_out) return CBM_ERR_NULL;
+    if (n < 0 || batch_max_entries < 0 || batch_max_entries > 64) return CBM_ERR_SHAPE;
+    try {
+        // sort key, descending, stable: rows above the limit by their 64-entry gather rounds (as
+        // cbm_schedule_rows), then the rows of at most `limit` entries by their 8-entry chunks, empty rows last
+        const int32_t T = batch_max_entries;
+        std::vector<int32_t> key(n);
+        int32_t max_key = 0;
+        int64_t n_wide = 0;
+        for (int32_t r = 0; r < n; r++) {
+            const int32_t len = rowptr[r + 1] - rowptr[r];
+            if (len < 0) return CBM_ERR_SHAPE;
+            if (len > T) { key[r] = 9 + (len + 63) / 64; n_wide++; }
+            else key[r] = (len + 7) / 8;                    // 0 .. 8
+            max_key = std::max(max_key, key[r]);
+        }
+        std::vector<int64_t> first(max_key + 2, 0);
+        for (int32_t r = 0; r < n; r++) first[max_key - key[r] + 1]++;
+        for (int32_t b = 0; b <= max_key; b++) first[b + 1] += first[b];
+        for (int32_t r = 0; r < n; r++) {
+            int32_t* o = sched_out + 4 * first[max_key - key[r]]++;
+            const float scale = (m && parent && parent[r] < 0) ? m[r] : 1.0f;
+            o[0] = rowptr[r]; o[1] = rowptr[r + 1]; o[2] = r;
+            std::memcpy(&o[3], &scale, sizeof(float));
+        }
+        int32_t* t = sched_out + 4 * (int64_t)n;            // the trailer
+        t[0] = (int32_t)n_wide; t[1] = T; t[2] = CBM_SCHED_BATCH_MAGIC; t[3] = 0;
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        return CBM_ERR_ALLOC;
+    }
+}
+
 int64_t cbm_schedule_blocks_count(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t chunk, int32_t col_blocks,
                                   int32_t* n_long_out) {
     if (!rowptr || n < 0 || (chunk != 0 && chunk < 64) || col_blocks < 0 || (col_blocks >= 2 && !idx && n > 0 && rowptr[n] > 0))

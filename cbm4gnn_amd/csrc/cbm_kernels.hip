@@ -347,7 +347,10 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
     const int32_t* __restrict__ rowptr, const int4* __restrict__ sched, const uint32_t* __restrict__ idx,
     const float* __restrict__ val, const float* __restrict__ m, const int32_t* __restrict__ parent,
     const float* __restrict__ X, float* __restrict__ Z, int n, int d, int vec_out, int n_slabs,
-    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz, int relu, float* __restrict__ partials) {
+    int64_t x_slab_stride, int64_t x_row_stride, int64_t ldz, int relu, float* __restrict__ partials, int batched) {
+    // batched: the schedule comes from cbm_schedule_rows_batched -- descriptor n is a trailer whose first word
+    // says how many descriptors are walked one row per wavefront; the rows behind them are short and taken
+    // kStep at a time, one per lane group (below).
     // n is the number of row descriptors (rows of the matrix, unless the schedule cuts long rows
     // into pieces: a descriptor whose row field has CBM_SCHED_PIECE set is a piece, and its sum goes
     // to slot (row field & ~CBM_SCHED_PIECE) of `partials`, n_slabs x 32 floats per slot, unscaled).
@@ -381,6 +384,7 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
             slab0 = xcd % n_slabs; slab_step = n_slabs;      // a single slab for this XCD
         }
     }
+    const int n_wide = batched ? __builtin_amdgcn_readfirstlane(sched[n].x) : n;
     for (int slab = slab0; slab < n_slabs; slab += slab_step) {
         const float* __restrict__ Xs = X + slab * x_slab_stride + li * 4;
         float* __restrict__ Zs = Z + slab * kSlab + li * 4;
@@ -396,14 +400,14 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
         };
         int i = first;
         int4 nxt = make_int4(0, 0, 0, 0);
-        if (i < n) nxt = fetch(i);
-        while (i < n) {
+        if (i < n_wide) nxt = fetch(i);
+        while (i < n_wide) {
             const int start = __builtin_amdgcn_readfirstlane(nxt.x);
             const int end = __builtin_amdgcn_readfirstlane(nxt.y);
             const int row = __builtin_amdgcn_readfirstlane(nxt.z);
             const float row_scale = __int_as_float(__builtin_amdgcn_readfirstlane(nxt.w));
             i += stride;
-            if (i < n) nxt = fetch(i);
+            if (i < n_wide) nxt = fetch(i);
 
             float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             // One gather round = UU instructions of kStep entries each.  Every load of a round is
@@ -473,6 +477,63 @@ __global__ __launch_bounds__(kWave * kWavesPerBlock) void spmm_slab_per_xcd(
 #pragma unroll
                     for (int e = 0; e < 4; e++)
                         if (col + e < d) zr[e] = acc[e];
+                }
+            }
+        }
+        // Short rows, a batch of kStep at a time: lane group `sub` owns row n_wide + b * kStep + sub of the
+        // schedule and sums it alone, LPE entries per chunk -- its LPE lanes fetch one index each, every lane
+        // then gathers all LPE rows of X (its own float4 of each) and adds them strictly in entry order.  The
+        // groups of a wavefront walk in lockstep up to the longest row of the batch (the schedule sorts the
+        // short rows by chunk count); entries past a row's end are clamped and get coefficient 0.  No sum
+        // crosses lanes, and one round of loads serves kStep rows.
+        for (int b = first; b * kStep < n - n_wide; b += stride) {
+            const int di = n_wide + b * kStep + sub;
+            const int4 dsc = di < n ? sched[di] : make_int4(0, 0, -1, 0);
+            const int start = dsc.x, len = dsc.y - dsc.x;
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int c = 0; __builtin_amdgcn_ballot_w64(c < len) != 0; c += LPE) {
+                const int kc = max(min(start + c + li, dsc.y - 1), 0);
+                const uint32_t p_all = idx[kc];
+                float f_all = 0.0f;
+                if constexpr (COEF == kCoefStream) f_all = val[kc];
+                uint32_t p[LPE];
+                float f[LPE];
+                float x[LPE][4];
+#pragma unroll
+                for (int e = 0; e < LPE; e++) {
+                    p[e] = __shfl(p_all, lane - li + e, kWave);
+                    if constexpr (COEF == kCoefStream) f[e] = __shfl(f_all, lane - li + e, kWave);
+                }
+#pragma unroll
+                for (int e = 0; e < LPE; e++) {
+                    const uint32_t col = p[e] & 0x7fffffffu;
+                    if constexpr (COEF != kCoefStream) {
+                        const uint32_t mag = COEF == kCoefSignM ? __float_as_uint(m[col]) : 0x3f800000u;
+                        f[e] = __uint_as_float(mag ^ (p[e] & 0x80000000u));
+                    }
+                    f[e] = c + e < len ? f[e] : 0.0f;
+                    load_vec<4>(Xs + (int64_t)col * x_row_stride, x[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < LPE; e++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) acc[q] = fmaf(f[e], x[e][q], acc[q]);
+            }
+            if (dsc.z >= 0) {
+                const float row_scale = __int_as_float(dsc.w);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    acc[q] *= row_scale;
+                    if (relu) acc[q] = acc[q] < 0.0f ? 0.0f : acc[q];
+                }
+                const int col = slab * kSlab + li * 4;
+                float* __restrict__ zr = Zs + (int64_t)dsc.z * ldz;
+                if (vec_out) {
+                    if (col < d) store_vec<4>(zr, acc);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (col + q < d) zr[q] = acc[q];
                 }
             }
         }
@@ -1590,8 +1651,12 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
                 const int32_t* parent, const int32_t* sched, const float* X, float* Z, float* workspace,
                 int32_t flags, int32_t n, int32_t d, int64_t ldx, int64_t ldz, hipStream_t s, int32_t n_desc = 0,
                 float* partials = nullptr, int32_t n_pieces = 0) {
-    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED)) return CBM_ERR_UNSUPPORTED;
+    if (flags & ~(CBM_SPMM_WORKSPACE_READY | CBM_SPMM_RELU | CBM_SPMM_WORKSPACE_PRESCALED | CBM_SPMM_SCHED_BATCHED))
+        return CBM_ERR_UNSUPPORTED;
     const int relu = (flags & CBM_SPMM_RELU) ? 1 : 0;
+    // a batched schedule: n + 1 descriptors; rows cut into pieces have their own kind of schedule
+    const int batched = (flags & CBM_SPMM_SCHED_BATCHED) ? 1 : 0;
+    if (batched && (!sched || n_desc > 0)) return CBM_ERR_UNSUPPORTED;
     if ((flags & CBM_SPMM_WORKSPACE_PRESCALED) && (!PACKED || !m || !(flags & CBM_SPMM_WORKSPACE_READY)))
         return CBM_ERR_UNSUPPORTED;                       // only a ready copy of a normalised multiply can be pre-scaled
     if ((!rowptr && !sched) || !X || !Z) return CBM_ERR_NULL;
@@ -1647,7 +1712,8 @@ int launch_spmm(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const f
             const int vec_out = (plan.vec_out && aligned(Zl, 16)) ? 1 : 0;
 #define LAUNCH_SLAB(LL, CF, UU)                                                                                  \
     hipLaunchKernelGGL((spmm_slab_per_xcd<LL, PACKED, CF, UU>), grid, block, 0, s, rowptr, sc, idx, val, m, parent, \
-                       Xl, Zl, n_rows, d_l, vec_out, slabs, slab_stride, row_stride, ldz, relu, partials_l)
+                       Xl, Zl, n_rows, d_l, vec_out, slabs, slab_stride, row_stride, ldz, relu, partials_l,             \
+                       (batched && nnz > 0) ? 1 : 0)
             switch (L * 4 + coef_mode) {
                 case 8 * 4 + kCoefStream: LAUNCH_SLAB(8, kCoefStream, CBM_SLAB_ROUNDS); break;
                 case 8 * 4 + kCoefSign: LAUNCH_SLAB(8, kCoefSign, CBM_SLAB_ROUNDS); break;
@@ -1999,7 +2065,8 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
                         const int32_t* level_off_host, int32_t n_levels, const float* X, float* Y, float* workspace,
                         int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
     if (!parent) return CBM_ERR_NULL;
-    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED |
+                  CBM_UPDATE_SCHED_BATCHED))
         return CBM_ERR_UNSUPPORTED;
     if (X == Y) return CBM_ERR_SHAPE;                    // the SpMM overwrites Y while gathering X
     const bool relu = (flags & CBM_UPDATE_RELU) != 0;
@@ -2009,6 +2076,7 @@ int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz,
     const bool flat = n_levels <= 1;
     int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
     if (flags & CBM_UPDATE_WORKSPACE_PRESCALED) spmm_flags |= CBM_SPMM_WORKSPACE_PRESCALED;
+    if (flags & CBM_UPDATE_SCHED_BATCHED) spmm_flags |= CBM_SPMM_SCHED_BATCHED;
     if (relu && flat) spmm_flags |= CBM_SPMM_RELU;
     int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, Y, workspace, spmm_flags, n, d, ldx, ldy,
                           stream);
@@ -2032,7 +2100,8 @@ int cbm_spmm_update_paths_f32(const int32_t* rowptr, const uint32_t* idx, int64_
                                    n_levels, X, Y, workspace, n, d, ldx, ldy, flags, stream);
     if (!parent || !z_scratch || !Y) return CBM_ERR_NULL;
     if (X == Y) return CBM_ERR_SHAPE;                    // as cbm_spmm_update_f32
-    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED))
+    if (flags & ~(CBM_PROP_SCALE_ROOTS | CBM_UPDATE_RELU | CBM_UPDATE_WORKSPACE_READY | CBM_UPDATE_WORKSPACE_PRESCALED |
+                  CBM_UPDATE_SCHED_BATCHED))
         return CBM_ERR_UNSUPPORTED;
     if (int rc = check_matrix(n, d, ldy)) return rc;
     if (int rc = validate_levels(level_off_host, n_levels, n)) return rc;
@@ -2045,6 +2114,7 @@ int cbm_spmm_update_paths_f32(const int32_t* rowptr, const uint32_t* idx, int64_
         return CBM_ERR_SHAPE;
     int spmm_flags = (flags & CBM_UPDATE_WORKSPACE_READY) ? CBM_SPMM_WORKSPACE_READY : 0;
     if (flags & CBM_UPDATE_WORKSPACE_PRESCALED) spmm_flags |= CBM_SPMM_WORKSPACE_PRESCALED;
+    if (flags & CBM_UPDATE_SCHED_BATCHED) spmm_flags |= CBM_SPMM_SCHED_BATCHED;
     // children of the root are scaled by the SpMM epilogue: their rows of the scratch are final
     if (int rc = cbm_spmm_f32(rowptr, idx, nnz, m, coef, parent, row_sched, X, z_scratch, workspace, spmm_flags, n, d, ldx,
                               ldz, stream))

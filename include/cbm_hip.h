@@ -45,8 +45,9 @@ enum {
 enum {
     CBM_SPMM_WORKSPACE_READY = 1, /* workspace already holds cbm_relayout_slabs_f32(X): do not copy again */
     CBM_SPMM_RELU = 2,            /* store max(z, 0) instead of z (after the left scale of root children) */
-    CBM_SPMM_WORKSPACE_PRESCALED = 4 /* with WORKSPACE_READY, cbm_spmm_f32 with m only: the copy was made by
+    CBM_SPMM_WORKSPACE_PRESCALED = 4, /* with WORKSPACE_READY, cbm_spmm_f32 with m only: the copy was made by
                                      cbm_relayout_slabs_scaled_f32(X, m) (or the masked variant with m) */
+    CBM_SPMM_SCHED_BATCHED = 8    /* row_sched comes from cbm_schedule_rows_batched (n + 1 descriptors) */
 };
 
 /* flags of cbm_propagate_f32 */
@@ -62,7 +63,8 @@ enum {
                                        separate pass); in the SpMM epilogue when the tree is flat,
                                        one extra pass over Y otherwise */
     CBM_UPDATE_WORKSPACE_READY = 4, /* as CBM_SPMM_WORKSPACE_READY */
-    CBM_UPDATE_WORKSPACE_PRESCALED = 8 /* as CBM_SPMM_WORKSPACE_PRESCALED */
+    CBM_UPDATE_WORKSPACE_PRESCALED = 8, /* as CBM_SPMM_WORKSPACE_PRESCALED */
+    CBM_UPDATE_SCHED_BATCHED = 16   /* as CBM_SPMM_SCHED_BATCHED */
 };
 
 /* The CBM format as built on the host.  All arrays are malloc'd by cbm_build_host and are
@@ -152,6 +154,21 @@ void cbm_build_host_timings(double* out4);
  * No reference counterpart: MKL keeps its own scheduling inside mkl_sparse_s_mm. */
 int cbm_schedule_rows(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
                       int32_t* sched_out);
+
+/* cbm_schedule_rows for matrices with many SHORT rows -- the delta rows of a matrix that compresses well
+ * hold a handful of entries each.  Rows of more than batch_max_entries entries (at most 64) come first, in
+ * the order of cbm_schedule_rows; the others follow, sorted by descending number of 8-entry chunks (stable),
+ * and the slab kernel takes them a BATCH at a time: every lane group of a wavefront (8 rows per wavefront on
+ * 128-byte slabs) sums a row of its own, entries strictly in order, so that one index load and one round of
+ * gathers serve 8 rows instead of one and no sum is reduced across lanes.  sched_out holds 4 * (n + 1)
+ * int32: the n descriptors and a trailer { rows before the batched part, batch_max_entries,
+ * CBM_SCHED_BATCH_MAGIC, 0 }; pass it with CBM_SPMM_SCHED_BATCHED (CBM_UPDATE_SCHED_BATCHED).  The fp32
+ * order of a batched row is the in-order sum (as if cbm_spmm_summation_groups were 1 for that row) wherever
+ * the slab kernel runs; other kernels walk the same descriptors and ignore the trailer.  HOST pointers.
+ * No reference counterpart (MKL schedules rows internally). */
+#define CBM_SCHED_BATCH_MAGIC 0x62617463
+int cbm_schedule_rows_batched(const int32_t* rowptr, const int32_t* parent, const float* m, int32_t n,
+                              int32_t batch_max_entries, int32_t* sched_out);
 
 /* cbm_schedule_rows for matrices with very long rows (hubs of a power-law graph): a row with more
  * than `chunk` entries (chunk >= 64) is cut into pieces of `chunk` entries, each with a descriptor

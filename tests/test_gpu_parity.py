@@ -45,11 +45,16 @@ def tail_for(d, ld=None, workspace=False):
     return int(_lib.hip_lib().cbm_spmm_tail_columns(d, ld, ld, C.c_void_p(256), C.c_void_p(256), int(workspace)))
 
 
-def grouped_spmm(orc, rp, col, val, xs, groups, tail=0, threads=1):
-    """``orc.csr_spmm`` in ``groups`` interleaved partial sums, the last ``tail`` columns in 16."""
+def grouped_spmm(orc, rp, col, val, xs, groups, tail=0, threads=1, seq_upto=0):
+    """``orc.csr_spmm`` in ``groups`` interleaved partial sums, the last ``tail`` columns in 16; rows of at
+    most ``seq_upto`` entries strictly in order where the others are not (the slab kernel sums such rows a
+    batch at a time, every lane group a row of its own: ``cbm_schedule_rows_batched``)."""
     y = orc.csr_spmm(rp, col, val, xs, threads=threads, groups=groups)
     if tail and groups != 16:
         y[:, xs.shape[1] - tail:] = orc.csr_spmm(rp, col, val, xs, threads=threads, groups=16)[:, xs.shape[1] - tail:]
+    if seq_upto and groups > 1:
+        short = np.diff(np.asarray(rp, np.int64)) <= seq_upto
+        y[short] = orc.csr_spmm(rp, col, val, xs, threads=threads, groups=1)[short]
     return y
 
 
@@ -94,10 +99,11 @@ def oracle_product(orc, mat, ei, n, x, normalized, threads=4, groups=None, presc
     if prescaled:
         xs = (m[:, None] * x).astype(np.float32)
         z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), xs, g, tail,
-                         threads)
+                         threads, seq_upto=mat.batch_rows)
         return orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads)
     val = sign.numpy() * (m[col.numpy()] if normalized else np.float32(1))
-    z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32), x, g, tail, threads)
+    z = grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val.astype(np.float32), x, g, tail, threads,
+                     seq_upto=mat.batch_rows)
     return (orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z, threads) if m is None
             else orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z, threads))
 
@@ -196,13 +202,14 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         rp = np.concatenate([[0], np.cumsum(np.bincount(lr, minlength=n))]).astype(np.int32)
         return remote + orc.csr_spmm(rp, lc[order].astype(np.int32), ls[order], xs, groups=1)
     if not normalized:
-        return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, g, tail)
+        return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32), x, g, tail,
+                            seq_upto=mat.batch_rows)
     m = orc.col_multiplier(ei, n)
     if brings_workspace(mat.relayout, mat.nnz, n, d) and g > 1:      # the copy of X is scaled by m
         return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), sign.numpy().astype(np.float32),
-                            (m[:, None] * x).astype(np.float32), g, tail)
+                            (m[:, None] * x).astype(np.float32), g, tail, seq_upto=mat.batch_rows)
     val = (sign.numpy() * m[col.numpy()]).astype(np.float32)
-    return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, g, tail)
+    return grouped_spmm(orc, mat.rowptr.numpy(), col.numpy().astype(np.int32), val, x, g, tail, seq_upto=mat.batch_rows)
 
 
 TILED_FUSED = True            # state of cbm_set_tiled_fused (the library's default), for the oracle's order
@@ -317,6 +324,67 @@ def test_workloads_against_oracle(orc, name, scale, alphas, spmm_kernel):
         assert orc.max_rel_err(yd.cpu().numpy(), csr) <= 1e-5
         g = groups_for(x.shape[1], workspace=brings_workspace(True, ei.shape[1], w.n, x.shape[1]))
         assert np.array_equal(yd.cpu().numpy(), csr if g == 1 else orc.csr_spmm(rp, ei[1][order], vals, x, threads=4, groups=g))
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+@pytest.mark.parametrize("kind", ["staircases", "sbm"])
+def test_short_rows_summed_in_batches(orc, kind, normalized):
+    """cbm_schedule_rows_batched + CBM_SPMM_SCHED_BATCHED: rows of at most ``batch_rows`` entries are summed by
+    one lane group each, several rows per wavefront, entries strictly in order.  Against the oracle in that
+    order, bit for bit, for every limit (0 = off, 8 = one chunk, 16, 64 = every row of these graphs' short
+    part in up to 8 chunks), on 128-byte slabs from the copy, the 64-byte half slab (d = 41), 128- and
+    256-byte slabs gathered in place (d = 64 / 512 without a copy), with streamed, sign-only and gathered
+    coefficients; the CSR baseline takes the same schedules."""
+    if kind == "staircases":
+        ei = graphs.staircases(30, 70, 6, 2.0, seed=1)           # most delta rows hold 1 .. 6 entries
+        n = int(ei.max()) + 1
+    else:
+        n = 700
+        ei = graphs.sbm(n, 10, 0.3, 0.01, seed=5)                  # delta rows of 10 .. 40 entries
+    if normalized:
+        ei = graphs.add_self_loops(ei, n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0 if kind == "staircases" else 1, normalized=normalized)
+    mat.single_launch_max_bytes = 0
+    lens = np.diff(mat.rowptr.numpy())
+    assert (lens > 8).any() and ((lens <= 8).any() if kind == "staircases" else (lens <= 64).all())
+    for d in (41, 64, 100, 256, 512):
+        x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+        results = {}
+        for limit in (0, 8, 16, 64):
+            for relayout in (True, False):
+                mat.batch_rows, mat.relayout = limit, relayout
+                if not relayout and mat_groups(mat, d) == 1:
+                    continue                                       # one wavefront per row: no slabs, no batches
+                for stream in ((True, False) if (normalized and not relayout) else (True,)):
+                    mat.stream_coefficients = stream
+                    say("batched rows", kind, normalized, "d", d, "limit", limit, "copy", relayout, "stream", stream)
+                    got = gpu_product(mat, x, normalized)
+                    want = oracle_product(orc, mat, ei, n, x, normalized)
+                    assert np.array_equal(got, want)
+                    results[(limit, relayout, stream)] = got
+        mat.stream_coefficients, mat.relayout = True, True
+        assert not np.array_equal(results[(0, True, True)], results[(64, True, True)])      # the order does differ
+        assert orc.max_rel_err(results[(64, True, True)], orc.dense_product(ei, n, x, normalized)) <= TOL_CBM
+    # the CSR baseline on a batched schedule: same rule
+    from cbm4gnn_amd.cbm import schedule_rows
+    order = np.lexsort((ei[1], ei[0]))
+    rp = np.concatenate([[0], np.cumsum(np.bincount(ei[0], minlength=n))]).astype(np.int32)
+    col = ei[1][order].astype(np.int32)
+    m = orc.col_multiplier(ei, n) if normalized else None
+    vals = (m[ei[0][order]] * m[col]).astype(np.float32) if normalized else None
+    x = np.random.default_rng(3).standard_normal((n, 96)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    for limit in (0, 8, 64):
+        sched = schedule_rows(torch.from_numpy(rp), batch=limit).cuda()
+        assert sched.shape[0] == n + (1 if limit else 0)
+        yd = torch.full((n, 96), float("nan"), device="cuda")
+        csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(col).cuda(), None if vals is None else torch.from_numpy(vals).cuda(),
+                 xd, yd, sched)
+        g = groups_for(96, workspace=brings_workspace(True, col.shape[0], n, 96))
+        assert g > 1
+        assert np.array_equal(yd.cpu().numpy(), grouped_spmm(orc, rp, col, vals, x, g, seq_upto=limit))
+    with pytest.raises(ValueError):
+        csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(col).cuda(), None, xd, yd, sched[:-2])
 
 
 def test_reference_test_matmul_correctness(orc):

@@ -240,3 +240,41 @@ def test_tiling_rejects_unsorted_and_out_of_range_columns():
         assert run(bad)[0] == _lib.CBM_ERR_SHAPE, damage
     signed = good.copy(); signed[4 * 9 + 1] |= np.uint32(0x80000000)         # a negative entry in range is fine
     assert run(signed)[0] == 0
+
+
+def test_batched_schedule_layout():
+    """cbm_schedule_rows_batched: rows above the limit first, in the order of cbm_schedule_rows; then the others by
+    descending number of 8-entry chunks, natural order inside a chunk count; a trailer says where they start."""
+    from cbm4gnn_amd.cbm import schedule_rows
+    rng = np.random.default_rng(2)
+    lens = rng.integers(0, 200, size=500)
+    lens[rng.random(500) < 0.5] //= 12
+    rp = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+    parent = torch.from_numpy(np.where(rng.random(500) < 0.3, -1, 0).astype(np.int32))
+    m = torch.from_numpy((rng.random(500) + 0.5).astype(np.float32))
+    plain = schedule_rows(rp, parent, m).numpy()
+    for limit in (1, 8, 20, 64):
+        s = schedule_rows(rp, parent, m, batch=limit).numpy()
+        assert s.shape == (501, 4)
+        n_wide, t, magic, zero = s[-1]
+        assert t == limit and magic == 0x62617463 and zero == 0 and n_wide == int((lens > limit).sum())
+        body = s[:-1]
+        assert sorted(body[:, 2].tolist()) == list(range(500))                      # every row once
+        assert np.array_equal(body[:, 0], rp.numpy()[body[:, 2]]) and np.array_equal(body[:, 1], rp.numpy()[body[:, 2] + 1])
+        want_scale = np.where(parent.numpy()[body[:, 2]] < 0, m.numpy()[body[:, 2]], np.float32(1)).astype(np.float32)
+        assert np.array_equal(body[:, 3].view(np.float32), want_scale)
+        wide = body[:n_wide]
+        assert np.array_equal(wide, plain[lens[plain[:, 2]] > limit])               # same relative order as the plain schedule
+        short = body[n_wide:]
+        sl = lens[short[:, 2]]
+        assert (sl <= limit).all()
+        chunks = (sl + 7) // 8
+        assert (np.diff(chunks) <= 0).all()
+        for c in np.unique(chunks):
+            assert (np.diff(short[chunks == c, 2]) > 0).all()                       # stable
+    import ctypes as C
+    from cbm4gnn_amd import _lib
+    out = np.empty(4 * 501, np.int32)
+    ptr = lambda a: C.c_void_p(a.ctypes.data)
+    assert _lib.host_lib().cbm_schedule_rows_batched(ptr(rp.numpy()), None, None, 500, 65, ptr(out)) == _lib.CBM_ERR_SHAPE
+    assert _lib.host_lib().cbm_schedule_rows_batched(None, None, None, 500, 8, ptr(out)) == _lib.CBM_ERR_NULL
