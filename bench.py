@@ -307,7 +307,7 @@ def measure_multiply(w, alpha, d, args, torch, vendor=False, sample_rows=512, cp
     Returns (row dict, handles for the caller that wants more)."""
     import numpy as np
 
-    from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm, schedule_rows
+    from cbm4gnn_amd.cbm import DEFAULT_BATCH_ROWS, cbm_matrix, csr_spmm, schedule_rows
 
     t0 = time.perf_counter()
     mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=w.normalized, builder=args.builder,
@@ -329,7 +329,7 @@ def measure_multiply(w, alpha, d, args, torch, vendor=False, sample_rows=512, cp
     rp_d, col_d = torch.from_numpy(rp).cuda(), torch.from_numpy(col).cuda()
     val_d = None if val is None else torch.from_numpy(val).cuda()
     ycsr = torch.empty_like(xd)
-    csr_sched = schedule_rows(torch.from_numpy(rp)).to(xd.device)
+    csr_sched = schedule_rows(torch.from_numpy(rp), batch=DEFAULT_BATCH_ROWS).to(xd.device)
     csr_step = lambda: csr_spmm(rp_d, col_d, val_d, xd, ycsr, csr_sched)
     _, csr_ms, _ = time_gpu(csr_step, args.steps, args.warmup, torch)
     # ten times as many calls where a call is short (launch gaps and clock ramps weigh on 20 calls of 20 us)
@@ -589,7 +589,7 @@ def alpha_sweep_bench(args):
     import torch
 
     from cbm4gnn_amd import graphs
-    from cbm4gnn_amd.cbm import cbm_matrix, csr_spmm, schedule_rows
+    from cbm4gnn_amd.cbm import DEFAULT_BATCH_ROWS, cbm_matrix, csr_spmm, schedule_rows
 
     w = graphs.workload(args.workload if args.workload != "c3" else "c5", scale=args.scale)
     d = args.d or w.d
@@ -602,7 +602,7 @@ def alpha_sweep_bench(args):
     rp, col = torch.from_numpy(rp_np).cuda(), torch.from_numpy(col_np).cuda()
     val = None if val_np is None else torch.from_numpy(val_np).cuda()
     ycsr = torch.empty_like(xd)
-    sched = schedule_rows(rp).to(xd.device)
+    sched = schedule_rows(rp, batch=DEFAULT_BATCH_ROWS).to(xd.device)
     _, csr_ms, _ = time_gpu(lambda: csr_spmm(rp, col, val, xd, ycsr, sched), args.steps, args.warmup, torch)
     rows = []
     alphas = [args.alpha] if args.alpha is not None else list(w.alphas)

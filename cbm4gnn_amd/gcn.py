@@ -41,7 +41,7 @@ import torch
 from torch import nn
 
 from . import _lib
-from .cbm import CBMMatmul, _ld, _ptr, _wants_workspace, cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
+from .cbm import DEFAULT_BATCH_ROWS, CBMMatmul, _ld, _ptr, _wants_workspace, cbm_matrix, csr_spmm, relayout_slabs, schedule_rows
 
 __all__ = ["CBMGCNLayer", "CSRGCNLayer", "TwoLayerGCN", "build_operator", "csr_operator", "CSRMatmul", "tuned_gemms"]
 
@@ -212,7 +212,7 @@ def csr_operator(edge_index, n: int, values, device):
     col = ei[1][order].to(torch.int32)
     val = None if values is None else values[order].to(torch.float32)
     return (rowptr.to(device), col.to(device), None if val is None else val.to(device),
-            schedule_rows(rowptr).to(device))
+            schedule_rows(rowptr, batch=DEFAULT_BATCH_ROWS).to(device))
 
 
 class CSRGCNLayer(nn.Module):

@@ -15,7 +15,7 @@ import statistics
 import numpy as np
 import torch
 
-from .cbm import cbm_matrix, csr_spmm, schedule_rows
+from .cbm import DEFAULT_BATCH_ROWS, cbm_matrix, csr_spmm, schedule_rows
 
 __all__ = ["time_calls", "tune_alpha", "DEFAULT_ALPHAS"]
 
@@ -79,7 +79,7 @@ def tune_alpha(edge_index, d: int, alphas=DEFAULT_ALPHAS, normalized: bool = Fal
     if normalized:
         m = torch.bincount(ei[0].to(torch.int64), minlength=n).to(torch.float32).pow(-0.5)
         val = (m[ei[0][order].long()] * m[col.long()]).to(dev)
-    rowptr_d, col_d, sched_d = rowptr.to(dev), col.to(dev), schedule_rows(rowptr).to(dev)
+    rowptr_d, col_d, sched_d = rowptr.to(dev), col.to(dev), schedule_rows(rowptr, batch=DEFAULT_BATCH_ROWS).to(dev)
     y_csr = torch.empty_like(x)
     csr_ms, _ = time_calls(lambda: csr_spmm(rowptr_d, col_d, val, x, y_csr, sched_d), iters, warmup)
     scale = float(y_csr.abs().max())
