@@ -47,7 +47,9 @@ namespace {
 #define CBM_TILED_VECS 6                   // 16-byte index vectors requested together per row in the tiled kernel
 #endif
 #ifndef CBM_TILED_REMOTE_U8
-#define CBM_TILED_REMOTE_U8 8              // remote entries per row in flight in the tiled kernel, 128-byte slabs (2 rows per lane)
+#define CBM_TILED_REMOTE_U8 6              // remote entries per row in flight in the tiled kernel, 128-byte slabs (2 rows per lane):
+                                           // 8 need 24 registers more than a 1024-thread workgroup has (spilled: 1.62 ms on the
+                                           // 233k-row community graph at d = 128), 7: 1.58, 6: 1.57 with none spilled, 5: 1.58
 #endif
 #ifndef CBM_TILED_REMOTE_U4
 #define CBM_TILED_REMOTE_U4 8              // the same for the 64-byte half slab (1 row per lane)
