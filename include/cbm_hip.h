@@ -38,8 +38,14 @@ enum {
                                 cbm_spmm_update_static_f32 holds                     */
 };
 
-/* Floats of the per-device static scratch array of cbm_spmm_update_static_f32 (128 MiB). */
+/* Floats of the per-device static scratch array of cbm_spmm_update_static_f32 (128 MiB).  The array is part
+ * of the library's device image: every device a process uses the library on gives up this much memory from
+ * the moment the library's code is loaded there, whether or not that entry point is ever called.  A build
+ * that wants less (or more) defines the macro on the compiler's command line, for the library and its users
+ * alike. */
+#ifndef CBM_STATIC_SCRATCH_FLOATS
 #define CBM_STATIC_SCRATCH_FLOATS (32 * 1024 * 1024)
+#endif
 
 /* flags of cbm_spmm_f32 / csr_spmm_f32 */
 enum {
@@ -464,7 +470,9 @@ int64_t cbm_spmm_update_paths_scratch_floats(int32_t n, int32_t d, int32_t n_lev
  * allocates and frees nothing, on host or device.  All calls on one device share that device's
  * array: calls that may overlap in time on one device (different streams, different threads)
  * race on it; serialise them.  The array keeps the previous call's contents; every float the
- * gather reads is rewritten by the copy first. */
+ * gather reads is rewritten by the copy first.  "Bit for bit" holds while the process-wide hooks
+ * (cbm_set_spmm_kernel) are not changed by another thread during the call: the size of the copy and the
+ * launch plan are both derived from them. */
 int cbm_spmm_update_static_f32(const int32_t* rowptr_dev, const uint32_t* idx_dev, int64_t nnz, const float* m_dev,
                                const float* coef_dev, const int32_t* parent_dev, const int32_t* row_sched_dev,
                                const int32_t* order_dev, const int32_t* level_off_dev,
