@@ -90,6 +90,11 @@ def _check_f32_matrix(t, name, n=None):
 
 # Rows with fewer delta entries than this on average do not repay the slab-major copy of X
 _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT = 24
+# ... and while all of X is at most this many bytes (it stays in the L2s, and the copy is one more dependent
+# launch of ~10 us) rows must average this many entries: 12,000 x 128 floats, 35 entries per row: 33.1 us with
+# the copy, 27.1 us gathered in place; 194 entries per row: 79.9 / 80.9 us
+_SMALL_X_BYTES = 8 << 20
+_MIN_ENTRIES_PER_ROW_SMALL_X = 96
 
 
 def _wants_workspace(x, y, nnz):
@@ -100,7 +105,8 @@ def _wants_workspace(x, y, nnz):
     n, d = x.shape
     if n == 0 or d == 0:
         return False
-    if nnz >= _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT * n:
+    need = _MIN_ENTRIES_PER_ROW_SMALL_X if 4 * n * d <= _SMALL_X_BYTES else _MIN_ENTRIES_PER_ROW_FOR_RELAYOUT
+    if nnz >= need * n:
         return True
     return int(_lib.hip_lib().cbm_spmm_summation_groups(d, _ld(x), _ld(y), _ptr(x), _ptr(y), 0)) == 1
 

@@ -31,6 +31,15 @@ def _need_gpu():
     _lib.hip_lib()
 
 
+@pytest.fixture(autouse=True)
+def _copy_rule_of_large_matrices(monkeypatch):
+    """The matrices of these tests are small (X of a few MB), where the Python layer asks for 96 entries per row
+    before it copies X slab-major; the tests are about the kernels behind that choice, so they run under the rule
+    for large matrices (24 entries per row).  ``test_small_x_is_gathered_in_place`` covers the small-X rule."""
+    from cbm4gnn_amd import cbm as cbm_mod
+    monkeypatch.setattr(cbm_mod, "_SMALL_X_BYTES", 0)
+
+
 def groups_for(d, ld=None, workspace=False):
     """Partial sums per output element the SpMM keeps for 16-byte aligned [*, d] matrices of row
     stride ld (1 = strictly in order), with or without a workspace for the slab-major copy of X;
@@ -59,9 +68,11 @@ def grouped_spmm(orc, rp, col, val, xs, groups, tail=0, threads=1, seq_upto=0):
 
 
 def brings_workspace(relayout, nnz, n, d, ld=None):
-    """The Python layer's rule: a workspace when rows average >= 24 entries, or when the width would
-    otherwise run one wavefront per row."""
-    return bool(relayout) and n > 0 and (nnz >= 24 * n or groups_for(d, ld) == 1)
+    """The Python layer's rule: a workspace when rows average >= 24 entries (>= 96 while all of X is at most
+    ``_SMALL_X_BYTES``), or when the width would otherwise run one wavefront per row."""
+    from cbm4gnn_amd import cbm as cbm_mod
+    need = cbm_mod._MIN_ENTRIES_PER_ROW_SMALL_X if 4 * n * d <= cbm_mod._SMALL_X_BYTES else cbm_mod._MIN_ENTRIES_PER_ROW_FOR_RELAYOUT
+    return bool(relayout) and n > 0 and (nnz >= need * n or groups_for(d, ld) == 1)
 
 
 def mat_groups(mat, d, ld=None, update=False):
@@ -385,6 +396,28 @@ def test_short_rows_summed_in_batches(orc, kind, normalized):
         assert np.array_equal(yd.cpu().numpy(), grouped_spmm(orc, rp, col, vals, x, g, seq_upto=limit))
     with pytest.raises(ValueError):
         csr_spmm(torch.from_numpy(rp).cuda(), torch.from_numpy(col).cuda(), None, xd, yd, sched[:-2])
+
+
+def test_small_x_is_gathered_in_place(orc, monkeypatch):
+    """While all of X is at most 8 MB the copy must repay one more dependent launch: rows then need 96 entries on
+    average, not 24.  Same matrix under both rules: different kernels, each bit-exact against its order model."""
+    from cbm4gnn_amd import cbm as cbm_mod
+    n, d = 3000, 128
+    ei = graphs.add_self_loops(graphs.sbm(n, 30, 0.4, 0.002, seed=8), n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=True)
+    assert 24 * n <= mat.nnz < 96 * n
+    x = np.random.default_rng(8).standard_normal((n, d)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    results = []
+    for small_bytes in (8 << 20, 0):
+        monkeypatch.setattr(cbm_mod, "_SMALL_X_BYTES", small_bytes)
+        say("small X rule", small_bytes)
+        assert cbm_mod._wants_workspace(xd, xd, mat.nnz) == (small_bytes == 0)
+        got = gpu_product(mat, x, True)
+        assert np.array_equal(got, oracle_product(orc, mat, ei, n, x, True))
+        results.append(got)
+    assert orc.max_rel_err(results[0], results[1]) <= 1e-6 and not np.array_equal(results[0], results[1])
+    assert cbm_mod._wants_workspace(torch.empty((n, 41), device="cuda"), torch.empty((n, 41), device="cuda"), mat.nnz)   # odd widths always
 
 
 def test_reference_test_matmul_correctness(orc):
