@@ -4,17 +4,26 @@
 //   (1)  spmm_slab_per_xcd    delta SpMM  Z = D * diag(m) * X  with the feature dimension cut into
 //                             128-byte slabs (256-byte on the row-major path of wide d): one slab per
 //                             XCD (so an XCD's L2 only ever sees its slab of X), persistent waves
-//                             walking a longest-first row schedule, 8 lanes per delta entry, 64
-//                             entries in flight per wave.  Any width when the caller brings a
-//                             workspace for the slab-major copy of X (relayout_slabs).
+//                             walking a longest-first row schedule.  Long rows: one row per wave, 8
+//                             lanes per delta entry, 64 entries in flight.  Short rows (a batched
+//                             schedule): 8 rows per wave, one lane group each, entries in order.  Any
+//                             width when the caller brings a workspace for the slab-major copy of X
+//                             (relayout_slabs).
+//        spmm_tiled_local     the same product for matrices whose entries cluster: tiles of the copy
+//                             staged in LDS, one row per lane group, the scattered rest from the copy
+//                             in global memory in the same launch.
 //        spmm_wave_per_row    the same product without a workspace for widths that are not a
 //                             multiple of 32: one wave per row, lanes span the feature columns,
 //                             packed indices broadcast with v_readlane so X-row addresses are scalar.
-//   (2)  propagate_level / propagate_narrow_levels / propagate_chain / scale_level0
-//                             tree propagation  Y[v] (+)= Y[parent(v)]  level-synchronously over a
-//                             host-computed (level, id) ordering: one launch per wide level, one
-//                             single-workgroup launch per run of narrow levels, one
-//                             register-carried launch per chain of single-row levels.
+//   (2)  tree propagation  Y[v] (+)= Y[parent(v)]:
+//        propagate_level / propagate_narrow_levels / propagate_chain / scale_level0
+//                             level-synchronously over a host-computed (level, id) ordering: one
+//                             launch per wide level, one single-workgroup launch per run of narrow
+//                             levels, one register-carried launch per chain of single-row levels;
+//        propagate_subtrees   every subtree below a level in ONE launch: a wave walks a host-made
+//                             depth-first sequence, parent values in a register and LDS slots;
+//        propagate_paths / spmm_update_paths_wave_per_row
+//                             shallow trees: every row sums down its own ancestor path (one launch).
 // The SpMM instantiations with PACKED = false are the plain CSR baseline.
 //
 // What each launcher replaces in the reference is stated in include/cbm_hip.h.
