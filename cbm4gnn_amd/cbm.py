@@ -742,8 +742,7 @@ class cbm_matrix:
     def _host_walk_plan(self, cut, d):
         """``cbm_walk_plan_build`` for this tree at ``cut`` (CPU tensors + stats), cached.  The bins are sized so
         that (bins x 64-column slices) wavefronts fill the GPU a few times over."""
-        slices = (d + 63) // 64
-        target_bins = max(64, 8192 // slices)
+        target_bins = self._walk_bin_target(d)
         key = (int(cut), target_bins)
         plan = self._walk_plans.get(key)
         if plan is None:
@@ -783,18 +782,44 @@ class cbm_matrix:
             raise ValueError('subtree_walk must be "auto", "on", "off" or a cut level')
         key = ("choice", policy, (d + 63) // 64)
         if key not in self._walk_plans:
-            best, best_cost = None, None
-            for cut in range(0, min(self.n_levels - 1, 4)):           # deeper cuts: the levels above cost launches again
-                plan = self._host_walk_plan(cut, d)
-                if not plan or plan["n_entries"] == 0:
+            # candidates: every cut level up to 16 (deeper cuts pay a launch per level above them anyway),
+            # ranked by the estimate from the subtree sizes alone; only the winner's plan is built
+            sizes, target = self._subtree_sizes(), self._walk_bin_target(d)
+            lo, order = self.level_off.tolist(), self.order.numpy()
+            best_cut, best_cost = None, None
+            for cut in range(0, min(self.n_levels - 1, 16)):
+                heads = sizes[order[lo[cut]:lo[cut + 1]]]
+                heads = heads[heads > 1]
+                if heads.size == 0:
                     continue
-                cost = self._subtree_plan_cost_us(plan, d)
-                if best is None or cost < best_cost:
-                    best, best_cost = plan, cost
-            if best is not None and policy == "auto" and best_cost > 0.8 * self._level_plan_cost_us(d):
+                entries = int(heads.sum())
+                longest = max(int(heads.max()), -(-entries // target), 32)   # small subtrees are packed into bins
+                cost = (self._level_plan_cost_us(d, 1, cut + 1) + self._WALK_US_PER_LAUNCH +
+                        max(longest * self._WALK_US_PER_ENTRY, entries * d * 8 / self._WALK_BYTES_PER_US))
+                if best_cut is None or cost < best_cost:
+                    best_cut, best_cost = cut, cost
+            best = self._host_walk_plan(best_cut, d) if best_cut is not None else None
+            if best and policy == "auto" and self._subtree_plan_cost_us(best, d) > 0.8 * self._level_plan_cost_us(d):
                 best = None
-            self._walk_plans[key] = best
+            self._walk_plans[key] = best or None
         return self._walk_plans[key]
+
+    def _subtree_sizes(self):
+        """Rows in the subtree of every row (itself included), int64 NumPy; computed once."""
+        sizes = self._walk_plans.get("sizes")
+        if sizes is None:
+            sizes = np.ones(self.num_rows, np.int64)
+            lo, order, parent = self.level_off.tolist(), self.order.numpy(), self.parent.numpy()
+            for l in range(self.n_levels - 1, 0, -1):                       # leaves first
+                rows = order[lo[l]:lo[l + 1]]
+                np.add.at(sizes, parent[rows], sizes[rows])
+            self._walk_plans["sizes"] = sizes
+        return sizes
+
+    @staticmethod
+    def _walk_bin_target(d):
+        """Bins a plan aims for: (bins x 64-column slices) wavefronts fill the GPU a few times over."""
+        return max(64, 8192 // ((d + 63) // 64))
 
     def _walk_struct(self, st, plan):
         """``struct cbm_walk_dev`` over the device copy of ``plan`` (uploaded once per device and cut)."""

@@ -175,3 +175,35 @@ def test_walk_policy_by_estimate():
     flat = cbm_matrix(torch.from_numpy(graphs.erdos_renyi(50, 0.3, 1)), None, alpha=10_000)
     flat.subtree_walk = "on"
     assert flat.walk_plan(64) is None
+
+
+def test_auto_finds_a_deeper_cut_when_the_top_of_the_tree_is_narrow():
+    """One child of the root, 4 rows below it, 256 below those, then 256 chains of 100 rows: walked from the
+    root's child the whole tree is ONE sequence; below level 2 it is 256 independent ones.  The estimate must
+    pick that cut (levels 1 and 2 level by level, the rest in one launch)."""
+    from cbm4gnn_amd.cbm import tree_levels
+    par = [-1] + [0] * 4 + [1 + i // 64 for i in range(256)]
+    first_chain = len(par)
+    for depth in range(100):
+        par += [first_chain - 256 + i if depth == 0 else first_chain + (depth - 1) * 256 + i for i in range(256)]
+    par = np.array(par, np.int64)
+    n = par.shape[0]
+    kids = [[] for _ in range(n + 1)]
+    for v in range(n):
+        kids[n if par[v] < 0 else par[v]].append(v)
+    mst_col = np.array(sum(kids, []), np.int32)
+    mst_row = np.concatenate([[0], np.cumsum([len(k) for k in kids])]).astype(np.int32)
+    parent, order, level_off = tree_levels(mst_row, mst_col)
+    mat = cbm_matrix.__new__(cbm_matrix)
+    mat.num_rows, mat.n_levels = n, level_off.shape[0] - 1
+    mat.parent, mat.order, mat.level_off = (torch.from_numpy(a) for a in (parent, order, level_off))
+    mat._walk_plans, mat.subtree_walk = {}, "auto"
+    assert mat.n_levels == 103
+    plan = mat.walk_plan(256)
+    assert plan is not None and plan["cut"] == 2 and plan["longest_bin"] <= 2 * 101 and plan["n_entries"] == 256 * 101
+    assert mat._subtree_plan_cost_us(plan, 256) < 0.2 * mat._level_plan_cost_us(256)
+    sizes = mat._subtree_sizes()
+    assert sizes[0] == n and (sizes[1:5] == 1 + 64 * 101).all() and sizes[-1] == 1
+    # a forced cut of 0 is still honoured (one bin, one long sequence)
+    mat.subtree_walk = 0
+    assert mat.walk_plan(256)["n_bins"] == 1
