@@ -275,6 +275,72 @@ def test_duplication_graph_full_size():
         assert torch.equal(_mul(mat, xd), got)
 
 
+def test_duplication_graph_at_the_configured_size():
+    """c2b: the duplication process held to the ~240k undirected edges the configuration names (489,520
+    non-zeros with A + I), normalised, d = 128, alpha 0 and 8: 1,024 rows against fp64 SciPy rows, everything
+    against the GPU CSR baseline, and the one-launch path walk against the level-by-level walk."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c2b")
+    assert abs((w.edge_index.shape[1] - w.n) // 2 - 240_000) < 5_000
+    rp, col = _csr(w.edge_index, w.n)
+    x = w.features(0)
+    xd = x.cuda()
+    rows = np.sort(np.random.default_rng(3).choice(w.n, size=1024, replace=False))
+    rows_d = torch.from_numpy(rows).cuda()
+    for alpha in (0, 8):
+        print("[gpu-case] c2b full size alpha", alpha, flush=True); sys.stdout.flush()
+        mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=alpha, normalized=True)
+        assert mat.n_levels >= 3 and 1.0 < mat.compression_ratio() < 1.3
+        m = mat.col_multiplier.numpy()
+        got = _mul(mat, xd)
+        _assert_rows_close(got[rows_d].cpu().numpy().astype(np.float64), _rows_fp64(rp, col, m, x.numpy(), rows))
+        val = torch.from_numpy((np.repeat(m, np.diff(rp)) * m[col]).astype(np.float32)).cuda()
+        base = torch.empty_like(xd)
+        csr_spmm(torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda(), val, xd, base)
+        assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+        assert mat._walks_paths(w.n, xd.size(1))
+        mat.path_walk_max_bytes = 0                          # the walk by subtrees / level by level instead
+        assert torch.equal(_mul(mat, xd), got)
+        mat.subtree_walk = "off"
+        assert torch.equal(_mul(mat, xd), got)
+
+
+def test_deep_and_wide_tree_full_size():
+    """c6: 182,400 rows in 800 staircases + noise, compression 9.4, 65 tree levels of ~3,000 rows: the walk by
+    subtrees (one launch) against the level-by-level walk bit for bit, 1,024 rows against fp64 SciPy rows, the
+    whole product against the GPU CSR baseline; short delta rows in batches against one row per wavefront."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c6")
+    print("[gpu-case] c6 full size, building", flush=True); sys.stdout.flush()
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=0, normalized=True)
+    assert mat.compression_ratio() > 8 and mat.n_levels > 50
+    widths = np.diff(mat.level_off.numpy())
+    assert int((widths > 64).sum()) >= 50
+    plan = mat.walk_plan(w.d)
+    assert plan is not None and plan["cut"] == 0 and plan["n_bins"] > 1000      # "auto" takes the subtree walk
+    rp, col = _csr(w.edge_index, w.n)
+    m = mat.col_multiplier.numpy()
+    x = w.features(0)
+    xd = x.cuda()
+    print("[gpu-case] c6 full size, multiply", flush=True); sys.stdout.flush()
+    got = _mul(mat, xd)
+    rows = np.sort(np.random.default_rng(5).choice(w.n, size=1024, replace=False))
+    rows_d = torch.from_numpy(rows).cuda()
+    _assert_rows_close(got[rows_d].cpu().numpy().astype(np.float64), _rows_fp64(rp, col, m, x.numpy(), rows))
+    val = torch.from_numpy((np.repeat(m, np.diff(rp)) * m[col]).astype(np.float32)).cuda()
+    base = torch.empty_like(xd)
+    csr_spmm(torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda(), val, xd, base)
+    assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+    mat.subtree_walk = "off"
+    print("[gpu-case] c6 full size, level-by-level walk", flush=True); sys.stdout.flush()
+    assert torch.equal(_mul(mat, xd), got)
+    mat.batch_rows = 0                                       # another summation order for the short rows
+    unbatched = _mul(mat, xd)
+    assert float((unbatched - got).abs().max() / got.abs().max()) <= 1e-5
+
+
 def test_alpha_sweep_graph_same_format_for_every_alpha():
     """On the dense-community graph alpha <= 32 prunes nothing (every admissible pair clears the
     threshold by far more): the builder must return the arrays of alpha = 0 for the whole sweep."""
