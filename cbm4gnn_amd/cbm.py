@@ -440,7 +440,7 @@ class cbm_matrix:
                 raise ValueError(f"{path} is damaged: {e}") from None
             except KeyError as e:
                 raise ValueError(f"{path} lacks the array {e}") from None
-        problem = cls._validate_loaded(self, host, m, edges, fingerprint)
+        problem = self._validate_loaded(host, m, edges, fingerprint)
         if problem:
             raise ValueError(f"{path} does not hold a consistent CBM format: {problem}")
         for k in cls._SAVED_ARRAYS:
@@ -457,7 +457,6 @@ class cbm_matrix:
         self._init_tiling("auto")
         return self
 
-    @staticmethod
     def _validate_loaded(self, host, m, edges, fingerprint):
         """Why the arrays read from a file are not a format the kernels may run on (a string), or None.
         O(N + nnz) vectorised NumPy.  Checked: dtypes and lengths; row offsets start at 0, never decrease
