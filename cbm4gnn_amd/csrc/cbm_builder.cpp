@@ -1057,12 +1057,14 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                 for (int32_t r = p * P; r < r_end; r++) {
                     int64_t at_r = out->rowptr_r[r];
                     // Columns ascend within a row, so the entries of one block form one run.  Inside a
-                    // segment the entries are stored parity-major: a row of even index lists its entries
-                    // in even columns first (ascending), then those in odd columns; a row of odd index
-                    // the other way round.  A 128-byte row of the tile covers half of the LDS banks,
-                    // chosen by the parity of its index; the kernel serves two neighbouring matrix
-                    // rows per cycle, and with this order they read opposite halves nearly always.
-                    const uint32_t first_parity = (uint32_t)(r & 1);
+                    // segment the entries are stored by the class q = (column - row) mod 4, in the order
+                    // q = 0, 2, 1, 3, ascending inside a class.  A 128-byte row of the tile covers half of
+                    // the LDS banks, chosen by the parity of its index, and the kernel serves two
+                    // neighbouring matrix rows per cycle: with q = 0, 2 first a row of even index reads even
+                    // columns first and its odd neighbour odd ones -- opposite halves nearly always.  A
+                    // 64-byte row (the half slab) covers a quarter of the banks, chosen by its index mod 4,
+                    // and four neighbouring matrix rows are served per cycle: in step they read the four
+                    // different classes.
                     int64_t k = rowptr[r];
                     const int64_t k_end = rowptr[r + 1];
                     while (k < k_end) {
@@ -1073,10 +1075,11 @@ int cbm_tile_rows(const int32_t* rowptr, const uint32_t* idx, int32_t n, int32_t
                         int64_t k1 = k;
                         while (k1 < k_end && (int32_t)((idx[k1] & 0x7fffffffu) / (uint32_t)T) == t) k1++;
                         int64_t at = (int64_t)out->seg[(size_t)b * (P + 1) + (r - p * P)] * 8;
-                        for (int pass = 0; pass < 2; pass++)
+                        static const uint32_t kClassOrder[4] = {0u, 2u, 1u, 3u};
+                        for (int pass = 0; pass < 4; pass++)
                             for (int64_t q = k; q < k1; q++) {
                                 const uint32_t c = idx[q] & 0x7fffffffu;
-                                if (((c & 1u) == first_parity) != (pass == 0)) continue;
+                                if (((c - (uint32_t)r) & 3u) != kClassOrder[pass]) continue;
                                 out->lidx[at++] = (uint16_t)(((c - (uint32_t)t * (uint32_t)T) * 8u) | ((idx[q] >> 31) << 15));
                             }
                         k = k1;

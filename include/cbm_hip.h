@@ -214,10 +214,10 @@ int cbm_schedule_rows_blocks(const int32_t* rowptr, const uint32_t* idx, const i
  *   blk_tile[n_blocks]        tile index of each block (first row of X it covers = tile * tile_rows)
  *   seg[n_blocks][panel_rows + 1]  per block and panel row: start of the row's segment in lidx, in
  *                             units of 8 entries; a segment holds the row's entries inside the
- *                             block, padded to a multiple of 8, parity-major: a row of even index
- *                             lists its entries in even columns first (ascending), then those in odd
- *                             columns (ascending); a row of odd index the other way round (the two
- *                             rows the kernel serves in one LDS cycle then read opposite bank halves)
+ *                             block, padded to a multiple of 8, ordered by the class
+ *                             q = (column - row) mod 4 in the order q = 0, 2, 1, 3, ascending inside a
+ *                             class: the two 128-byte rows (four 64-byte rows of the half slab) the
+ *                             kernel serves in one LDS cycle then read different bank halves (quarters)
  *   lidx[nnz_local_padded]    (row of X - first row of the tile) * 8 | (negative ? 1 << 15 : 0);
  *                             padding = tile_rows * 8, the all-zero row behind the tile
  *   rowptr_r / idx_r          the remote entries, packed like idx, columns ascending
@@ -517,7 +517,7 @@ int64_t cbm_spmm_tiled_workspace_floats(const cbm_tiling_dev* t, int32_t n, int3
  * copy, scaled by m when m is given (so no entry carries a coefficient).  flags: CBM_SPMM_RELU;
  * CBM_SPMM_WORKSPACE_READY (with m: together with CBM_SPMM_WORKSPACE_PRESCALED).  Per output
  * element the fp32 sum is (remote entries, summed as cbm_spmm_f32 sums a row) + (local entries,
- * one after the other in storage order -- blocks by ascending tile, parity-major inside a block,
+ * one after the other in storage order -- blocks by ascending tile, by class (column - row) mod 4 inside a block,
  * see cbm_tile_rows -- starting from zero), then the left scale, then the ReLU.  Worth it when most entries are local: 232 965 rows x 491 entries, 89 % of them in
  * blocks of a 50-community graph, d = 128: 1.99 ms against 2.78 ms for cbm_spmm_f32.
  * Replaces the same mkl_sparse_s_mm call as cbm_spmm_f32 (cbm_extensions.cpp:1133-1159). */

@@ -207,9 +207,10 @@ def oracle_delta_spmm(orc, mat, ei, n, x, normalized):
         else:
             remote = grouped_with_cuts(orc, rp, c[~local].astype(np.int32), sg[~local], xs,
                                        mat.split_chunk if mat.has_cut_rows() else 0, plan_groups, plan_tail)
-        # local entries in storage order: by tile, then the columns of the row's own parity, then the others
+        # local entries in storage order: by tile, then by class (column - row) mod 4 in the order 0, 2, 1, 3
         lr, lc, ls = row[local], c[local], sg[local]
-        order = np.lexsort((lc, (lc + lr) % 2, lc // mat.tile_rows, lr))
+        phase = np.array([0, 2, 1, 3])[(lc - lr) % 4]
+        order = np.lexsort((lc, phase, lc // mat.tile_rows, lr))
         rp = np.concatenate([[0], np.cumsum(np.bincount(lr, minlength=n))]).astype(np.int32)
         return remote + orc.csr_spmm(rp, lc[order].astype(np.int32), ls[order], xs, groups=1)
     if not normalized:

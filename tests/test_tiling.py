@@ -48,10 +48,10 @@ def decode(th, n):
                 off = (real & 0x7FFF) // 8
                 assert ((real & 0x7FFF) % 8 == 0).all() and (off < T).all()
                 r = p * P + pr
-                # parity-major: the columns of the row's own parity first, each half ascending
-                first = off[off % 2 == r % 2]
-                assert np.array_equal(off, np.concatenate([first, off[off % 2 != r % 2]]))
-                assert (np.diff(first) > 0).all() and (np.diff(off[off % 2 != r % 2]) > 0).all()
+                # by class (column - row) mod 4 in the order 0, 2, 1, 3 (so: own parity first), ascending inside a class
+                cls = (off - r) % 4
+                want = np.concatenate([np.sort(off[cls == q]) for q in (0, 2, 1, 3)])
+                assert np.array_equal(off, want)
                 assert k == 0 or r < n
                 out += [(r, int(bt[b]) * T + int(o), int(v >> 15)) for o, v in zip(off, real)]
     return sorted(out)
