@@ -207,3 +207,77 @@ def test_auto_finds_a_deeper_cut_when_the_top_of_the_tree_is_narrow():
     # a forced cut of 0 is still honoured (one bin, one long sequence)
     mat.subtree_walk = 0
     assert mat.walk_plan(256)["n_bins"] == 1
+
+
+def _fake_matrix(par):
+    """A ``cbm_matrix`` shell holding only a tree (what the walk plan reads)."""
+    from cbm4gnn_amd.cbm import tree_levels
+    n = par.shape[0]
+    kids = [[] for _ in range(n + 1)]
+    for v in range(n):
+        kids[n if par[v] < 0 else par[v]].append(v)
+    mst_col = np.array(sum(kids, []), np.int32)
+    mst_row = np.concatenate([[0], np.cumsum([len(k) for k in kids])]).astype(np.int32)
+    parent, order, level_off = tree_levels(mst_row, mst_col)
+    mat = cbm_matrix.__new__(cbm_matrix)
+    mat.num_rows, mat.n_levels = n, level_off.shape[0] - 1
+    mat.parent, mat.order, mat.level_off = (torch.from_numpy(a) for a in (parent, order, level_off))
+    mat.mst_row, mat.mst_col = torch.from_numpy(mst_row), torch.from_numpy(mst_col)
+    mat._walk_plans, mat.subtree_walk = {}, "auto"
+    return mat
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_plans_of_random_trees_walk_like_the_oracle(orc, seed):
+    """Random forests of every shape the builder can produce and some it rarely does -- random recursive trees
+    (bushy, ~2 ln n levels), brooms (a chain ending in a star), caterpillars, forests of stars, near-binary trees,
+    single rows -- at every cut level: the plan's layout invariants hold and its interpretation equals the
+    oracle's walk (plain and fused) bit for bit."""
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.choice([1, 2, 17, 200, 1500]))
+    kind = ["recursive", "broom", "caterpillar", "stars", "binary", "forest"][seed % 6]
+    roots = int(rng.integers(1, max(2, n // 10 + 1)))
+    par = np.full(n, -1, np.int64)
+    for v in range(roots, n):
+        if kind == "recursive" or kind == "forest":
+            par[v] = int(rng.integers(0, v))
+        elif kind == "broom":
+            par[v] = v - roots if v < n // 2 else int(rng.integers(max(roots, n // 2 - roots), max(roots + 1, n // 2)))
+        elif kind == "caterpillar":
+            par[v] = v - 2 * roots if (v - roots) % 2 == 0 and v >= 3 * roots else max(v - roots - (v - roots) % 2 * roots, 0) if v >= 2 * roots else v - roots
+        elif kind == "stars":
+            par[v] = v % roots
+        else:
+            par[v] = (v - roots) // 2 if (v - roots) // 2 < v else 0
+    par = np.minimum(par, np.arange(n) - 1)                    # a parent always precedes its child: no cycles
+    par[:roots] = -1
+    mat = _fake_matrix(par)
+    d = int(rng.choice([1, 8, 19]))
+    z = rng.standard_normal((n, d)).astype(np.float32)
+    m = (rng.random(n).astype(np.float32) + 0.5)
+    for fused in (False, True):
+        want = (orc.update_fused(mat.mst_row.numpy(), mat.mst_col.numpy(), m, z.copy()) if fused
+                else orc.update_plain(mat.mst_row.numpy(), mat.mst_col.numpy(), z.copy()))
+        z0 = z.copy()
+        if fused:
+            rt = mat.parent.numpy() < 0
+            z0[rt] = (z0[rt] * m[rt, None]).astype(np.float32)
+        level_of = np.empty(n, np.int64)
+        level_of[mat.order.numpy()] = np.repeat(np.arange(mat.n_levels), np.diff(mat.level_off.numpy()))
+        for cut in sorted({0, mat.n_levels // 2, max(mat.n_levels - 2, 0)}):
+            if cut >= mat.n_levels:
+                continue
+            plan = mat._host_walk_plan(cut, d)
+            assert plan, (kind, n, cut)
+            if plan["n_entries"]:
+                check_plan_shape(mat, plan, cut)
+            y = z0.copy()
+            above = level_of <= cut
+            y[above] = want[above]
+            written = interpret(plan, m if fused else None, y)
+            assert np.array_equal(written, (~above).astype(np.int32))
+            assert np.array_equal(y, want), (kind, n, fused, cut)
+    # the estimate-driven choice never fails to produce a usable answer
+    mat.subtree_walk = "on"
+    chosen = mat.walk_plan(64)
+    assert chosen is None or 0 <= chosen["cut"] < mat.n_levels
