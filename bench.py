@@ -367,26 +367,31 @@ def measure_multiply(w, alpha, d, args, torch, vendor=False, sample_rows=512, cp
     b_min = compulsory_bytes(n, nnz, d)
     # the dominant kernel alone; a small product on a shallow tree is ONE launch that does everything
     if not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(n, d):
-        relayout_ms, spmm_ms, prop_ms, kernel, slab = 0.0, span_ms, 0.0, "spmm_update_paths_wave_per_row", False
+        relayout_ms, spmm_ms, prop_ms, prop_how, kernel, slab = 0.0, span_ms, 0.0, None, "spmm_update_paths_wave_per_row", False
         roof = roofline_of(w.name, alpha, d, kernel, spmm_ms, b_spmm + b_prop, b_min, args.scale)
     else:
         relayout_ms, spmm_ms, zd, kernel = spmm_alone(mat, xd, w.normalized, args.steps, args.warmup, torch)
-        prop_ms = 0.0
-        if tree_edges:
-            _, prop_ms, _ = time_gpu(lambda: mat._run_propagate(zd, use_m=w.normalized), args.steps, args.warmup, torch)
+        prop_ms, prop_how = 0.0, None
+        if tree_edges and walks_paths_in_multiply(mat, n, d):
+            # the path walk reads Z from a scratch the multiply fills: it cannot run on its own
+            prop_ms, prop_how = max(span_ms - relayout_ms - spmm_ms, 0.0), "multiply minus copy and SpMM (the path walk runs only inside the multiply)"
+        elif tree_edges:
+            # the walk as the multiply runs it: the root children were scaled in the SpMM's epilogue
+            _, prop_ms, _ = time_gpu(lambda: mat._run_propagate(zd, use_m=w.normalized, scale_roots=False), args.steps, args.warmup, torch)
+            prop_how = "the walk's launches alone, in place on Z"
         slab = kernel != "spmm_wave_per_row"
         roof = roofline_of(w.name, alpha, d, kernel, spmm_ms, b_spmm, b_min, args.scale)
         del zd
     row = {
         "workload": f"{w.name}: {w.note}", "alpha": alpha, "d": d, "nodes": n, "nnz_A": n_edges, "nnz_delta": nnz,
         "compression_ratio": mat.compression_ratio(), "tree_levels": mat.n_levels, "tree_edges": tree_edges,
-        "launches_per_multiply": launches_per_multiply(mat, n, d),
+        "launches_per_multiply": launches_per_multiply(mat, n, d, copies_x=relayout_ms > 0.0),
         "cbm_ms": span_ms, "cbm_ms_median": med_ms, "gpu_csr_ms": csr_ms, "speedup_vs_gpu_csr": csr_ms / span_ms,
         "flat_binary_ms": flat_ms, "speedup_from_compression": (flat_ms / span_ms) if flat_ms else None,
         "cbm_ms_back_to_back": loop_ms, "gpu_csr_ms_back_to_back": csr_loop_ms,
         "flat_binary_ms_back_to_back": flat_loop_ms,
         "speedup_vs_gpu_csr_back_to_back": csr_loop_ms / loop_ms, "back_to_back_calls": reps,
-        "kernel_ms": {"relayout_slabs": relayout_ms, "delta_spmm": spmm_ms, "propagate": prop_ms},
+        "kernel_ms": {"relayout_slabs": relayout_ms, "delta_spmm": spmm_ms, "propagate": prop_ms, "propagate_is": prop_how},
         "walk_share": prop_ms / (relayout_ms + spmm_ms + prop_ms) if prop_ms else 0.0,
         "cbm_GBps": (b_spmm + b_prop) / (span_ms * 1e-3) / 1e9,
         "edges_x_features_per_s": n_edges * d / (span_ms * 1e-3),
@@ -433,22 +438,29 @@ def level_launches(lo, first_level, last_level):
     return launches
 
 
-def launches_per_multiply(mat, n, d):
+def walks_paths_in_multiply(mat, n, d):
+    """Whether a multiply of ``mat`` with an [n, d] matrix ends in the one-launch path walk (the Python
+    layer's rule: untiled, no cut rows, a shallow tree, a product within the path walk's size limit)."""
+    return mat.n_levels > 1 and not (mat.is_tiled() or mat.has_cut_rows()) and mat._walks_paths(n, d)
+
+
+def launches_per_multiply(mat, n, d, copies_x=True):
     """Kernel launches one multiply of ``mat`` with an [n, d] matrix issues, by the rules the Python layer
-    applies: one for a small product on a shallow tree; else the copy of X + the SpMM (+ adding the pieces of
-    cut rows), then the walk -- one launch for the path walk of a shallow tree, the levels above the cut + one
-    for the walk by subtrees, or the level-by-level plan."""
+    applies: one for a small product on a shallow tree; else the copy of X (``copies_x``: short rows and
+    small X are gathered in place) + the SpMM (+ adding the pieces of cut rows), then the walk -- one launch
+    for the path walk of a shallow tree, the levels above the cut + one for the walk by subtrees, or the
+    level-by-level plan."""
     tiled_or_cut = mat.is_tiled() or mat.has_cut_rows()
     if not tiled_or_cut and mat._single_launch(n, d):
         return 1
-    launches = 2 + (1 if mat.has_cut_rows() else 0)
+    launches = (2 if copies_x or tiled_or_cut else 1) + (1 if mat.has_cut_rows() else 0)
     if mat.n_levels <= 1:
         return launches
     lo = mat.level_off.tolist()
-    if (mat.is_tiled() or not mat._walks_paths(n, d)) and mat.walk_plan(d) is not None:
-        return launches + level_launches(lo, 1, mat.walk_plan(d)["cut"] + 1) + 1
-    if not tiled_or_cut and mat._walks_paths(n, d):
+    if walks_paths_in_multiply(mat, n, d):
         return launches + 1
+    if mat.walk_plan(d) is not None:
+        return launches + level_launches(lo, 1, mat.walk_plan(d)["cut"] + 1) + 1
     return launches + level_launches(lo, 1, mat.n_levels)
 
 

@@ -70,6 +70,14 @@ def test_launch_count_follows_the_walk_plan():
     assert bench.launches_per_multiply(fake(deep, subtrees=0), 2000, 64) == 2 + 1
     assert bench.launches_per_multiply(fake(deep, subtrees=2), 2000, 64) == 2 + 2 + 1
     assert bench.launches_per_multiply(fake(deep, subtrees=0, paths=True), 2000, 64) == 2 + 1      # the path walk asks first
+    # short rows / a small X are gathered in place: no copy launch
+    assert bench.launches_per_multiply(fake([500]), 500, 64, copies_x=False) == 1
+    assert bench.launches_per_multiply(fake([500, 300, 200], paths=True), 1000, 64, copies_x=False) == 2
+    assert bench.launches_per_multiply(fake(deep, subtrees=0), 2000, 64, copies_x=False) == 1 + 1
+    assert bench.launches_per_multiply(fake([500], cut=True), 500, 64, copies_x=False) == 3       # pieces always go through the copy
+    assert bench.walks_paths_in_multiply(fake([500, 300, 200], paths=True), 1000, 64)
+    assert not bench.walks_paths_in_multiply(fake([500, 300, 200], paths=True, tiled=True), 1000, 64)
+    assert not bench.walks_paths_in_multiply(fake([500], paths=True), 500, 64)
     # a lone narrow level between wide ones is a launch of its own
     assert bench.launches_per_multiply(fake([900, 100, 7, 100]), 2000, 64) == 2 + 3
 
