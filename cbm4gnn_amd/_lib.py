@@ -83,7 +83,24 @@ class CbmWalkDev(C.Structure):
     ]
 
 
+class CbmWalkStream(C.Structure):
+    """Mirror of ``struct cbm_walk_stream`` (host arrays made by ``cbm_walk_stream_build``)."""
+    _fields_ = [
+        ("n", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32), ("n_elems", C.c_int32), ("longest_bin", C.c_int64),
+        ("gidx", C.POINTER(C.c_uint32)), ("ginfo", C.POINTER(C.c_int32)), ("bin_goff", C.POINTER(C.c_int32)),
+    ]
+
+
+class CbmWalkStreamDev(C.Structure):
+    """Mirror of ``struct cbm_walk_stream_dev`` (a multiply stream in device memory)."""
+    _fields_ = [
+        ("n", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32), ("n_elems", C.c_int32),
+        ("gidx", C.c_void_p), ("ginfo", C.c_void_p), ("bin_goff", C.c_void_p),
+    ]
+
+
 CBM_WALK_LOAD_ONLY = 63
+CBM_STREAM_LAST, CBM_STREAM_DUMMY, CBM_STREAM_COL_MASK = 0x40000000, 0x20000000, 0x1FFFFFFF
 CBM_WALK_MAX_SLOTS = 31
 
 _P = C.c_void_p
@@ -105,6 +122,8 @@ HOST_SYMBOLS = {
     "cbm_tiling_free": (None, [C.POINTER(CbmTiling)]),
     "cbm_walk_plan_build": (C.c_int, [_P, _P, _P, _I32, _I32, _I32, _I32, C.POINTER(CbmWalkPlan)]),
     "cbm_walk_plan_free": (None, [C.POINTER(CbmWalkPlan)]),
+    "cbm_walk_stream_build": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, C.POINTER(CbmWalkStream)]),
+    "cbm_walk_stream_free": (None, [C.POINTER(CbmWalkStream)]),
     "cbm_builder_create": (C.c_int, [_P, _P, _I64, _I32, _I32, C.POINTER(_P)]),
     "cbm_builder_arrays": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
                                      C.POINTER(_P), C.POINTER(_I64)]),
@@ -129,6 +148,7 @@ HIP_SYMBOLS = {
     "cbm_relayout_slabs_scaled_f32": (C.c_int, [_P, _P, _P, _I32, _I32, _I64, _P]),
     "cbm_propagate_f32": (C.c_int, [_P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
     "cbm_propagate_subtrees_f32": (C.c_int, [C.POINTER(CbmWalkDev), _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I32, _P]),
+    "cbm_spmm_update_subtrees_f32": (C.c_int, [C.POINTER(CbmWalkStreamDev), _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_paths_f32": (C.c_int, [_P, _P, _I64, _P, _P, _P, _P, _P, _P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),
     "cbm_spmm_update_single_f32": (C.c_int, [_P, _P, _P, _P, _P, _I32, _P, _P, _I32, _I32, _I64, _I64, _I32, _P]),

@@ -590,6 +590,11 @@ class cbm_matrix:
         # per level; "on" / "off" force it; an integer forces it with that cut level.
         self.subtree_walk = "auto"
         self._walk_plans = {}
+        # Deep trees with short delta rows: the whole multiply as ONE launch that walks the subtrees and sums
+        # every row's delta entries on the way (``cbm_spmm_update_subtrees_f32``: the SpMM result never goes to
+        # memory and back).  "auto": when an estimate says the launch is bound by the bytes it moves, not by its
+        # longest bin (see stream_plan); "on": whenever the matrix is neither tiled nor has cut rows; "off".
+        self.stream_multiply = "auto"
         self._batch_rows = DEFAULT_BATCH_ROWS
 
     def _path_gather_ratio(self):
@@ -802,6 +807,87 @@ class cbm_matrix:
                 best = None
             self._walk_plans[key] = best or None
         return self._walk_plans[key]
+
+    # One wavefront alone on its bin streams an entry (one gathered row of X) in about this long; the launch as
+    # a whole moves about this many bytes per microsecond.  Measured on staircase graphs of 11,400 .. 280,000
+    # rows, d = 64 .. 512: the launch takes max(longest bin x the first, bytes / the second) within 10 %.
+    _STREAM_US_PER_ENTRY = 0.105
+    _STREAM_BYTES_PER_US = 6.5e6
+
+    def _host_stream(self, d):
+        """``cbm_walk_stream_build`` for this matrix (CPU tensors + stats), cached per bin target; False when the
+        tree needs more kept values than the kernel has slots (or more than 2^29 rows)."""
+        target_bins = self._walk_bin_target(d)
+        key = ("stream", target_bins)
+        plan = self._walk_plans.get(key)
+        if plan is None:
+            p = _lib.CbmWalkStream()
+            idx = self.idx.contiguous()
+            rc = _lib.host_lib().cbm_walk_stream_build(
+                _ptr(self.rowptr), _ptr(idx), _ptr(self.parent), _ptr(self.order), _ptr(self.level_off), self.num_rows,
+                self.n_levels, target_bins, C.byref(p)) if self.num_rows <= _lib.CBM_STREAM_COL_MASK else 6
+            try:
+                if rc == 6:
+                    plan = False
+                else:
+                    _lib.check(rc, "cbm_walk_stream_build")
+                    take = lambda ptr, count: torch.from_numpy(
+                        np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(np.int32, copy=True))
+                    plan = {"n_bins": int(p.n_bins), "n_slots": int(p.n_slots), "n_elems": int(p.n_elems),
+                            "longest_bin": int(p.longest_bin), "gidx": take(p.gidx, p.n_elems),
+                            "ginfo": take(p.ginfo, 2 * p.n_elems).view(-1, 2), "bin_goff": take(p.bin_goff, p.n_bins + 1)}
+            finally:
+                _lib.host_lib().cbm_walk_stream_free(C.byref(p))
+            self._walk_plans[key] = plan
+        return plan
+
+    def _stream_weights(self):
+        """Stream entries in the subtree of every row (an empty row counts one), int64 NumPy; computed once."""
+        weights = self._walk_plans.get("weights")
+        if weights is None:
+            weights = np.maximum(np.diff(self.rowptr.numpy().astype(np.int64)), 1)
+            lo, order, parent = self.level_off.tolist(), self.order.numpy(), self.parent.numpy()
+            for l in range(self.n_levels - 1, 0, -1):                       # leaves first
+                rows = order[lo[l]:lo[l + 1]]
+                np.add.at(weights, parent[rows], weights[rows])
+            self._walk_plans["weights"] = weights
+        return weights
+
+    def stream_plan(self, d):
+        """The plan of the one-launch multiply by subtrees for width ``d``, or None when the multiply runs as
+        SpMM + walk: by ``stream_multiply`` -- "off": None; "on": the plan whenever the tree has two levels or
+        more and the matrix is neither tiled nor has cut rows; "auto": the plan when, by the shape of the tree
+        and the lengths of the delta rows, the launch is bound by the bytes it moves (every delta entry's row
+        of X once, every row of Y once) rather than by the wavefront with the longest bin -- then it moves
+        fewer bytes than the SpMM and the walk apart, which write and re-read the SpMM result."""
+        policy = self.stream_multiply
+        if policy == "off" or self.n_levels < 2 or self.num_rows == 0 or d <= 0:
+            return None
+        if policy not in ("auto", "on"):
+            raise ValueError('stream_multiply must be "auto", "on" or "off"')
+        if self._host_tiling():
+            return None
+        key = ("stream-choice", policy, (d + 63) // 64, d if policy == "auto" else 0)
+        if key not in self._walk_plans:
+            take = True
+            if policy == "auto":
+                weights, target = self._stream_weights(), self._walk_bin_target(d)
+                heads = weights[self.order.numpy()[:int(self.level_off[1])]]
+                total = int(heads.sum())
+                longest = max(int(heads.max()), -(-total // target), 64)      # small subtrees are packed into bins
+                take = longest * self._STREAM_US_PER_ENTRY <= (total + self.num_rows) * d * 4 / self._STREAM_BYTES_PER_US
+            self._walk_plans[key] = (self._host_stream(d) or None) if take else None
+        return self._walk_plans[key]
+
+    def _stream_struct(self, st, plan):
+        """``struct cbm_walk_stream_dev`` over the device copy of ``plan`` (uploaded once per device)."""
+        key = ("stream", plan["n_bins"], plan["n_elems"])
+        dev = st.get(key)
+        if dev is None:
+            device = st["rowptr"].device
+            dev = st[key] = (plan["gidx"].to(device), plan["ginfo"].contiguous().to(device), plan["bin_goff"].to(device))
+        return _lib.CbmWalkStreamDev(self.num_rows, plan["n_bins"], plan["n_slots"], plan["n_elems"], dev[0].data_ptr(),
+                                     dev[1].data_ptr(), dev[2].data_ptr())
 
     def _subtree_sizes(self):
         """Rows in the subtree of every row (itself included), int64 NumPy; computed once."""
@@ -1150,6 +1236,17 @@ class cbm_matrix:
             if yd is not y:
                 y.copy_(yd)
             return
+        if st["tiled"] is None and workspace is None and not workspace_ready:
+            sp = self.stream_plan(x.size(1))
+            if sp is not None:                                  # a deep tree, short delta rows: one launch does it all
+                with torch.cuda.device(xd.device):
+                    rc = _lib.hip_lib().cbm_spmm_update_subtrees_f32(
+                        C.byref(self._stream_struct(st, sp)), _ptr(st["m"]) if use_m else None, _ptr(xd), _ptr(yd), n,
+                        x.size(1), _ld(xd), _ld(yd), _lib.CBM_UPDATE_RELU if relu else 0, _stream(xd.device))
+                _lib.check(rc, "cbm_spmm_update_subtrees_f32")
+                if yd is not y:
+                    y.copy_(yd)
+                return
         if (tiled or not self._walks_paths(n, x.size(1))) and self.walk_plan(x.size(1)) is not None:
             # a deep tree: the SpMM (root children scaled in its epilogue), then the walk by subtrees
             self._run_spmm(xd, yd, use_m, scale_roots=use_m, workspace=workspace, workspace_ready=workspace_ready,

@@ -788,18 +788,23 @@ void cbm_walk_plan_free(cbm_walk_plan* p) {
     std::memset(p, 0, sizeof(*p));
 }
 
-int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32_t* level_off, int32_t n,
-                        int32_t n_levels, int32_t cut, int32_t target_bins, cbm_walk_plan* out) {
-    if (!out) return CBM_ERR_NULL;
-    std::memset(out, 0, sizeof(*out));
-    if (!parent || !order || !level_off) return CBM_ERR_NULL;
-    if (n <= 0 || n_levels < 1 || cut < 0 || cut >= n_levels || target_bins < 1) return CBM_ERR_SHAPE;
-    if (level_off[0] != 0 || level_off[n_levels] != n) return CBM_ERR_SHAPE;
-    for (int32_t l = 0; l < n_levels; l++)
-        if (level_off[l + 1] < level_off[l]) return CBM_ERR_SHAPE;
-    try {
+}  // extern "C"
+
+namespace {
+
+// The arborescence as child lists, for the plans that walk it depth-first.
+struct WalkTree {
+    std::vector<int32_t> level, child_ptr, child, size;
+
+    // Validates parent / order / level_off against each other and builds the child lists, lightest subtree
+    // first (ties by id): the value of a row then has to be kept only while the walk is inside one of its
+    // lighter children, which bounds the kept values by log2(subtree size).
+    int build(const int32_t* parent, const int32_t* order, const int32_t* level_off, int32_t n, int32_t n_levels) {
+        if (level_off[0] != 0 || level_off[n_levels] != n) return CBM_ERR_SHAPE;
+        for (int32_t l = 0; l < n_levels; l++)
+            if (level_off[l + 1] < level_off[l]) return CBM_ERR_SHAPE;
         // level of every row; order must be a permutation whose rows sit one level below their parents
-        std::vector<int32_t> level(n, -1);
+        level.assign(n, -1);
         for (int32_t l = 0; l < n_levels; l++)
             for (int32_t i = level_off[l]; i < level_off[l + 1]; i++) {
                 const int32_t v = order[i];
@@ -812,7 +817,9 @@ int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32
             if (u < 0 ? level[v] != 0 : level[u] + 1 != level[v]) return CBM_ERR_SHAPE;
         }
         // children lists (CSR by parent) and subtree sizes (leaves first: order[] backwards)
-        std::vector<int32_t> child_ptr(n + 1, 0), child(n > 0 ? n : 1), size(n, 1);
+        child_ptr.assign(n + 1, 0);
+        child.assign(n > 0 ? n : 1, 0);
+        size.assign(n, 1);
         for (int32_t v = 0; v < n; v++)
             if (parent[v] >= 0) child_ptr[parent[v] + 1]++;
         for (int32_t v = 0; v < n; v++) child_ptr[v + 1] += child_ptr[v];
@@ -825,11 +832,71 @@ int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32
             const int32_t v = order[i];
             if (parent[v] >= 0) size[parent[v]] += size[v];
         }
-        // lightest child first, heaviest last (ties by id): the value of a row then has to be kept only while
-        // the walk is inside one of its lighter children, which bounds the kept values by log2(subtree size)
         for (int32_t v = 0; v < n; v++)
             std::sort(child.begin() + child_ptr[v], child.begin() + child_ptr[v + 1],
                       [&](int32_t a, int32_t b) { return size[a] != size[b] ? size[a] < size[b] : a < b; });
+        return CBM_OK;
+    }
+
+    // The subtree of r in depth-first pre-order as { row, ctl } pairs (ctl as in struct cbm_walk_plan), handed
+    // to put(row, ctl) one by one.  False if a row would need more than CBM_WALK_MAX_SLOTS kept values.
+    template <class Put>
+    bool emit(int32_t r, int32_t& max_slots, Put put) {
+        int32_t kept = 0;                                  // rows on the current path whose value sits in a slot
+        {
+            int32_t ctl = CBM_WALK_LOAD_ONLY;
+            if (child_ptr[r + 1] - child_ptr[r] >= 2) { kept++; ctl |= kept << 8; }
+            put(r, ctl);
+        }
+        stack.clear();
+        slot_of_depth.clear();
+        stack.emplace_back(r, 0);
+        slot_of_depth.push_back(kept);                     // slot of the stack's rows (0 = none)
+        max_slots = std::max(max_slots, kept);
+        while (!stack.empty()) {
+            const int32_t u = stack.back().first;
+            const int32_t i = stack.back().second;
+            const int32_t k = child_ptr[u + 1] - child_ptr[u];
+            if (i == k) { stack.pop_back(); slot_of_depth.pop_back(); continue; }
+            stack.back().second = i + 1;
+            const int32_t v = child[child_ptr[u] + i];
+            // source of the parent's value: the row visited just before (first child), else the parent's slot;
+            // the last child frees that slot before taking one of its own
+            int32_t ctl = (i == 0) ? 0 : slot_of_depth.back();
+            if (i == k - 1 && k >= 2) kept--;
+            const int32_t kv = child_ptr[v + 1] - child_ptr[v];
+            int32_t mine = 0;
+            if (kv >= 2) {
+                mine = ++kept;
+                if (mine > CBM_WALK_MAX_SLOTS) return false;
+                max_slots = std::max(max_slots, mine);
+                ctl |= mine << 8;
+            }
+            put(v, ctl);
+            if (kv > 0) { stack.emplace_back(v, 0); slot_of_depth.push_back(mine); }
+        }
+        return true;
+    }
+
+private:
+    std::vector<std::pair<int32_t, int32_t>> stack;        // (row, next child to visit)
+    std::vector<int32_t> slot_of_depth;
+};
+
+}  // namespace
+
+extern "C" {
+
+int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32_t* level_off, int32_t n,
+                        int32_t n_levels, int32_t cut, int32_t target_bins, cbm_walk_plan* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if (!parent || !order || !level_off) return CBM_ERR_NULL;
+    if (n <= 0 || n_levels < 1 || cut < 0 || cut >= n_levels || target_bins < 1) return CBM_ERR_SHAPE;
+    try {
+        WalkTree tree;
+        if (int rc = tree.build(parent, order, level_off, n, n_levels)) return rc;
+        const std::vector<int32_t>& size = tree.size;
         // tasks: the rows of level `cut` that have children, longest subtree first (ties by id)
         std::vector<int32_t> roots;
         for (int32_t i = level_off[cut]; i < level_off[cut + 1]; i++)
@@ -847,46 +914,14 @@ int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32
         std::vector<int32_t> bin_off(1, 0);
         int64_t at = 0, in_bin = 0, longest = 0;
         int32_t max_slots = 0;
-        std::vector<std::pair<int32_t, int32_t>> stack;    // (row, next child to visit)
         for (int32_t r : roots) {
             if (in_bin >= target) { bin_off.push_back((int32_t)at); longest = std::max(longest, in_bin); in_bin = 0; }
             in_bin += size[r];
-            // iterative pre-order walk; `kept` = rows on the current path whose value sits in a slot
-            int32_t kept = 0;
-            out->entries[2 * at] = r; out->entries[2 * at + 1] = CBM_WALK_LOAD_ONLY; 
-            {
-                const int32_t k = child_ptr[r + 1] - child_ptr[r];
-                if (k >= 2) { kept++; out->entries[2 * at + 1] |= kept << 8; }
-            }
-            at++;
-            stack.clear();
-            stack.emplace_back(r, 0);
-            std::vector<int32_t> slot_of_depth;            // slot of the stack's rows (0 = none)
-            slot_of_depth.push_back(kept);
-            max_slots = std::max(max_slots, kept);
-            while (!stack.empty()) {
-                const int32_t u = stack.back().first;
-                const int32_t i = stack.back().second;
-                const int32_t k = child_ptr[u + 1] - child_ptr[u];
-                if (i == k) { stack.pop_back(); slot_of_depth.pop_back(); continue; }
-                stack.back().second = i + 1;
-                const int32_t v = child[child_ptr[u] + i];
-                // source of the parent's value: the row visited just before (first child), else the parent's slot;
-                // the last child frees that slot before taking one of its own
-                int32_t ctl = (i == 0) ? 0 : slot_of_depth.back();
-                if (i == k - 1 && k >= 2) kept--;
-                const int32_t kv = child_ptr[v + 1] - child_ptr[v];
-                int32_t mine = 0;
-                if (kv >= 2) {
-                    mine = ++kept;
-                    if (mine > CBM_WALK_MAX_SLOTS) return (cbm_walk_plan_free(out), CBM_ERR_UNSUPPORTED);
-                    max_slots = std::max(max_slots, mine);
-                    ctl |= mine << 8;
-                }
-                out->entries[2 * at] = v; out->entries[2 * at + 1] = ctl;
+            const bool fits = tree.emit(r, max_slots, [&](int32_t row, int32_t ctl) {
+                out->entries[2 * at] = row; out->entries[2 * at + 1] = ctl;
                 at++;
-                if (kv > 0) { stack.emplace_back(v, 0); slot_of_depth.push_back(mine); }
-            }
+            });
+            if (!fits) return (cbm_walk_plan_free(out), CBM_ERR_UNSUPPORTED);
         }
         if (at != total) return (cbm_walk_plan_free(out), CBM_ERR_INTERNAL);
         if (total > 0) { bin_off.push_back((int32_t)at); longest = std::max(longest, in_bin); }
@@ -899,6 +934,102 @@ int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32
         return CBM_OK;
     } catch (const std::bad_alloc&) {
         cbm_walk_plan_free(out);
+        return CBM_ERR_ALLOC;
+    }
+}
+
+void cbm_walk_stream_free(cbm_walk_stream* p) {
+    if (!p) return;
+    free(p->gidx); free(p->ginfo); free(p->bin_goff);
+    std::memset(p, 0, sizeof(*p));
+}
+
+int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int32_t* parent, const int32_t* order,
+                          const int32_t* level_off, int32_t n, int32_t n_levels, int32_t target_bins,
+                          cbm_walk_stream* out) {
+    if (!out) return CBM_ERR_NULL;
+    std::memset(out, 0, sizeof(*out));
+    if (!rowptr || !parent || !order || !level_off) return CBM_ERR_NULL;
+    if (n <= 0 || n_levels < 1 || target_bins < 1 || (uint32_t)n > CBM_STREAM_COL_MASK) return CBM_ERR_SHAPE;
+    if (rowptr[0] != 0) return CBM_ERR_SHAPE;
+    for (int32_t r = 0; r < n; r++)
+        if (rowptr[r + 1] < rowptr[r]) return CBM_ERR_SHAPE;
+    if (rowptr[n] > 0 && !idx) return CBM_ERR_NULL;
+    for (int64_t k = 0; k < rowptr[n]; k++)
+        if ((idx[k] & 0x7fffffffu) >= (uint32_t)n) return CBM_ERR_SHAPE;
+    try {
+        WalkTree tree;
+        if (int rc = tree.build(parent, order, level_off, n, n_levels)) return rc;
+        // a row costs its delta entries (an empty row one stand-in entry); a subtree the sum over its rows
+        std::vector<int64_t> weight(n);
+        int64_t total = 0;
+        for (int32_t v = 0; v < n; v++) total += weight[v] = std::max(rowptr[v + 1] - rowptr[v], 1);
+        if (total > INT32_MAX) return CBM_ERR_SHAPE;
+        for (int32_t i = n - 1; i >= 0; i--) {
+            const int32_t v = order[i];
+            if (parent[v] >= 0) weight[parent[v]] += weight[v];
+        }
+        // tasks: every child of the root, heaviest subtree first (ties by id)
+        std::vector<int32_t> roots(order, order + level_off[1]);
+        std::sort(roots.begin(), roots.end(),
+                  [&](int32_t a, int32_t b) { return weight[a] != weight[b] ? weight[a] > weight[b] : a < b; });
+        // bins: consecutive tasks of the sorted list until a bin holds `target` stream entries
+        const int64_t target = std::max<int64_t>((total + target_bins - 1) / target_bins, CBM_STREAM_MIN_BIN);
+        std::vector<int32_t> entries;                      // { row, ctl } in walk order
+        entries.reserve(2 * (size_t)n);
+        std::vector<int32_t> bin_first(1, 0);              // first row (position in entries) of every bin
+        int64_t in_bin = 0;
+        int32_t max_slots = 0;
+        for (int32_t r : roots) {
+            if (in_bin >= target) { bin_first.push_back((int32_t)(entries.size() / 2)); in_bin = 0; }
+            in_bin += weight[r];
+            if (!tree.emit(r, max_slots, [&](int32_t row, int32_t ctl) { entries.push_back(row); entries.push_back(ctl); }))
+                return CBM_ERR_UNSUPPORTED;
+        }
+        if (entries.size() != 2 * (size_t)n) return CBM_ERR_INTERNAL;
+        bin_first.push_back(n);
+        const int32_t n_bins = (int32_t)bin_first.size() - 1;
+        out->n = n; out->n_bins = n_bins; out->n_slots = max_slots; out->n_elems = (int32_t)total;
+        out->gidx = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)total);
+        out->ginfo = (int32_t*)calloc(2 * (size_t)total, sizeof(int32_t));   // zeroed: "no row landed here"
+        out->bin_goff = (int32_t*)malloc(sizeof(int32_t) * ((size_t)n_bins + 1));
+        if (!out->gidx || !out->ginfo || !out->bin_goff) throw std::bad_alloc();
+        int64_t g = 0, longest = 0;
+        for (int32_t b = 0; b < n_bins; b++) {
+            const int64_t g0 = g;
+            out->bin_goff[b] = (int32_t)g0;
+            int64_t stretch = -1;
+            int32_t in_stretch = 0;
+            for (int32_t k = bin_first[b]; k < bin_first[b + 1]; k++) {
+                const int32_t row = entries[2 * (size_t)k], ctl = entries[2 * (size_t)k + 1];
+                const int32_t len = rowptr[row + 1] - rowptr[row];
+                if (len == 0) {
+                    out->gidx[g++] = (uint32_t)row | CBM_STREAM_DUMMY | CBM_STREAM_LAST;
+                } else {
+                    for (int32_t e = 0; e < len; e++) out->gidx[g++] = idx[rowptr[row] + e];
+                    out->gidx[g - 1] |= CBM_STREAM_LAST;
+                }
+                // the rows that end inside a stretch of 64 entries, in order, sit at the head of that stretch
+                const int64_t s = (g - 1 - g0) / 64;
+                if (s != stretch) { stretch = s; in_stretch = 0; }
+                int32_t* info = out->ginfo + 2 * (g0 + s * 64 + in_stretch++);
+                info[0] = row; info[1] = ctl | INT32_MIN;  // marked: a slot that is in use
+            }
+            longest = std::max(longest, g - g0);
+            // slots no row landed in: a valid row (the kernel loads them, and m of their row, without using them)
+            const int32_t filler = entries[2 * (size_t)bin_first[b]];
+            for (int64_t q = g0; q < g; q++) {
+                int32_t* info = out->ginfo + 2 * q;
+                if (info[1] < 0) info[1] &= INT32_MAX;
+                else { info[0] = filler; info[1] = 0; }
+            }
+        }
+        if (g != total) return (cbm_walk_stream_free(out), CBM_ERR_INTERNAL);
+        out->bin_goff[n_bins] = (int32_t)total;
+        out->longest_bin = longest;
+        return CBM_OK;
+    } catch (const std::bad_alloc&) {
+        cbm_walk_stream_free(out);
         return CBM_ERR_ALLOC;
     }
 }

@@ -1162,6 +1162,122 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     }
 }
 
+// The whole multiply of a DEEP tree with SHORT delta rows in one launch: the walk of propagate_subtrees with
+// the SpMM result of a row summed on the spot instead of read back.  The host lays the delta entries of a
+// bin's rows end to end in the order the walk visits them (gidx: col | sign << 31, kStreamLast on a row's
+// last entry, kStreamDummy on the one stand-in entry of an empty row); a wavefront streams that list 64 entries
+// at a time, lane l decoding entry l (its coefficient +-1 or +-m[col], the byte offset of row col of X), and
+// gathers its 64 feature columns of every entry's row half a stretch ahead of their use, unconditionally.  The
+// sum of a row runs strictly in entry order (fma(coef, x, acc) from zero: the order of spmm_wave_per_row);
+// when its last entry is in, the row takes its walk step exactly as in propagate_subtrees (the head of a
+// subtree is a child of the root: its sum times m) and is stored once -- through the ReLU if asked, the raw
+// value staying in the register / LDS slot its children read.  ginfo holds, per stretch of 64 entries, the
+// {row, ctl} of the rows that end inside it, in order.  Z never exists in memory.
+constexpr uint32_t kStreamLast = CBM_STREAM_LAST, kStreamDummy = CBM_STREAM_DUMMY, kStreamCol = CBM_STREAM_COL_MASK;
+
+template <bool NORM>
+__global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
+    const uint32_t* __restrict__ gidx, const int2* __restrict__ ginfo, const int32_t* __restrict__ bin_goff, int n_bins,
+    int slices, const float* __restrict__ m, const float* __restrict__ X, float* __restrict__ Y, int d, int dv, int64_t ldx,
+    int64_t ldy, int n_slots, int relu) {
+    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int w = blockIdx.x * kSubWaves + (threadIdx.x >> 6);
+    const int bin = w / slices;
+    if (bin >= n_bins) return;
+    const int j = (w % slices) * kWave + lane;                    // feature column of this thread
+    const bool live = j < d;
+    const int jj = live ? j : 0;                                  // lanes past d gather column 0 and store nothing
+    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
+    const int first = bin_goff[bin], count = bin_goff[bin + 1] - first;
+    auto at = [&](int base) -> int { return first + min(base + lane, count - 1); };   // past the end: the last entry
+    auto bcast64 = [&](int64_t off_ids, int k) -> int64_t {
+        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)off_ids, k);
+        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)((uint64_t)off_ids >> 32), k);
+        return (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+    const uint32_t jj4 = (uint32_t)jj * 4u;
+    auto x_off = [&](uint32_t p) -> int64_t { return (int64_t)(p & kStreamCol) * ldx * 4; };
+    auto coef = [&](uint32_t p) -> float {
+        uint32_t mag = 0x3f800000u;
+        if constexpr (NORM) mag = __float_as_uint(m[p & kStreamCol]);
+        return __uint_as_float(mag ^ (p & 0x80000000u));
+    };
+    auto request = [&](float (&z)[kChainHalf], int64_t xo_ids, int half) {
+#pragma unroll
+        for (int u = 0; u < kChainHalf; u++)
+            z[u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(X) + bcast64(xo_ids, half * kChainHalf + u) + jj4);
+    };
+    float acc = 0.0f, run = 0.0f, mu = 1.0f;
+    int rs = 0;                                                   // rows finished in the current stretch (wave-uniform)
+    auto consume = [&](const float (&z)[kChainHalf], uint32_t p_ids, float f_ids, int2 i_ids, float mr_ids, int base, int half) {
+#pragma unroll
+        for (int u = 0; u < kChainHalf; u++) {
+            const int k = half * kChainHalf + u;
+            if (base + k < count) {
+                const uint32_t p = (uint32_t)bcast_i((int)p_ids, k);          // wave-uniform: the branches are scalar
+                if (!(p & kStreamDummy)) acc = fmaf(bcast_f(f_ids, k), z[u], acc);
+                if (p & kStreamLast) {
+                    const int ctl = bcast_i(i_ids.y, rs);
+                    const int src = ctl & 63, dst = (ctl >> 8) & 63;
+                    const float mv = NORM ? bcast_f(mr_ids, rs) : 1.0f;
+                    if (src == CBM_WALK_LOAD_ONLY) {                          // a child of the root
+                        run = NORM ? acc * mv : acc;
+                    } else {
+                        float a = run, ma = mu;
+                        if (src) {
+                            a = st[(src - 1) * 2 * kWave];
+                            if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
+                        }
+                        if constexpr (NORM) {
+                            const float inv_mu = 1.0f / ma;
+                            run = (jj < dv) ? fmaf(a, inv_mu, acc) * mv : (acc + a / ma) * mv;
+                        } else {
+                            run = acc + a;
+                        }
+                    }
+                    if (live) {
+                        float* yr = reinterpret_cast<float*>(reinterpret_cast<char*>(Y) + (int64_t)bcast_i(i_ids.x, rs) * ldy * 4 + jj4);
+                        *yr = (relu && run < 0.0f) ? 0.0f : run;              // keeps NaN, as torch.relu does
+                    }
+                    mu = mv;
+                    if (dst) {
+                        st[(dst - 1) * 2 * kWave] = run;
+                        if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
+                    }
+                    acc = 0.0f;
+                    rs++;
+                }
+            }
+        }
+    };
+    uint32_t p_cur = gidx[at(0)], p_nxt = gidx[at(kWave)];
+    int2 i_cur = ginfo[at(0)], i_nxt = ginfo[at(kWave)];
+    float f_cur = coef(p_cur), mr_cur = 1.0f;
+    if constexpr (NORM) mr_cur = m[i_cur.x];
+    int64_t xo_cur = x_off(p_cur), xo_nxt = x_off(p_nxt);
+    float za[kChainHalf], zb[kChainHalf];
+    request(za, xo_cur, 0);
+    for (int base = 0; base < count; base += kWave) {
+        // requested first, needed last: the entries and rows of the stretch after the next, and what depends on
+        // the next stretch's (their entries came in an iteration ago)
+        const uint32_t p_far = gidx[at(base + 2 * kWave)];
+        const int2 i_far = ginfo[at(base + 2 * kWave)];
+        const float f_nxt = coef(p_nxt);
+        float mr_nxt = 1.0f;
+        if constexpr (NORM) mr_nxt = m[i_nxt.x];
+        request(zb, xo_cur, 1);
+        rs = 0;
+        consume(za, p_cur, f_cur, i_cur, mr_cur, base, 0);
+        request(za, xo_nxt, 0);
+        consume(zb, p_cur, f_cur, i_cur, mr_cur, base, 1);
+        p_cur = p_nxt; p_nxt = p_far;
+        i_cur = i_nxt; i_nxt = i_far;
+        f_cur = f_nxt; mr_cur = mr_nxt;
+        xo_cur = xo_nxt; xo_nxt = x_off(p_far);
+    }
+}
+
 // The walk of a SHALLOW tree in one launch, out of place: the wavefront of row v follows parent[]
 // up to the child of the root above it (at most kMaxPathLevels - 1 steps, the ids kept one per
 // lane), then adds the rows of Z down that path with exactly the arithmetic of propagate_row, so
@@ -1877,6 +1993,21 @@ int launch_subtrees(const cbm_walk_dev* w, const float* m, float* Y, int32_t d, 
     return check_launch();
 }
 
+template <bool NORM>
+int launch_stream(const cbm_walk_stream_dev* w, const float* m, const float* X, float* Y, int32_t d, int64_t ldx,
+                  int64_t ldy, int relu, hipStream_t s) {
+    if (w->n_bins == 0) return CBM_OK;
+    const int slices = (d + kWave - 1) / kWave;
+    const int64_t waves = (int64_t)w->n_bins * slices;
+    const int64_t blocks = (waves + kSubWaves - 1) / kSubWaves;
+    if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
+    const size_t lds = (size_t)kSubWaves * w->n_slots * 2 * kWave * sizeof(float);       // at most 62 KB
+    hipLaunchKernelGGL((spmm_update_subtrees<NORM>), dim3((unsigned)blocks), dim3(kWave * kSubWaves), lds, s, w->gidx,
+                       reinterpret_cast<const int2*>(w->ginfo), w->bin_goff, w->n_bins, slices, m, X, Y, d, d - d % 8, ldx,
+                       ldy, w->n_slots, relu);
+    return check_launch();
+}
+
 }  // namespace
 
 extern "C" {
@@ -2069,6 +2200,24 @@ int cbm_propagate_subtrees_f32(const cbm_walk_dev* walk, const int32_t* parent, 
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
     hipLaunchKernelGGL(relu_rows, dim3((unsigned)blocks), dim3(256), 0, s, Y, total, d, ldy);
     return check_launch();
+}
+
+int cbm_spmm_update_subtrees_f32(const cbm_walk_stream_dev* ws, const float* m, const float* X, float* Y, int32_t n,
+                                 int32_t d, int64_t ldx, int64_t ldy, int32_t flags, void* stream) {
+    if (!ws || !X || !Y) return CBM_ERR_NULL;
+    if (int rc = check_matrix(n, d, ldx)) return rc;
+    if (int rc = check_matrix(n, d, ldy)) return rc;
+    if (flags & ~CBM_UPDATE_RELU) return CBM_ERR_UNSUPPORTED;
+    if (X == Y) return CBM_ERR_SHAPE;                    // rows of Y are stored while rows of X are still gathered
+    if (n == 0 || d == 0) return CBM_OK;
+    if (ws->n != n || ws->n_bins < 0 || ws->n_elems < 0 || ws->n_slots < 0 || ws->n_slots > CBM_WALK_MAX_SLOTS)
+        return CBM_ERR_SHAPE;
+    if ((uint32_t)n > kStreamCol) return CBM_ERR_SHAPE;  // the column shares its word with two flags and the sign
+    if (ws->n_bins > 0 && (!ws->gidx || !ws->ginfo || !ws->bin_goff || !aligned(ws->ginfo, 8))) return CBM_ERR_NULL;
+    if ((int64_t)n * ldy * 4 > ((int64_t)1 << 46) || (int64_t)n * ldx * 4 > ((int64_t)1 << 46)) return CBM_ERR_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int relu = (flags & CBM_UPDATE_RELU) != 0;
+    return m ? launch_stream<true>(ws, m, X, Y, d, ldx, ldy, relu, s) : launch_stream<false>(ws, m, X, Y, d, ldx, ldy, relu, s);
 }
 
 int cbm_spmm_update_f32(const int32_t* rowptr, const uint32_t* idx, int64_t nnz, const float* m, const float* coef,

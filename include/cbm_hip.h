@@ -273,6 +273,39 @@ int cbm_walk_plan_build(const int32_t* parent, const int32_t* order, const int32
                         int32_t n_levels, int32_t cut, int32_t target_bins, cbm_walk_plan* out);
 void cbm_walk_plan_free(cbm_walk_plan* p);
 
+/* Plan of the ONE-LAUNCH multiply by subtrees (cbm_spmm_update_subtrees_f32), for deep trees whose delta rows
+ * are short: the walk plan at cut 0 extended to every child of the root (also those without children), with
+ * the delta entries of the rows laid end to end in walk order, so that a wavefront streams them, sums a row
+ * on the spot and takes its walk step without the SpMM result ever going through memory.
+ *   gidx       [n_elems] uint32: the delta entries (col | sign << 31, as idx) of a bin's rows in walk order;
+ *              CBM_STREAM_LAST marks a row's last entry; an empty row has one stand-in entry with
+ *              CBM_STREAM_DUMMY (| LAST) whose column is the row itself and which adds nothing
+ *   ginfo      [n_elems][2] int32 { row, ctl } (ctl as in cbm_walk_plan.entries; CBM_WALK_LOAD_ONLY = a child of
+ *              the root: its sum, times m[row] when normalised, is its value): for every stretch of 64 stream
+ *              entries of a bin, the rows that END inside that stretch, in order, starting at the stretch's
+ *              first position; positions no row landed in hold { first row of the bin, 0 }
+ *   bin_goff   [n_bins + 1] offsets into gidx / ginfo: a bin is what one wavefront streams (whole subtrees,
+ *              heaviest first by stream entries, small ones packed together up to about n_elems / target_bins)
+ *   n_slots    most LDS slots any subtree uses;  longest_bin  stream entries of the longest bin
+ * n must be below 2^29 (the column shares its word with the sign and the two marks).  HOST pointers; release
+ * with cbm_walk_stream_free.  CBM_ERR_UNSUPPORTED as for cbm_walk_plan_build.  No reference counterpart: the
+ * reference keeps the SpMM (MKL) and the walk apart (cbm_extensions.cpp:1133-1218). */
+#define CBM_STREAM_LAST 0x40000000u
+#define CBM_STREAM_DUMMY 0x20000000u
+#define CBM_STREAM_COL_MASK 0x1fffffffu
+#define CBM_STREAM_MIN_BIN 64
+typedef struct cbm_walk_stream {
+    int32_t n, n_bins, n_slots, n_elems;
+    int64_t longest_bin;
+    uint32_t* gidx;
+    int32_t* ginfo;
+    int32_t* bin_goff;
+} cbm_walk_stream;
+int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int32_t* parent, const int32_t* order,
+                          const int32_t* level_off, int32_t n, int32_t n_levels, int32_t target_bins,
+                          cbm_walk_stream* out);
+void cbm_walk_stream_free(cbm_walk_stream* p);
+
 /* ------------------------------------------------------------------ libcbm_hip.so ----------- */
 
 const char* cbm_version(void);
@@ -411,6 +444,26 @@ int cbm_propagate_subtrees_f32(const cbm_walk_dev* walk, const int32_t* parent_d
                                const int32_t* level_off_dev, const int32_t* level_off_host, int32_t n_levels,
                                const float* m_dev, float* Y_dev, int32_t n, int32_t d, int64_t ldy, int32_t flags,
                                void* stream);
+
+/* A multiply stream (cbm_walk_stream_build) in DEVICE memory.  The struct itself lives in HOST memory. */
+typedef struct cbm_walk_stream_dev {
+    int32_t n, n_bins, n_slots, n_elems;
+    const uint32_t* gidx;       /* [n_elems] */
+    const int32_t* ginfo;       /* [n_elems][2], 8-byte aligned */
+    const int32_t* bin_goff;    /* [n_bins + 1] */
+} cbm_walk_stream_dev;
+
+/* Y = A_hat * X in ONE launch for a deep tree with short delta rows: one wavefront per (bin of the stream,
+ * 64 feature columns) walks its subtrees depth-first and sums every row's delta entries on the spot, so the
+ * SpMM result never goes to memory and back.  A row's sum runs strictly in entry order (fma(+-1 or +-m[col],
+ * x, acc) from zero, the reference's per-entry arithmetic, cbm_extensions.cpp:504-585); the walk step per
+ * row is that of cbm_propagate_f32.  flags: CBM_UPDATE_RELU (in the store; children still read the raw
+ * value).  X must not alias Y.
+ * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);
+ * m != NULL replaces seq_/omp_s_fused_spmm_update_csr_int32_ (:845-996, :1224-1374). */
+int cbm_spmm_update_subtrees_f32(const cbm_walk_stream_dev* stream_plan, const float* m_dev, const float* X_dev,
+                                 float* Y_dev, int32_t n, int32_t d, int64_t ldx, int64_t ldy, int32_t flags,
+                                 void* stream);
 
 /* Y = A_hat * X in one call: cbm_spmm_f32 followed by cbm_propagate_f32 on the same stream.
  * m == NULL replaces seq_/omp_s_spmm_update_csr_int32_ (cbm_extensions.cpp:650-740, :1108-1219);

@@ -307,8 +307,8 @@ def test_duplication_graph_at_the_configured_size():
 
 
 def test_deep_and_wide_tree_full_size():
-    """c6: 182,400 rows in 800 staircases + noise, compression 9.4, 65 tree levels of ~3,000 rows: the walk by
-    subtrees (one launch) against the level-by-level walk bit for bit, 1,024 rows against fp64 SciPy rows, the
+    """c6: 182,400 rows in 800 staircases + noise, compression 9.4, 65 tree levels of ~3,000 rows: the one-launch
+    multiply by subtrees against the SpMM + walk, the walk by subtrees against the level-by-level walk bit for bit, 1,024 rows against fp64 SciPy rows, the
     whole product against the GPU CSR baseline; short delta rows in batches against one row per wavefront."""
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
@@ -320,6 +320,7 @@ def test_deep_and_wide_tree_full_size():
     assert int((widths > 64).sum()) >= 50
     plan = mat.walk_plan(w.d)
     assert plan is not None and plan["cut"] == 0 and plan["n_bins"] > 1000      # "auto" takes the subtree walk
+    assert mat.stream_plan(w.d) is not None                  # and, before it, the one-launch multiply by subtrees
     rp, col = _csr(w.edge_index, w.n)
     m = mat.col_multiplier.numpy()
     x = w.features(0)
@@ -333,6 +334,11 @@ def test_deep_and_wide_tree_full_size():
     base = torch.empty_like(xd)
     csr_spmm(torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda(), val, xd, base)
     assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+    print("[gpu-case] c6 full size, SpMM + walk by subtrees", flush=True); sys.stdout.flush()
+    mat.stream_multiply = "off"                              # the SpMM and the walk apart: another summation order
+    one_launch, got = got, _mul(mat, xd)
+    assert float((one_launch - got).abs().max() / got.abs().max()) <= 1e-5
+    _assert_rows_close(got[rows_d].cpu().numpy().astype(np.float64), _rows_fp64(rp, col, m, x.numpy(), rows))
     mat.subtree_walk = "off"
     print("[gpu-case] c6 full size, level-by-level walk", flush=True); sys.stdout.flush()
     assert torch.equal(_mul(mat, xd), got)

@@ -75,6 +75,14 @@ def brings_workspace(relayout, nnz, n, d, ld=None):
     return bool(relayout) and n > 0 and (nnz >= need * n or groups_for(d, ld) == 1)
 
 
+def takes_stream(mat, d):
+    """Whether ``*_spmm_update`` of width ``d`` runs as the one-launch multiply by subtrees (the Python layer's
+    rule: after the single launch of small products, for matrices that are neither tiled nor have cut rows)."""
+    if mat.is_tiled() or mat.has_cut_rows() or mat._single_launch(mat.num_rows, d):
+        return False
+    return mat.stream_plan(d) is not None
+
+
 def mat_groups(mat, d, ld=None, update=False):
     """The same for a multiply through ``cbm_matrix``, which brings a workspace when rows are long enough.
     ``update``: the whole product (``*_spmm_update``), which for small products on shallow, sparse trees is
@@ -82,11 +90,15 @@ def mat_groups(mat, d, ld=None, update=False):
     n = mat.num_rows
     if update and not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(n, d):
         return 1
+    if update and takes_stream(mat, d):                     # every row strictly in entry order
+        return 1
     return groups_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, n, d, ld))
 
 
 def mat_tail(mat, d, ld=None, update=False):
     if update and not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(mat.num_rows, d):
+        return 0
+    if update and takes_stream(mat, d):
         return 0
     return tail_for(d, ld, workspace=brings_workspace(mat.relayout, mat.nnz, mat.num_rows, d, ld))
 
@@ -503,7 +515,7 @@ def test_deep_chain_uses_the_chain_kernel(orc):
     for normalized, d in ((False, 512), (True, 96), (True, 41), (False, 10), (True, 1100)):
         e2 = graphs.add_self_loops(ei, n) if normalized else ei
         mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
-        mat.subtree_walk = "off"                           # this test is about the level plan's chain kernel
+        mat.subtree_walk = mat.stream_multiply = "off"     # this test is about the level plan's chain kernel
         assert mat.n_levels >= 151
         widths = np.diff(mat.level_off.numpy())
         assert (widths[-120:] == 1).all()
@@ -525,7 +537,7 @@ def test_chain_lengths_around_the_stretch_size(orc):
         for normalized, d in ((False, 96), (True, 41)):
             e2 = graphs.add_self_loops(ei, n) if normalized else ei
             mat = cbm_matrix(torch.from_numpy(e2), None, alpha=0, normalized=normalized)
-            mat.subtree_walk = "off"                       # the level plan's chain kernel
+            mat.subtree_walk = mat.stream_multiply = "off" # the level plan's chain kernel
             widths = np.diff(mat.level_off.numpy())
             run = int(np.argmax(widths[::-1] != 1)) if (widths != 1).any() else len(widths)
             runs.add(run)
@@ -547,6 +559,10 @@ def _walk_graph(kind):
     if kind == "staircases":
         ei = graphs.staircases(30, 70, 6, 2.0, seed=1)
         return ei, int(ei.max()) + 1
+    if kind == "bipartite":                                # identical rows on either side: empty delta rows
+        u, v = np.meshgrid(np.arange(40), 40 + np.arange(500), indexing="ij")
+        e = np.stack([u.ravel(), v.ravel()])
+        return np.concatenate([e, e[::-1]], 1).astype(np.int32), 540
     n = 1200
     return graphs.duplication(n, 0.7, 3, 8, seed=2), n
 
@@ -566,6 +582,7 @@ def test_subtree_walk_equals_the_level_walk_and_the_oracle(orc, kind, normalized
     mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
     mat.single_launch_max_bytes = 0
     mat.path_walk_max_bytes = 0
+    mat.stream_multiply = "off"                            # the SpMM and the walk apart
     assert mat.n_levels >= 3
     slots = mat._host_walk_plan(0, 64)["n_slots"]
     assert (slots >= 2) if kind in ("bushy", "duplication") else True
@@ -684,6 +701,84 @@ def test_subtree_walk_status_codes():
     bad = _lib.CbmWalkDev(0, good.n_entries, good.n_bins, 40, good.entries, good.bin_off)
     assert call(bad) == _lib.CBM_ERR_SHAPE                               # more slots than a wavefront has
     bad = _lib.CbmWalkDev(0, good.n_entries, good.n_bins, good.n_slots, None, good.bin_off)
+    assert call(bad) == _lib.CBM_ERR_NULL
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+@pytest.mark.parametrize("kind", ["staircases", "bushy", "chain", "duplication", "bipartite"])
+def test_stream_multiply_against_oracle(orc, kind, normalized):
+    """cbm_spmm_update_subtrees_f32: the whole multiply in one launch, every subtree walked depth-first and every
+    row's delta entries summed on the way, strictly in entry order with fma(+-1 or +-m[col], x, acc) -- the
+    reference's per-entry arithmetic -- then the walk step of the level-by-level walk.  Bit for bit the oracle's
+    in-order product on the same tree, for widths of one to eighteen 64-column slices (ragged last slice,
+    d % 8 != 0 for the division tail), trees that are deep and wide, bushy (slots in use), one long chain (a bin
+    of many stretches, rows of hundreds of entries that span stretches) and rows with no delta entry at all;
+    with the ReLU in the store; on matrices whose rows are further apart than d."""
+    ei, n = _walk_graph(kind)
+    if normalized:
+        ei = graphs.add_self_loops(ei, n)
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=normalized)
+    mat.single_launch_max_bytes = 0
+    mat.stream_multiply = "on"
+    assert mat.n_levels >= 2
+    plan = mat.stream_plan(64)
+    lens = np.diff(mat.rowptr.numpy())
+    if kind == "bipartite" and not normalized:
+        assert int((lens == 0).sum()) >= 400
+    if kind == "chain":
+        assert plan["longest_bin"] > 2000 and int(lens.max()) > 64      # many stretches; rows that span stretches
+    if kind in ("bushy", "duplication"):
+        assert plan["n_slots"] >= 2
+    for d in (1, 19, 41, 64, 100, 128, 258, 1100):
+        say("stream multiply", kind, normalized, "d", d, "levels", mat.n_levels, "bins", plan["n_bins"], "slots", plan["n_slots"],
+            "longest bin", plan["longest_bin"])
+        assert takes_stream(mat, d)
+        x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+        got = gpu_product(mat, x, normalized)
+        want = oracle_product(orc, mat, ei, n, x, normalized)
+        assert np.array_equal(got, want)
+        assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= TOL_CBM
+        if d in (41, 128):
+            xd = torch.from_numpy(x).cuda()
+            relu = torch.full_like(xd, float("nan"))
+            mat._run_spmm_update(xd, relu, use_m=normalized, relu=True)
+            assert float(got.min()) < 0 and np.array_equal(relu.cpu().numpy(), np.maximum(got, 0.0))
+            # rows of X and Y further apart than d: the columns beyond stay as they were
+            wide_x = torch.full((n, d + 3), float("nan"), device="cuda"); wide_x[:, :d] = xd
+            wide_y = torch.full((n, d + 7), 3.0, device="cuda")
+            mat._run_spmm_update(wide_x[:, :d], wide_y[:, :d], use_m=normalized)
+            assert np.array_equal(wide_y[:, :d].cpu().numpy(), got) and bool((wide_y[:, d:] == 3.0).all())
+    # integer features: every summation order is exact, so the SpMM + walk path returns the same bits
+    xi = np.random.default_rng(1).integers(-4, 5, size=(n, 72)).astype(np.float32)
+    if not normalized:
+        got = gpu_product(mat, xi, False)
+        mat.stream_multiply = "off"
+        assert np.array_equal(gpu_product(mat, xi, False), got)
+
+
+def test_stream_multiply_status_codes():
+    lib = _lib.hip_lib()
+    ei = graphs.add_self_loops(graphs.staircases(8, 20, 6, 2.0, seed=4))
+    mat = cbm_matrix(torch.from_numpy(ei), None, alpha=0, normalized=True)
+    mat.stream_multiply = "on"
+    n, d = mat.num_rows, 64
+    x = torch.randn((n, d), device="cuda")
+    y = torch.zeros((n, d), device="cuda")
+    st = mat._device_arrays(y.device)
+    good = mat._stream_struct(st, mat.stream_plan(d))
+    p = lambda t: C.c_void_p(t.data_ptr())
+    call = lambda w, xx=x, flags=0, rows=n: lib.cbm_spmm_update_subtrees_f32(
+        C.byref(w) if w is not None else None, p(st["m"]), p(xx), p(y), rows, d, d, d, flags, None)
+    say("stream multiply status codes")
+    assert call(good) == 0
+    assert call(None) == _lib.CBM_ERR_NULL
+    assert call(good, xx=y) == _lib.CBM_ERR_SHAPE                        # X must not be Y
+    assert call(good, flags=_lib.CBM_PROP_SCALE_ROOTS) == 6              # only the ReLU flag
+    assert call(good, rows=n - 1) == _lib.CBM_ERR_SHAPE                  # a plan of another matrix
+    bad = _lib.CbmWalkStreamDev(n, good.n_bins, 40, good.n_elems, good.gidx, good.ginfo, good.bin_goff)
+    assert call(bad) == _lib.CBM_ERR_SHAPE                               # more slots than a wavefront has
+    bad = _lib.CbmWalkStreamDev(n, good.n_bins, good.n_slots, good.n_elems, None, good.ginfo, good.bin_goff)
     assert call(bad) == _lib.CBM_ERR_NULL
     torch.cuda.synchronize()
 

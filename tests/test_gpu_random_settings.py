@@ -16,8 +16,8 @@ def test_random_settings_against_oracle(orc, seed, monkeypatch):
     """40 cases per seed: SBM / Erdos-Renyi / hub-row graphs of 7 .. 3,000 nodes, plain and normalised,
     alpha 0 .. huge, widths 1 .. 258, with and without the LDS tiling, the depth limit, rows cut by
     length and at column-block boundaries, the one-launch path walk and the one-launch product on and off, the
-    walk by subtrees off / by estimate / forced (with a forced cut), short rows in batches of every limit; also
-    staircase graphs (deep and wide trees)."""
+    walk by subtrees off / by estimate / forced (with a forced cut), the one-launch multiply by subtrees off / by
+    estimate / forced, short rows in batches of every limit; also staircase graphs (deep and wide trees)."""
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     rng = np.random.default_rng(seed)
@@ -51,10 +51,11 @@ def test_random_settings_against_oracle(orc, seed, monkeypatch):
         mat.batch_rows = int(rng.choice([0, 8, 32, 64]))
         walk = ["off", "auto", "on", 0, 2][int(rng.integers(5))]
         mat.subtree_walk = walk
+        mat.stream_multiply = ["off", "auto", "on"][int(rng.integers(3))]
         x = rng.standard_normal((n, d)).astype(np.float32)
         parity.say("random settings", seed, case, kind, n, mat.nnz, mat.n_levels, normalized, alpha, d, tiling, mat.is_tiled(),
                    mat.has_cut_rows(), mat.split_chunk, mat.column_blocks, max_levels, mat.path_walk_max_bytes,
-                   mat.single_launch_max_bytes, "batch", mat.batch_rows, "walk", walk)
+                   mat.single_launch_max_bytes, "batch", mat.batch_rows, "walk", walk, "stream", mat.stream_multiply)
         got = parity.gpu_product(mat, x, normalized)
         assert np.array_equal(got, parity.oracle_product(orc, mat, ei, n, x, normalized)), (seed, case)
         assert orc.max_rel_err(got, orc.dense_product(ei, n, x, normalized)) <= parity.TOL_CBM, (seed, case)
