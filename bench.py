@@ -369,6 +369,10 @@ def measure_multiply(w, alpha, d, args, torch, vendor=False, sample_rows=512, cp
     if not mat.is_tiled() and not mat.has_cut_rows() and mat._single_launch(n, d):
         relayout_ms, spmm_ms, prop_ms, prop_how, kernel, slab = 0.0, span_ms, 0.0, None, "spmm_update_paths_wave_per_row", False
         roof = roofline_of(w.name, alpha, d, kernel, spmm_ms, b_spmm + b_prop, b_min, args.scale)
+    elif streams_in_multiply(mat, n, d):
+        # a deep tree with short delta rows: ONE launch sums the rows and walks the subtrees
+        relayout_ms, spmm_ms, prop_ms, prop_how, kernel, slab = 0.0, span_ms, 0.0, None, "spmm_update_subtrees", False
+        roof = roofline_of(w.name, alpha, d, kernel, spmm_ms, b_spmm + b_prop, b_min, args.scale)
     else:
         relayout_ms, spmm_ms, zd, kernel = spmm_alone(mat, xd, w.normalized, args.steps, args.warmup, torch)
         prop_ms, prop_how = 0.0, None
@@ -438,6 +442,13 @@ def level_launches(lo, first_level, last_level):
     return launches
 
 
+def streams_in_multiply(mat, n, d):
+    """Whether a multiply of ``mat`` with an [n, d] matrix is the one-launch multiply by subtrees (the Python
+    layer's rule: after the single launch of small products, for matrices neither tiled nor with cut rows)."""
+    return (mat.n_levels > 1 and not (mat.is_tiled() or mat.has_cut_rows()) and not mat._single_launch(n, d)
+            and mat.stream_plan(d) is not None)
+
+
 def walks_paths_in_multiply(mat, n, d):
     """Whether a multiply of ``mat`` with an [n, d] matrix ends in the one-launch path walk (the Python
     layer's rule: untiled, no cut rows, a shallow tree, a product within the path walk's size limit)."""
@@ -446,12 +457,15 @@ def walks_paths_in_multiply(mat, n, d):
 
 def launches_per_multiply(mat, n, d, copies_x=True):
     """Kernel launches one multiply of ``mat`` with an [n, d] matrix issues, by the rules the Python layer
-    applies: one for a small product on a shallow tree; else the copy of X (``copies_x``: short rows and
+    applies: one for a small product on a shallow tree, one for the multiply by subtrees of a deep tree with
+    short delta rows; else the copy of X (``copies_x``: short rows and
     small X are gathered in place) + the SpMM (+ adding the pieces of cut rows), then the walk -- one launch
     for the path walk of a shallow tree, the levels above the cut + one for the walk by subtrees, or the
     level-by-level plan."""
     tiled_or_cut = mat.is_tiled() or mat.has_cut_rows()
     if not tiled_or_cut and mat._single_launch(n, d):
+        return 1
+    if streams_in_multiply(mat, n, d):
         return 1
     launches = (2 if copies_x or tiled_or_cut else 1) + (1 if mat.has_cut_rows() else 0)
     if mat.n_levels <= 1:

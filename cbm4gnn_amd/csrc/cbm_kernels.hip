@@ -22,6 +22,8 @@
 //                             levels, one register-carried launch per chain of single-row levels;
 //        propagate_subtrees   every subtree below a level in ONE launch: a wave walks a host-made
 //                             depth-first sequence, parent values in a register and LDS slots;
+//        spmm_update_subtrees the same walk with every row's delta entries summed on the way (deep trees,
+//                             short delta rows): SpMM and walk in one launch, no SpMM result in memory;
 //        propagate_paths / spmm_update_paths_wave_per_row
 //                             shallow trees: every row sums down its own ancestor path (one launch).
 // The SpMM instantiations with PACKED = false are the plain CSR baseline.

@@ -51,11 +51,12 @@ def test_launch_count_follows_the_walk_plan():
     import types
     import torch
 
-    def fake(widths, tiled=False, cut=False, single=False, paths=False, subtrees=None):
+    def fake(widths, tiled=False, cut=False, single=False, paths=False, subtrees=None, stream=False):
         lo = torch.tensor([0] + list(__import__("itertools").accumulate(widths)), dtype=torch.int32)
         return types.SimpleNamespace(level_off=lo, n_levels=len(widths), is_tiled=lambda: tiled, has_cut_rows=lambda: cut,
                                      _single_launch=lambda n, d: single, _walks_paths=lambda n, d: paths,
-                                     walk_plan=lambda d: ({"cut": subtrees} if subtrees is not None else None))
+                                     walk_plan=lambda d: ({"cut": subtrees} if subtrees is not None else None),
+                                     stream_plan=lambda d: ({"n_bins": 1} if stream else None))
 
     assert bench.launches_per_multiply(fake([500]), 500, 64) == 2                         # flat tree
     assert bench.launches_per_multiply(fake([500], cut=True), 500, 64) == 3               # + adding the pieces
@@ -70,6 +71,10 @@ def test_launch_count_follows_the_walk_plan():
     assert bench.launches_per_multiply(fake(deep, subtrees=0), 2000, 64) == 2 + 1
     assert bench.launches_per_multiply(fake(deep, subtrees=2), 2000, 64) == 2 + 2 + 1
     assert bench.launches_per_multiply(fake(deep, subtrees=0, paths=True), 2000, 64) == 2 + 1      # the path walk asks first
+    # the multiply by subtrees is one launch; small products and plan-based multiplies never ask for it
+    assert bench.launches_per_multiply(fake(deep, subtrees=0, stream=True), 2000, 64) == 1
+    assert bench.launches_per_multiply(fake(deep, subtrees=0, stream=True, tiled=True), 2000, 64) == 2 + 1
+    assert bench.launches_per_multiply(fake([500], stream=True), 500, 64) == 2
     # short rows / a small X are gathered in place: no copy launch
     assert bench.launches_per_multiply(fake([500]), 500, 64, copies_x=False) == 1
     assert bench.launches_per_multiply(fake([500, 300, 200], paths=True), 1000, 64, copies_x=False) == 2
