@@ -86,7 +86,7 @@ class CbmWalkDev(C.Structure):
 class CbmWalkStream(C.Structure):
     """Mirror of ``struct cbm_walk_stream`` (host arrays made by ``cbm_walk_stream_build``)."""
     _fields_ = [
-        ("n", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32), ("n_elems", C.c_int32), ("longest_bin", C.c_int64),
+        ("n", C.c_int32), ("n_bins", C.c_int32), ("n_slots", C.c_int32), ("n_elems", C.c_int32), ("heaviest_bin", C.c_int64),
         ("gidx", C.POINTER(C.c_uint32)), ("ginfo", C.POINTER(C.c_int32)), ("bin_goff", C.POINTER(C.c_int32)),
     ]
 
@@ -101,6 +101,7 @@ class CbmWalkStreamDev(C.Structure):
 
 CBM_WALK_LOAD_ONLY = 63
 CBM_STREAM_LAST, CBM_STREAM_DUMMY, CBM_STREAM_COL_MASK = 0x40000000, 0x20000000, 0x1FFFFFFF
+CBM_STREAM_ROW_COST = 5
 CBM_WALK_MAX_SLOTS = 31
 
 _P = C.c_void_p

@@ -808,16 +808,25 @@ class cbm_matrix:
             self._walk_plans[key] = best or None
         return self._walk_plans[key]
 
-    # One wavefront alone on its bin streams an entry (one gathered row of X) in about this long; the launch as
-    # a whole moves about this many bytes per microsecond.  Measured on staircase graphs of 11,400 .. 280,000
-    # rows, d = 64 .. 512: the launch takes max(longest bin x the first, bytes / the second) within 10 %.
-    _STREAM_US_PER_ENTRY = 0.105
-    _STREAM_BYTES_PER_US = 6.5e6
+    # The launch of the multiply by subtrees takes the longer of: the wavefront with the heaviest bin alone (this
+    # long per stream entry, a row weighing CBM_STREAM_ROW_COST entries more for its walk step and store), and
+    # the bytes of the launch (every stream entry's row of X, every row of Y once) at the second rate.  The SpMM
+    # of short rows moves its bytes at the third.  Measured on staircase graphs of 11,400 .. 280,000 rows, 3 ..
+    # 16 entries per delta row, d = 64 .. 512 (within 10 %).
+    _STREAM_US_PER_WEIGHT = 0.041
+    _STREAM_BYTES_PER_US = 7.5e6
+    _SHORT_ROW_SPMM_BYTES_PER_US = 6.5e6
+    _STREAM_MAX_ENTRIES_PER_ROW = 24          # "auto" asks only where the slab-major copy of X would not pay either
+
+    @staticmethod
+    def _stream_bin_target(d):
+        """Bins a multiply stream aims for: (bins x 64-column slices) wavefronts fill the GPU several times over."""
+        return max(64, 16384 // ((d + 63) // 64))
 
     def _host_stream(self, d):
         """``cbm_walk_stream_build`` for this matrix (CPU tensors + stats), cached per bin target; False when the
         tree needs more kept values than the kernel has slots (or more than 2^29 rows)."""
-        target_bins = self._walk_bin_target(d)
+        target_bins = self._stream_bin_target(d)
         key = ("stream", target_bins)
         plan = self._walk_plans.get(key)
         if plan is None:
@@ -834,7 +843,7 @@ class cbm_matrix:
                     take = lambda ptr, count: torch.from_numpy(
                         np.ctypeslib.as_array(ptr, shape=(max(count, 1),))[:count].astype(np.int32, copy=True))
                     plan = {"n_bins": int(p.n_bins), "n_slots": int(p.n_slots), "n_elems": int(p.n_elems),
-                            "longest_bin": int(p.longest_bin), "gidx": take(p.gidx, p.n_elems),
+                            "heaviest_bin": int(p.heaviest_bin), "gidx": take(p.gidx, p.n_elems),
                             "ginfo": take(p.ginfo, 2 * p.n_elems).view(-1, 2), "bin_goff": take(p.bin_goff, p.n_bins + 1)}
             finally:
                 _lib.host_lib().cbm_walk_stream_free(C.byref(p))
@@ -842,10 +851,11 @@ class cbm_matrix:
         return plan
 
     def _stream_weights(self):
-        """Stream entries in the subtree of every row (an empty row counts one), int64 NumPy; computed once."""
+        """Weight of the subtree of every row in the multiply stream (a row: its delta entries, an empty row one,
+        + CBM_STREAM_ROW_COST), int64 NumPy; computed once."""
         weights = self._walk_plans.get("weights")
         if weights is None:
-            weights = np.maximum(np.diff(self.rowptr.numpy().astype(np.int64)), 1)
+            weights = np.maximum(np.diff(self.rowptr.numpy().astype(np.int64)), 1) + _lib.CBM_STREAM_ROW_COST
             lo, order, parent = self.level_off.tolist(), self.order.numpy(), self.parent.numpy()
             for l in range(self.n_levels - 1, 0, -1):                       # leaves first
                 rows = order[lo[l]:lo[l + 1]]
@@ -853,13 +863,30 @@ class cbm_matrix:
             self._walk_plans["weights"] = weights
         return weights
 
+    def _stream_cost_us(self, heaviest_bin, d):
+        """Estimate for the one-launch multiply by subtrees (see the constants above)."""
+        n = self.num_rows
+        entries = max(self.nnz, n)                                          # about: empty rows count one
+        return self._WALK_US_PER_LAUNCH + max(heaviest_bin * self._STREAM_US_PER_WEIGHT,
+                                              (entries + n) * d * 4 / self._STREAM_BYTES_PER_US)
+
+    def _two_launch_cost_us(self, d):
+        """Estimate for the same product as SpMM (short rows, gathered in place) + walk."""
+        n = self.num_rows
+        spmm = self._WALK_US_PER_LAUNCH + (self.nnz + n) * d * 4 / self._SHORT_ROW_SPMM_BYTES_PER_US
+        if self._walks_paths(n, d):
+            return spmm + 2 * self._WALK_US_PER_LAUNCH                      # the one-launch path walk of a shallow tree
+        plan = self.walk_plan(d)
+        return spmm + (self._subtree_plan_cost_us(plan, d) if plan is not None else self._level_plan_cost_us(d))
+
     def stream_plan(self, d):
         """The plan of the one-launch multiply by subtrees for width ``d``, or None when the multiply runs as
         SpMM + walk: by ``stream_multiply`` -- "off": None; "on": the plan whenever the tree has two levels or
-        more and the matrix is neither tiled nor has cut rows; "auto": the plan when, by the shape of the tree
-        and the lengths of the delta rows, the launch is bound by the bytes it moves (every delta entry's row
-        of X once, every row of Y once) rather than by the wavefront with the longest bin -- then it moves
-        fewer bytes than the SpMM and the walk apart, which write and re-read the SpMM result."""
+        more and the matrix is neither tiled nor has cut rows; "auto": the plan when delta rows average at most
+        24 entries (the rows the SpMM gathers in place) and an estimate from the shape of the tree and the
+        lengths of the rows puts the launch at 0.85 of the SpMM + walk or below -- it moves fewer bytes (no SpMM
+        result written and read back) but runs one wavefront per bin of whole subtrees, so few large subtrees
+        or narrow matrices keep the two launches."""
         policy = self.stream_multiply
         if policy == "off" or self.n_levels < 2 or self.num_rows == 0 or d <= 0:
             return None
@@ -867,15 +894,16 @@ class cbm_matrix:
             raise ValueError('stream_multiply must be "auto", "on" or "off"')
         if self._host_tiling():
             return None
-        key = ("stream-choice", policy, (d + 63) // 64, d if policy == "auto" else 0)
+        key = ("stream-choice", policy, d if policy == "auto" else (d + 63) // 64, self.subtree_walk if policy == "auto" else None)
         if key not in self._walk_plans:
             take = True
             if policy == "auto":
-                weights, target = self._stream_weights(), self._walk_bin_target(d)
-                heads = weights[self.order.numpy()[:int(self.level_off[1])]]
-                total = int(heads.sum())
-                longest = max(int(heads.max()), -(-total // target), 64)      # small subtrees are packed into bins
-                take = longest * self._STREAM_US_PER_ENTRY <= (total + self.num_rows) * d * 4 / self._STREAM_BYTES_PER_US
+                take = self.nnz <= self._STREAM_MAX_ENTRIES_PER_ROW * self.num_rows
+                if take:
+                    weights, target = self._stream_weights(), self._stream_bin_target(d)
+                    heads = weights[self.order.numpy()[:int(self.level_off[1])]]
+                    heaviest = max(int(heads.max()), -(-int(heads.sum()) // target), 64)    # small subtrees are packed into bins
+                    take = self._stream_cost_us(heaviest, d) <= 0.85 * self._two_launch_cost_us(d)
             self._walk_plans[key] = (self._host_stream(d) or None) if take else None
         return self._walk_plans[key]
 

@@ -960,10 +960,11 @@ int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int3
     try {
         WalkTree tree;
         if (int rc = tree.build(parent, order, level_off, n, n_levels)) return rc;
-        // a row costs its delta entries (an empty row one stand-in entry); a subtree the sum over its rows
+        // a row costs its delta entries (an empty row one stand-in entry) + CBM_STREAM_ROW_COST for its walk
+        // step and store; a subtree the sum over its rows
         std::vector<int64_t> weight(n);
         int64_t total = 0;
-        for (int32_t v = 0; v < n; v++) total += weight[v] = std::max(rowptr[v + 1] - rowptr[v], 1);
+        for (int32_t v = 0; v < n; v++) total += weight[v] = std::max(rowptr[v + 1] - rowptr[v], 1) + CBM_STREAM_ROW_COST;
         if (total > INT32_MAX) return CBM_ERR_SHAPE;
         for (int32_t i = n - 1; i >= 0; i--) {
             const int32_t v = order[i];
@@ -973,30 +974,44 @@ int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int3
         std::vector<int32_t> roots(order, order + level_off[1]);
         std::sort(roots.begin(), roots.end(),
                   [&](int32_t a, int32_t b) { return weight[a] != weight[b] ? weight[a] > weight[b] : a < b; });
-        // bins: consecutive tasks of the sorted list until a bin holds `target` stream entries
+        // bins: consecutive tasks of the sorted list until a bin weighs `target`
         const int64_t target = std::max<int64_t>((total + target_bins - 1) / target_bins, CBM_STREAM_MIN_BIN);
         std::vector<int32_t> entries;                      // { row, ctl } in walk order
         entries.reserve(2 * (size_t)n);
         std::vector<int32_t> bin_first(1, 0);              // first row (position in entries) of every bin
-        int64_t in_bin = 0;
+        int64_t in_bin = 0, heaviest = 0;
         int32_t max_slots = 0;
         for (int32_t r : roots) {
             if (in_bin >= target) { bin_first.push_back((int32_t)(entries.size() / 2)); in_bin = 0; }
             in_bin += weight[r];
+            heaviest = std::max(heaviest, in_bin);
             if (!tree.emit(r, max_slots, [&](int32_t row, int32_t ctl) { entries.push_back(row); entries.push_back(ctl); }))
                 return CBM_ERR_UNSUPPORTED;
         }
         if (entries.size() != 2 * (size_t)n) return CBM_ERR_INTERNAL;
         bin_first.push_back(n);
         const int32_t n_bins = (int32_t)bin_first.size() - 1;
-        out->n = n; out->n_bins = n_bins; out->n_slots = max_slots; out->n_elems = (int32_t)total;
-        out->gidx = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)total);
-        out->ginfo = (int32_t*)calloc(2 * (size_t)total, sizeof(int32_t));   // zeroed: "no row landed here"
+        // every bin is padded to whole stretches of 64 entries (the kernel never tests for the end of a bin
+        // inside a stretch): copies of its last entry without marks, whose sum goes nowhere
+        std::vector<int64_t> goff(n_bins + 1, 0);
+        for (int32_t b = 0; b < n_bins; b++) {
+            int64_t elems = 0;
+            for (int32_t k = bin_first[b]; k < bin_first[b + 1]; k++) {
+                const int32_t row = entries[2 * (size_t)k];
+                elems += std::max(rowptr[row + 1] - rowptr[row], 1);
+            }
+            goff[b + 1] = goff[b] + (elems + 63) / 64 * 64;
+        }
+        const int64_t padded = goff[n_bins];
+        if (padded > INT32_MAX) return CBM_ERR_SHAPE;
+        out->n = n; out->n_bins = n_bins; out->n_slots = max_slots; out->n_elems = (int32_t)padded;
+        out->gidx = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)padded);
+        out->ginfo = (int32_t*)calloc(2 * (size_t)padded, sizeof(int32_t));   // zeroed: "no row landed here"
         out->bin_goff = (int32_t*)malloc(sizeof(int32_t) * ((size_t)n_bins + 1));
         if (!out->gidx || !out->ginfo || !out->bin_goff) throw std::bad_alloc();
-        int64_t g = 0, longest = 0;
         for (int32_t b = 0; b < n_bins; b++) {
-            const int64_t g0 = g;
+            const int64_t g0 = goff[b];
+            int64_t g = g0;
             out->bin_goff[b] = (int32_t)g0;
             int64_t stretch = -1;
             int32_t in_stretch = 0;
@@ -1015,7 +1030,8 @@ int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int3
                 int32_t* info = out->ginfo + 2 * (g0 + s * 64 + in_stretch++);
                 info[0] = row; info[1] = ctl | INT32_MIN;  // marked: a slot that is in use
             }
-            longest = std::max(longest, g - g0);
+            const uint32_t pad = out->gidx[g - 1] & CBM_STREAM_COL_MASK;
+            while (g < goff[b + 1]) out->gidx[g++] = pad;
             // slots no row landed in: a valid row (the kernel loads them, and m of their row, without using them)
             const int32_t filler = entries[2 * (size_t)bin_first[b]];
             for (int64_t q = g0; q < g; q++) {
@@ -1024,9 +1040,8 @@ int cbm_walk_stream_build(const int32_t* rowptr, const uint32_t* idx, const int3
                 else { info[0] = filler; info[1] = 0; }
             }
         }
-        if (g != total) return (cbm_walk_stream_free(out), CBM_ERR_INTERNAL);
-        out->bin_goff[n_bins] = (int32_t)total;
-        out->longest_bin = longest;
+        out->bin_goff[n_bins] = (int32_t)padded;
+        out->heaviest_bin = heaviest;
         return CBM_OK;
     } catch (const std::bad_alloc&) {
         cbm_walk_stream_free(out);

@@ -1082,14 +1082,15 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy, int n_slots) {
     extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
     const int lane = threadIdx.x & (kWave - 1);
-    const int w = blockIdx.x * kSubWaves + (threadIdx.x >> 6);
-    const int bin = w / slices;
+    const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
+    const int bin = w / slices;                                                                // known to be
     if (bin >= n_bins) return;
     const int j = (w % slices) * kWave + lane;                    // feature column of this thread
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d load column 0 and store nothing
     float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
-    const int first = bin_off[bin], count = bin_off[bin + 1] - first;
+    const int first = __builtin_amdgcn_readfirstlane(bin_off[bin]);
+    const int count = __builtin_amdgcn_readfirstlane(bin_off[bin + 1]) - first;
     const int2 e0 = entries[first];
     auto ids = [&](int base) -> int2 {                            // entry base + lane; past the end: the first one
         const int2 e = entries[first + min(base + lane, count - 1)];
@@ -1166,15 +1167,18 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
 
 // The whole multiply of a DEEP tree with SHORT delta rows in one launch: the walk of propagate_subtrees with
 // the SpMM result of a row summed on the spot instead of read back.  The host lays the delta entries of a
-// bin's rows end to end in the order the walk visits them (gidx: col | sign << 31, kStreamLast on a row's
-// last entry, kStreamDummy on the one stand-in entry of an empty row); a wavefront streams that list 64 entries
-// at a time, lane l decoding entry l (its coefficient +-1 or +-m[col], the byte offset of row col of X), and
-// gathers its 64 feature columns of every entry's row half a stretch ahead of their use, unconditionally.  The
-// sum of a row runs strictly in entry order (fma(coef, x, acc) from zero: the order of spmm_wave_per_row);
-// when its last entry is in, the row takes its walk step exactly as in propagate_subtrees (the head of a
-// subtree is a child of the root: its sum times m) and is stored once -- through the ReLU if asked, the raw
-// value staying in the register / LDS slot its children read.  ginfo holds, per stretch of 64 entries, the
-// {row, ctl} of the rows that end inside it, in order.  Z never exists in memory.
+// bin's rows end to end in the order the walk visits them (gidx: col | sign << 31, CBM_STREAM_LAST on a row's
+// last entry, CBM_STREAM_DUMMY on the one stand-in entry of an empty row) and pads the bin to whole stretches
+// of 64 entries; a wavefront streams that list a stretch at a time, lane l decoding entry l (its coefficient
+// +-1 or +-m[col], the address of row col of X), and gathers its 64 feature columns of every entry's row a
+// whole stretch ahead of their use: entry k's register is re-used for entry k of the next stretch as soon as
+// it has been added, so 64 gathers are in flight all the time and no load is conditional.  The sum of a row
+// runs strictly in entry order (fma(coef, x, acc) from zero: the order of spmm_wave_per_row); when its last
+// entry is in, the row takes its walk step exactly as in propagate_subtrees (the head of a subtree is a child
+// of the root: its sum times m) and is stored once -- through the ReLU if asked, the raw value staying in the
+// register / LDS slot its children read.  ginfo holds, per stretch, the {row, ctl} of the rows that end inside
+// it, in order.  Everything that steers control flow is wave-uniform (scalar branches, the common case falls
+// through).  Z never exists in memory.
 constexpr uint32_t kStreamLast = CBM_STREAM_LAST, kStreamDummy = CBM_STREAM_DUMMY, kStreamCol = CBM_STREAM_COL_MASK;
 
 template <bool NORM>
@@ -1184,82 +1188,44 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
     int64_t ldy, int n_slots, int relu) {
     extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
     const int lane = threadIdx.x & (kWave - 1);
-    const int w = blockIdx.x * kSubWaves + (threadIdx.x >> 6);
-    const int bin = w / slices;
+    const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
+    const int bin = w / slices;                                                                // known to be
     if (bin >= n_bins) return;
     const int j = (w % slices) * kWave + lane;                    // feature column of this thread
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d gather column 0 and store nothing
     float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
-    const int first = bin_goff[bin], count = bin_goff[bin + 1] - first;
-    auto at = [&](int base) -> int { return first + min(base + lane, count - 1); };   // past the end: the last entry
-    auto bcast64 = [&](int64_t off_ids, int k) -> int64_t {
-        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)off_ids, k);
-        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)((uint64_t)off_ids >> 32), k);
-        return (int64_t)(((uint64_t)hi << 32) | lo);
-    };
+    const int first = __builtin_amdgcn_readfirstlane(bin_goff[bin]);
+    const int count = __builtin_amdgcn_readfirstlane(bin_goff[bin + 1]) - first;       // a multiple of 64
+    auto at = [&](int base) -> int { return first + min(base, count - kWave) + lane; };   // past the end: the last stretch
     const uint32_t jj4 = (uint32_t)jj * 4u;
-    auto x_off = [&](uint32_t p) -> int64_t { return (int64_t)(p & kStreamCol) * ldx * 4; };
+    // what lane l keeps for entry l of a stretch: the address of its row of X (wave-uniform once broadcast:
+    // the gather then is one load with a scalar base and the lane's column offset)
+    auto x_row = [&](uint32_t p) -> uint64_t {
+        return (uint64_t)reinterpret_cast<uintptr_t>(X) + (uint64_t)(p & kStreamCol) * (uint64_t)ldx * 4u;
+    };
     auto coef = [&](uint32_t p) -> float {
         uint32_t mag = 0x3f800000u;
         if constexpr (NORM) mag = __float_as_uint(m[p & kStreamCol]);
         return __uint_as_float(mag ^ (p & 0x80000000u));
     };
-    auto request = [&](float (&z)[kChainHalf], int64_t xo_ids, int half) {
-#pragma unroll
-        for (int u = 0; u < kChainHalf; u++)
-            z[u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(X) + bcast64(xo_ids, half * kChainHalf + u) + jj4);
+    auto gather = [&](uint64_t xr_ids, int k) -> float {
+        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)xr_ids, k);
+        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)(xr_ids >> 32), k);
+        typedef const __attribute__((address_space(1))) char* global_bytes;      // device memory, not a flat address
+        typedef const __attribute__((address_space(1))) float* global_float;
+        const global_bytes row = (global_bytes)(uintptr_t)(((uint64_t)hi << 32) | lo);
+        return *(global_float)(row + jj4);
     };
     float acc = 0.0f, run = 0.0f, mu = 1.0f;
-    int rs = 0;                                                   // rows finished in the current stretch (wave-uniform)
-    auto consume = [&](const float (&z)[kChainHalf], uint32_t p_ids, float f_ids, int2 i_ids, float mr_ids, int base, int half) {
-#pragma unroll
-        for (int u = 0; u < kChainHalf; u++) {
-            const int k = half * kChainHalf + u;
-            if (base + k < count) {
-                const uint32_t p = (uint32_t)bcast_i((int)p_ids, k);          // wave-uniform: the branches are scalar
-                if (!(p & kStreamDummy)) acc = fmaf(bcast_f(f_ids, k), z[u], acc);
-                if (p & kStreamLast) {
-                    const int ctl = bcast_i(i_ids.y, rs);
-                    const int src = ctl & 63, dst = (ctl >> 8) & 63;
-                    const float mv = NORM ? bcast_f(mr_ids, rs) : 1.0f;
-                    if (src == CBM_WALK_LOAD_ONLY) {                          // a child of the root
-                        run = NORM ? acc * mv : acc;
-                    } else {
-                        float a = run, ma = mu;
-                        if (src) {
-                            a = st[(src - 1) * 2 * kWave];
-                            if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
-                        }
-                        if constexpr (NORM) {
-                            const float inv_mu = 1.0f / ma;
-                            run = (jj < dv) ? fmaf(a, inv_mu, acc) * mv : (acc + a / ma) * mv;
-                        } else {
-                            run = acc + a;
-                        }
-                    }
-                    if (live) {
-                        float* yr = reinterpret_cast<float*>(reinterpret_cast<char*>(Y) + (int64_t)bcast_i(i_ids.x, rs) * ldy * 4 + jj4);
-                        *yr = (relu && run < 0.0f) ? 0.0f : run;              // keeps NaN, as torch.relu does
-                    }
-                    mu = mv;
-                    if (dst) {
-                        st[(dst - 1) * 2 * kWave] = run;
-                        if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
-                    }
-                    acc = 0.0f;
-                    rs++;
-                }
-            }
-        }
-    };
     uint32_t p_cur = gidx[at(0)], p_nxt = gidx[at(kWave)];
     int2 i_cur = ginfo[at(0)], i_nxt = ginfo[at(kWave)];
     float f_cur = coef(p_cur), mr_cur = 1.0f;
     if constexpr (NORM) mr_cur = m[i_cur.x];
-    int64_t xo_cur = x_off(p_cur), xo_nxt = x_off(p_nxt);
-    float za[kChainHalf], zb[kChainHalf];
-    request(za, xo_cur, 0);
+    uint64_t xr_cur = x_row(p_cur), xr_nxt = x_row(p_nxt);
+    float z[kWave];
+#pragma unroll
+    for (int k = 0; k < kWave; k++) z[k] = gather(xr_cur, k);
     for (int base = 0; base < count; base += kWave) {
         // requested first, needed last: the entries and rows of the stretch after the next, and what depends on
         // the next stretch's (their entries came in an iteration ago)
@@ -1268,15 +1234,50 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
         const float f_nxt = coef(p_nxt);
         float mr_nxt = 1.0f;
         if constexpr (NORM) mr_nxt = m[i_nxt.x];
-        request(zb, xo_cur, 1);
-        rs = 0;
-        consume(za, p_cur, f_cur, i_cur, mr_cur, base, 0);
-        request(za, xo_nxt, 0);
-        consume(zb, p_cur, f_cur, i_cur, mr_cur, base, 1);
+        int rs = 0;                                               // rows finished in this stretch (wave-uniform)
+#pragma unroll
+        for (int k = 0; k < kWave; k++) {
+            // entries past the bin's last row (its padding) are added like any other: their sum is never stored
+            acc = fmaf(bcast_f(f_cur, k), z[k], acc);
+            z[k] = gather(xr_nxt, k);                                         // past the end: the last stretch again
+            const uint32_t p = (uint32_t)bcast_i((int)p_cur, k);              // wave-uniform: the branch is scalar
+            if (__builtin_expect((p & kStreamLast) != 0, 0)) {
+                if (p & kStreamDummy) acc = 0.0f;                             // an empty row: its stand-in added nothing
+                const int ctl = bcast_i(i_cur.y, rs);
+                const int src = ctl & 63, dst = (ctl >> 8) & 63;
+                const float mv = NORM ? bcast_f(mr_cur, rs) : 1.0f;
+                if (src == CBM_WALK_LOAD_ONLY) {                              // a child of the root
+                    run = NORM ? acc * mv : acc;
+                } else {
+                    float a = run, ma = mu;
+                    if (src) {
+                        a = st[(src - 1) * 2 * kWave];
+                        if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
+                    }
+                    if constexpr (NORM) {
+                        const float inv_mu = 1.0f / ma;
+                        run = (jj < dv) ? fmaf(a, inv_mu, acc) * mv : (acc + a / ma) * mv;
+                    } else {
+                        run = acc + a;
+                    }
+                }
+                if (live) {
+                    float* yr = reinterpret_cast<float*>(reinterpret_cast<char*>(Y) + (int64_t)bcast_i(i_cur.x, rs) * ldy * 4 + jj4);
+                    *yr = (relu && run < 0.0f) ? 0.0f : run;                  // keeps NaN, as torch.relu does
+                }
+                mu = mv;
+                if (dst) {
+                    st[(dst - 1) * 2 * kWave] = run;
+                    if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
+                }
+                acc = 0.0f;
+                rs++;
+            }
+        }
         p_cur = p_nxt; p_nxt = p_far;
         i_cur = i_nxt; i_nxt = i_far;
         f_cur = f_nxt; mr_cur = mr_nxt;
-        xo_cur = xo_nxt; xo_nxt = x_off(p_far);
+        xr_nxt = x_row(p_far);
     }
 }
 
@@ -2212,8 +2213,9 @@ int cbm_spmm_update_subtrees_f32(const cbm_walk_stream_dev* ws, const float* m, 
     if (flags & ~CBM_UPDATE_RELU) return CBM_ERR_UNSUPPORTED;
     if (X == Y) return CBM_ERR_SHAPE;                    // rows of Y are stored while rows of X are still gathered
     if (n == 0 || d == 0) return CBM_OK;
-    if (ws->n != n || ws->n_bins < 0 || ws->n_elems < 0 || ws->n_slots < 0 || ws->n_slots > CBM_WALK_MAX_SLOTS)
-        return CBM_ERR_SHAPE;
+    if (ws->n != n || ws->n_bins < 0 || ws->n_elems < 0 || ws->n_elems % kWave != 0 || ws->n_slots < 0 ||
+        ws->n_slots > CBM_WALK_MAX_SLOTS || (int64_t)ws->n_bins * kWave > ws->n_elems)
+        return CBM_ERR_SHAPE;                            // bins are whole stretches of 64 entries
     if ((uint32_t)n > kStreamCol) return CBM_ERR_SHAPE;  // the column shares its word with two flags and the sign
     if (ws->n_bins > 0 && (!ws->gidx || !ws->ginfo || !ws->bin_goff || !aligned(ws->ginfo, 8))) return CBM_ERR_NULL;
     if ((int64_t)n * ldy * 4 > ((int64_t)1 << 46) || (int64_t)n * ldx * 4 > ((int64_t)1 << 46)) return CBM_ERR_SHAPE;

@@ -279,14 +279,19 @@ void cbm_walk_plan_free(cbm_walk_plan* p);
  * on the spot and takes its walk step without the SpMM result ever going through memory.
  *   gidx       [n_elems] uint32: the delta entries (col | sign << 31, as idx) of a bin's rows in walk order;
  *              CBM_STREAM_LAST marks a row's last entry; an empty row has one stand-in entry with
- *              CBM_STREAM_DUMMY (| LAST) whose column is the row itself and which adds nothing
+ *              CBM_STREAM_DUMMY (| LAST) whose column is the row itself and which adds nothing; every bin is
+ *              padded to a multiple of 64 entries with unmarked copies of its last entry's column (summed
+ *              into an accumulator that is never stored)
  *   ginfo      [n_elems][2] int32 { row, ctl } (ctl as in cbm_walk_plan.entries; CBM_WALK_LOAD_ONLY = a child of
  *              the root: its sum, times m[row] when normalised, is its value): for every stretch of 64 stream
  *              entries of a bin, the rows that END inside that stretch, in order, starting at the stretch's
  *              first position; positions no row landed in hold { first row of the bin, 0 }
- *   bin_goff   [n_bins + 1] offsets into gidx / ginfo: a bin is what one wavefront streams (whole subtrees,
- *              heaviest first by stream entries, small ones packed together up to about n_elems / target_bins)
- *   n_slots    most LDS slots any subtree uses;  longest_bin  stream entries of the longest bin
+ *   bin_goff   [n_bins + 1] offsets into gidx / ginfo, multiples of 64: a bin is what one wavefront streams
+ *              (whole subtrees, heaviest first, small ones packed together up to about 1 / target_bins of
+ *              the total weight)
+ *   n_slots    most LDS slots any subtree uses;  heaviest_bin  weight of the heaviest bin, a row weighing its
+ *              stream entries + CBM_STREAM_ROW_COST (what the time of the wavefront that walks it follows; bins
+ *              are packed by this weight)
  * n must be below 2^29 (the column shares its word with the sign and the two marks).  HOST pointers; release
  * with cbm_walk_stream_free.  CBM_ERR_UNSUPPORTED as for cbm_walk_plan_build.  No reference counterpart: the
  * reference keeps the SpMM (MKL) and the walk apart (cbm_extensions.cpp:1133-1218). */
@@ -294,9 +299,10 @@ void cbm_walk_plan_free(cbm_walk_plan* p);
 #define CBM_STREAM_DUMMY 0x20000000u
 #define CBM_STREAM_COL_MASK 0x1fffffffu
 #define CBM_STREAM_MIN_BIN 64
+#define CBM_STREAM_ROW_COST 5
 typedef struct cbm_walk_stream {
     int32_t n, n_bins, n_slots, n_elems;
-    int64_t longest_bin;
+    int64_t heaviest_bin;
     uint32_t* gidx;
     int32_t* ginfo;
     int32_t* bin_goff;

@@ -727,12 +727,12 @@ def test_stream_multiply_against_oracle(orc, kind, normalized):
     if kind == "bipartite" and not normalized:
         assert int((lens == 0).sum()) >= 400
     if kind == "chain":
-        assert plan["longest_bin"] > 2000 and int(lens.max()) > 64      # many stretches; rows that span stretches
+        assert plan["heaviest_bin"] > 2000 and int(lens.max()) > 64     # many stretches; rows that span stretches
     if kind in ("bushy", "duplication"):
         assert plan["n_slots"] >= 2
     for d in (1, 19, 41, 64, 100, 128, 258, 1100):
         say("stream multiply", kind, normalized, "d", d, "levels", mat.n_levels, "bins", plan["n_bins"], "slots", plan["n_slots"],
-            "longest bin", plan["longest_bin"])
+            "heaviest bin", plan["heaviest_bin"])
         assert takes_stream(mat, d)
         x = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
         got = gpu_product(mat, x, normalized)

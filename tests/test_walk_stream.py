@@ -48,21 +48,30 @@ def interpret(plan, x):
 
 def check_stream_shape(mat, plan):
     """What the layout promises: every row exactly once, its entries the row's delta entries in order (one
-    stand-in for an empty row), heads = the children of the root, a row's parent is the row before it or sits
+    stand-in for an empty row), bins padded to whole stretches of 64, heads = the children of the root, a row's parent is the row before it or sits
     in the slot named, bins hold whole subtrees, every slot of ``ginfo`` names a valid row."""
     gidx, ginfo, goff = plan["gidx"].numpy().view(np.uint32), plan["ginfo"].numpy(), plan["bin_goff"].numpy()
     rp, idx, parent = mat.rowptr.numpy(), mat.idx.numpy().view(np.uint32), mat.parent.numpy()
     n = mat.num_rows
     lens = np.diff(rp)
-    assert plan["n_elems"] == int(np.maximum(lens, 1).sum()) == gidx.size == ginfo.shape[0]
+    assert plan["n_elems"] == gidx.size == ginfo.shape[0]
+    assert 0 <= gidx.size - int(np.maximum(lens, 1).sum()) < 64 * plan["n_bins"]          # the padding of the bins
     assert goff[0] == 0 and goff[-1] == gidx.size and (np.diff(goff) > 0).all() and goff.size == plan["n_bins"] + 1
-    assert int(np.diff(goff).max()) == plan["longest_bin"]
+    assert (goff % 64 == 0).all()
+    # the heaviest bin: entries + CBM_STREAM_ROW_COST per row
+    rows_in = lambda b: int((gidx[goff[b]:goff[b + 1]] & LAST != 0).sum())
+    real_in = lambda b: int(goff[b + 1] - goff[b]) - pad_of(b)
+    def pad_of(b):
+        seg = gidx[goff[b]:goff[b + 1]]
+        last = int(np.flatnonzero(seg & LAST)[-1])
+        return seg.size - 1 - last
+    assert plan["heaviest_bin"] == max(real_in(b) + _lib.CBM_STREAM_ROW_COST * rows_in(b) for b in range(plan["n_bins"]))
     assert int((gidx & LAST != 0).sum()) == n
     assert ginfo[:, 0].min() >= 0 and ginfo[:, 0].max() < n
     seen = np.zeros(n, np.int32)
     for b in range(plan["n_bins"]):
         first, count = int(goff[b]), int(goff[b + 1] - goff[b])
-        prev, slot_row, cur, first_src = None, {}, [], None
+        prev, slot_row, cur, first_src, last_col = None, {}, [], None, None
         for base in range(0, count, 64):
             rs = 0
             for k in range(min(64, count - base)):
@@ -89,11 +98,12 @@ def check_stream_shape(mat, plan):
                         slot_row[dst] = row
                         assert (parent == row).sum() >= 2
                     seen[row] += 1
+                    last_col = p & COL
                     prev, cur = row, []
             # the slots of this stretch that no row landed in: the bin's first row, control word 0
             for q in range(rs, min(64, count - base)):
                 assert tuple(ginfo[first + base + q]) == (ginfo[first, 0], 0)
-        assert cur == []                                            # a bin ends with the end of a row
+        assert cur == [last_col] * len(cur) and len(cur) < 64      # after its last row only the padding
         assert first_src == LOAD_ONLY                               # and starts with a child of the root
     assert (seen == 1).all()
 
@@ -140,7 +150,7 @@ def test_stream_policy():
     assert mat.stream_plan(4096) is not None
     assert mat.stream_plan(8) is None
     mat.stream_multiply = "on"
-    assert mat.stream_plan(8) is not None and mat.stream_plan(8)["n_elems"] == int(np.maximum(np.diff(mat.rowptr.numpy()), 1).sum())
+    assert mat.stream_plan(8) is not None and mat.stream_plan(8)["n_elems"] >= int(np.maximum(np.diff(mat.rowptr.numpy()), 1).sum())
     mat.stream_multiply = "off"
     assert mat.stream_plan(4096) is None
     mat.stream_multiply = "sometimes"
