@@ -712,7 +712,7 @@ class cbm_matrix:
     _WALK_US_PER_LAUNCH = 4.0
     _WALK_US_PER_NARROW_LEVEL = 2.0
     _WALK_US_PER_CHAIN_LEVEL = 0.085
-    _WALK_US_PER_ENTRY = 0.14
+    _WALK_US_PER_ENTRY = 0.125
     _WALK_BYTES_PER_US = 4.0e6
 
     def _level_plan_cost_us(self, d, first_level=1, last_level=None):

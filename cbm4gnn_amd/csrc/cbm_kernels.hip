@@ -1085,9 +1085,11 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
     const int bin = w / slices;                                                                // known to be
     if (bin >= n_bins) return;
-    const int j = (w % slices) * kWave + lane;                    // feature column of this thread
+    const int j0 = (w % slices) * kWave;                          // first feature column of this wavefront
+    const int j = j0 + lane;                                      // feature column of this thread
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d load column 0 and store nothing
+    const bool all_body = j0 + kWave <= dv;     // wave-uniform: no column of the division tail in this wavefront
     float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
     const int first = __builtin_amdgcn_readfirstlane(bin_off[bin]);
     const int count = __builtin_amdgcn_readfirstlane(bin_off[bin + 1]) - first;
@@ -1096,18 +1098,28 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
         const int2 e = entries[first + min(base + lane, count - 1)];
         return base + lane < count ? e : e0;
     };
-    auto row_of = [&](int64_t off_ids, int k) -> char* {          // off_ids: byte offsets row * ldy * 4, one per lane
-        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)off_ids, k);
-        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)((uint64_t)off_ids >> 32), k);
-        return reinterpret_cast<char*>(Y) + (int64_t)(((uint64_t)hi << 32) | lo);
+    typedef __attribute__((address_space(1))) char* global_bytes;      // device memory, not a flat address
+    typedef __attribute__((address_space(1))) float* global_float;
+    // what lane l keeps for entry l of a stretch: the address of its row of Y (wave-uniform once broadcast: a
+    // load or store then has a scalar base and the lane's column offset)
+    auto row_addr = [&](int row) -> uint64_t {
+        return (uint64_t)reinterpret_cast<uintptr_t>(Y) + (uint64_t)(uint32_t)row * (uint64_t)ldy * 4u;
     };
     const uint32_t jj4 = (uint32_t)jj * 4u;
-    auto request = [&](float (&z)[kChainHalf], int64_t off_ids, int half) {
-#pragma unroll
-        for (int u = 0; u < kChainHalf; u++) z[u] = *reinterpret_cast<const float*>(row_of(off_ids, half * kChainHalf + u) + jj4);
+    auto row_of = [&](uint64_t addr_ids, int k) -> global_float {
+        const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)addr_ids, k);
+        const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)(addr_ids >> 32), k);
+        return (global_float)((global_bytes)(uintptr_t)(((uint64_t)hi << 32) | lo) + jj4);
     };
-    float run = 0.0f, mu = 1.0f;
-    auto consume = [&](auto full, const float (&z)[kChainHalf], int64_t off_ids, int c_ids, float m_ids, int base, int half) {
+    auto request = [&](float (&z)[kChainHalf], uint64_t addr_ids, int half) {
+#pragma unroll
+        for (int u = 0; u < kChainHalf; u++) z[u] = *row_of(addr_ids, half * kChainHalf + u);
+    };
+    // mu, inv_mu: m of the row just finished and 1 / it (the reference divides once per row, cpp:1329-1354:
+    // here lane l does that division for the l-th row of a stretch, all 64 at once)
+    float run = 0.0f, mu = 1.0f, inv_mu = 1.0f;
+    auto consume = [&](auto full, const float (&z)[kChainHalf], uint64_t addr_ids, int c_ids, float m_ids, float im_ids, int base,
+                       int half) {
 #pragma unroll
         for (int u = 0; u < kChainHalf; u++) {
             const int k = half * kChainHalf + u;
@@ -1118,20 +1130,21 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
                 if (src == CBM_WALK_LOAD_ONLY) {
                     run = z[u];
                 } else {
-                    float a = run, ma = mu;
+                    float a = run, ma = mu, inv = inv_mu;
                     if (src) {
                         a = st[(src - 1) * 2 * kWave];
-                        if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
+                        if constexpr (NORM) { ma = st[(src - 1) * 2 * kWave + kWave]; inv = 1.0f / ma; }
                     }
                     if constexpr (NORM) {
-                        const float inv_mu = 1.0f / ma;
-                        run = (jj < dv) ? fmaf(a, inv_mu, z[u]) * mv : (z[u] + a / ma) * mv;
+                        if (all_body) run = fmaf(a, inv, z[u]) * mv;
+                        else run = (jj < dv) ? fmaf(a, inv, z[u]) * mv : (z[u] + a / ma) * mv;
                     } else {
                         run = z[u] + a;
                     }
-                    if (live) *reinterpret_cast<float*>(row_of(off_ids, k) + jj4) = run;
+                    if (live) *row_of(addr_ids, k) = run;
                 }
                 mu = mv;
+                if constexpr (NORM) inv_mu = bcast_f(im_ids, k);
                 if (dst) {
                     st[(dst - 1) * 2 * kWave] = run;
                     if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
@@ -1140,28 +1153,29 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
         }
     };
     int2 e_cur = ids(0), e_nxt = ids(kWave);
-    int64_t o_cur = (int64_t)e_cur.x * ldy * 4, o_nxt = (int64_t)e_nxt.x * ldy * 4;
-    float m_cur = 1.0f;
-    if constexpr (NORM) m_cur = m[e_cur.x];
+    uint64_t a_cur = row_addr(e_cur.x), a_nxt = row_addr(e_nxt.x);
+    float m_cur = 1.0f, im_cur = 1.0f;
+    if constexpr (NORM) { m_cur = m[e_cur.x]; im_cur = 1.0f / m_cur; }
     float za[kChainHalf], zb[kChainHalf];
-    request(za, o_cur, 0);
+    request(za, a_cur, 0);
     for (int base = 0; base < count; base += kWave) {
         const int2 e_far = ids(base + 2 * kWave);
         float m_nxt = 1.0f;
         if constexpr (NORM) m_nxt = m[e_nxt.x];
-        request(zb, o_cur, 1);
+        request(zb, a_cur, 1);
         if (base + kWave <= count) {
-            consume(std::true_type{}, za, o_cur, e_cur.y, m_cur, base, 0);
-            request(za, o_nxt, 0);
-            consume(std::true_type{}, zb, o_cur, e_cur.y, m_cur, base, 1);
+            consume(std::true_type{}, za, a_cur, e_cur.y, m_cur, im_cur, base, 0);
+            request(za, a_nxt, 0);
+            consume(std::true_type{}, zb, a_cur, e_cur.y, m_cur, im_cur, base, 1);
         } else {
-            consume(std::false_type{}, za, o_cur, e_cur.y, m_cur, base, 0);
-            request(za, o_nxt, 0);
-            consume(std::false_type{}, zb, o_cur, e_cur.y, m_cur, base, 1);
+            consume(std::false_type{}, za, a_cur, e_cur.y, m_cur, im_cur, base, 0);
+            request(za, a_nxt, 0);
+            consume(std::false_type{}, zb, a_cur, e_cur.y, m_cur, im_cur, base, 1);
         }
         e_cur = e_nxt; e_nxt = e_far;
-        o_cur = o_nxt; m_cur = m_nxt;
-        o_nxt = (int64_t)e_far.x * ldy * 4;
+        a_cur = a_nxt; m_cur = m_nxt;
+        if constexpr (NORM) im_cur = 1.0f / m_cur;
+        a_nxt = row_addr(e_far.x);
     }
 }
 
@@ -1191,9 +1205,11 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
     const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
     const int bin = w / slices;                                                                // known to be
     if (bin >= n_bins) return;
-    const int j = (w % slices) * kWave + lane;                    // feature column of this thread
+    const int j0 = (w % slices) * kWave;                          // first feature column of this wavefront
+    const int j = j0 + lane;                                      // feature column of this thread
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d gather column 0 and store nothing
+    const bool all_body = j0 + kWave <= dv;     // wave-uniform: no column of the division tail in this wavefront
     float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
     const int first = __builtin_amdgcn_readfirstlane(bin_goff[bin]);
     const int count = __builtin_amdgcn_readfirstlane(bin_goff[bin + 1]) - first;       // a multiple of 64
@@ -1217,11 +1233,13 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
         const global_bytes row = (global_bytes)(uintptr_t)(((uint64_t)hi << 32) | lo);
         return *(global_float)(row + jj4);
     };
-    float acc = 0.0f, run = 0.0f, mu = 1.0f;
+    // mu, inv_mu: m of the row just finished and 1 / it (the reference divides once per row, cpp:1329-1354:
+    // here lane l does that division for the l-th row of a stretch, all 64 at once)
+    float acc = 0.0f, run = 0.0f, mu = 1.0f, inv_mu = 1.0f;
     uint32_t p_cur = gidx[at(0)], p_nxt = gidx[at(kWave)];
     int2 i_cur = ginfo[at(0)], i_nxt = ginfo[at(kWave)];
-    float f_cur = coef(p_cur), mr_cur = 1.0f;
-    if constexpr (NORM) mr_cur = m[i_cur.x];
+    float f_cur = coef(p_cur), mr_cur = 1.0f, ir_cur = 1.0f;
+    if constexpr (NORM) { mr_cur = m[i_cur.x]; ir_cur = 1.0f / mr_cur; }
     uint64_t xr_cur = x_row(p_cur), xr_nxt = x_row(p_nxt);
     float z[kWave];
 #pragma unroll
@@ -1234,6 +1252,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
         const float f_nxt = coef(p_nxt);
         float mr_nxt = 1.0f;
         if constexpr (NORM) mr_nxt = m[i_nxt.x];
+        uint64_t yr_cur = (uint64_t)reinterpret_cast<uintptr_t>(Y) + (uint64_t)(uint32_t)i_cur.x * (uint64_t)ldy * 4u;
         int rs = 0;                                               // rows finished in this stretch (wave-uniform)
 #pragma unroll
         for (int k = 0; k < kWave; k++) {
@@ -1249,23 +1268,28 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
                 if (src == CBM_WALK_LOAD_ONLY) {                              // a child of the root
                     run = NORM ? acc * mv : acc;
                 } else {
-                    float a = run, ma = mu;
+                    float a = run, ma = mu, inv = inv_mu;
                     if (src) {
                         a = st[(src - 1) * 2 * kWave];
-                        if constexpr (NORM) ma = st[(src - 1) * 2 * kWave + kWave];
+                        if constexpr (NORM) { ma = st[(src - 1) * 2 * kWave + kWave]; inv = 1.0f / ma; }
                     }
                     if constexpr (NORM) {
-                        const float inv_mu = 1.0f / ma;
-                        run = (jj < dv) ? fmaf(a, inv_mu, acc) * mv : (acc + a / ma) * mv;
+                        if (all_body) run = fmaf(a, inv, acc) * mv;
+                        else run = (jj < dv) ? fmaf(a, inv, acc) * mv : (acc + a / ma) * mv;
                     } else {
                         run = acc + a;
                     }
                 }
                 if (live) {
-                    float* yr = reinterpret_cast<float*>(reinterpret_cast<char*>(Y) + (int64_t)bcast_i(i_cur.x, rs) * ldy * 4 + jj4);
-                    *yr = (relu && run < 0.0f) ? 0.0f : run;                  // keeps NaN, as torch.relu does
+                    const uint32_t lo = (uint32_t)bcast_i((int)(uint32_t)yr_cur, rs);
+                    const uint32_t hi = (uint32_t)bcast_i((int)(uint32_t)(yr_cur >> 32), rs);
+                    typedef __attribute__((address_space(1))) char* global_bytes_out;
+                    typedef __attribute__((address_space(1))) float* global_float_out;
+                    const global_bytes_out row = (global_bytes_out)(uintptr_t)(((uint64_t)hi << 32) | lo);
+                    *(global_float_out)(row + jj4) = (relu && run < 0.0f) ? 0.0f : run;   // keeps NaN, as torch.relu does
                 }
                 mu = mv;
+                if constexpr (NORM) inv_mu = bcast_f(ir_cur, rs);
                 if (dst) {
                     st[(dst - 1) * 2 * kWave] = run;
                     if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
@@ -1277,6 +1301,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
         p_cur = p_nxt; p_nxt = p_far;
         i_cur = i_nxt; i_nxt = i_far;
         f_cur = f_nxt; mr_cur = mr_nxt;
+        if constexpr (NORM) ir_cur = 1.0f / mr_cur;
         xr_nxt = x_row(p_far);
     }
 }
