@@ -192,3 +192,58 @@ def test_stream_build_rejects_bad_input():
     assert build(order=bad) != 0
     assert build(bins=0) != 0
     assert build(n=0) != 0
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_trees_and_random_delta_rows(seed):
+    """Arrays no builder made: a random recursive tree (bushy or nearly a chain), delta rows of 0 .. 200 random
+    signed entries (rows that span several stretches, runs of empty rows), every bin target from one bin to one
+    subtree per bin -- the layout must hold and the interpreted stream must equal the sum down every row's
+    ancestor path computed directly."""
+    import types
+
+    from cbm4gnn_amd.cbm import tree_levels
+    rng = np.random.default_rng(seed)
+    n = int(rng.choice([1, 2, 63, 64, 65, 500, 1500]))
+    roots = int(rng.integers(1, max(2, n // 4) + 1))
+    par = np.full(n, -1, np.int64)
+    stretch = float(rng.choice([0.0, 0.9, 0.995]))                   # how much a row prefers the row just before it
+    for v in range(roots, n):
+        par[v] = v - 1 if rng.random() < stretch else int(rng.integers(0, v))
+    kids = [[] for _ in range(n + 1)]
+    for v in range(n):
+        kids[n if par[v] < 0 else par[v]].append(v)
+    mst_col = np.array(sum(kids, []), np.int32)
+    mst_row = np.concatenate([[0], np.cumsum([len(k) for k in kids])]).astype(np.int32)
+    parent, order, level_off = tree_levels(mst_row, mst_col)
+    lens = rng.choice([0, 0, 1, 2, 3, 7, 64, 70, 200], size=n, p=[.15, .1, .2, .2, .15, .1, .04, .04, .02])
+    lens = np.minimum(lens, n)
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens] + [np.empty(0, np.int64)]).astype(np.uint32)
+    idx = (cols | (rng.integers(0, 2, size=cols.size).astype(np.uint32) << 31)).astype(np.uint32)
+    x = rng.integers(-8, 9, size=(n, 2)).astype(np.float64)
+    # the product directly: a row's own signed sum plus its parent's value, parents first
+    want = np.zeros((n, 2))
+    for v in order:
+        e = idx[rowptr[v]:rowptr[v + 1]]
+        own = (np.where(e >> 31, -1.0, 1.0)[:, None] * x[e & COL]).sum(0) if e.size else 0.0
+        want[v] = own + (want[parent[v]] if parent[v] >= 0 else 0.0)
+    mat = types.SimpleNamespace(rowptr=torch.from_numpy(rowptr), idx=torch.from_numpy(idx.view(np.int32)),
+                                parent=torch.from_numpy(np.asarray(parent, np.int32)), num_rows=n)
+    for bins in (1, 7, 100_000):
+        p = _lib.CbmWalkStream()
+        a = [np.ascontiguousarray(t, np.int32) for t in (parent, order, level_off)]
+        rc = _lib.host_lib().cbm_walk_stream_build(rowptr.ctypes.data, idx.ctypes.data, a[0].ctypes.data, a[1].ctypes.data,
+                                                   a[2].ctypes.data, n, len(level_off) - 1, bins, C.byref(p))
+        assert rc == 0
+        try:
+            take = lambda ptr, count: torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(count,)).astype(np.int32, copy=True))
+            plan = {"n_bins": int(p.n_bins), "n_slots": int(p.n_slots), "n_elems": int(p.n_elems), "heaviest_bin": int(p.heaviest_bin),
+                    "gidx": take(p.gidx, p.n_elems), "ginfo": take(p.ginfo, 2 * p.n_elems).view(-1, 2),
+                    "bin_goff": take(p.bin_goff, p.n_bins + 1)}
+        finally:
+            _lib.host_lib().cbm_walk_stream_free(C.byref(p))
+        assert plan["n_bins"] == 1 if bins == 1 else plan["n_bins"] >= 1
+        check_stream_shape(mat, plan)
+        y, written = interpret(plan, x)
+        assert (written == 1).all() and np.array_equal(y, want)
