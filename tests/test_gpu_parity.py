@@ -757,6 +757,64 @@ def test_stream_multiply_against_oracle(orc, kind, normalized):
         assert np.array_equal(gpu_product(mat, xi, False), got)
 
 
+def test_stream_multiply_on_hand_made_trees(orc):
+    """Trees the builder rarely produces and delta rows no builder made, through the C ABI alone
+    (cbm_walk_stream_build + cbm_spmm_update_subtrees_f32): a complete binary tree (a slot per level of the path),
+    a random recursive tree and a caterpillar, rows of 0 .. 200 random signed entries -- against the oracle's
+    in-order SpMM followed by its walk, bit for bit, plain and normalised."""
+    from cbm4gnn_amd.cbm import tree_levels
+    lib, host = _lib.hip_lib(), _lib.host_lib()
+    rng = np.random.default_rng(11)
+    trees = {}
+    n = 2047
+    trees["binary"] = np.concatenate([[-1], (np.arange(1, n) - 1) // 2])
+    n = 5000
+    par = np.full(n, -1, np.int64)
+    par[40:] = (rng.random(n - 40) * np.arange(40, n)).astype(np.int64)
+    trees["recursive"] = par
+    n = 1201
+    par = np.full(n, -1, np.int64)
+    par[1:601] = np.arange(0, 600)
+    par[601:] = np.arange(0, 600)
+    trees["caterpillar"] = par
+    p = lambda t: C.c_void_p(t.data_ptr())
+    for name, par in trees.items():
+        n = par.shape[0]
+        kids = [[] for _ in range(n + 1)]
+        for v in range(n):
+            kids[n if par[v] < 0 else par[v]].append(v)
+        mst_col = np.array(sum(kids, []), np.int32)
+        mst_row = np.concatenate([[0], np.cumsum([len(k) for k in kids])]).astype(np.int32)
+        parent, order, level_off = (torch.from_numpy(a) for a in tree_levels(mst_row, mst_col))
+        levels = level_off.numel() - 1
+        lens = rng.choice([0, 1, 2, 3, 7, 64, 70, 200], size=n, p=[.2, .2, .2, .15, .15, .04, .04, .02])
+        rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        cols = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+        sign = np.where(rng.integers(0, 2, size=cols.size) == 1, -1.0, 1.0).astype(np.float32)
+        idx = (cols.astype(np.uint32) | ((sign < 0).astype(np.uint32) << 31)).astype(np.uint32)
+        m = (rng.random(n).astype(np.float32) + 0.5)
+        plan = _lib.CbmWalkStream()
+        rp_t, idx_t = torch.from_numpy(rowptr), torch.from_numpy(idx.view(np.int32))
+        assert host.cbm_walk_stream_build(p(rp_t), p(idx_t), p(parent), p(order), p(level_off), n, levels, 256, C.byref(plan)) == 0
+        gidx = torch.from_numpy(np.ctypeslib.as_array(plan.gidx, shape=(plan.n_elems,)).astype(np.int32)).cuda()
+        ginfo = torch.from_numpy(np.ctypeslib.as_array(plan.ginfo, shape=(2 * plan.n_elems,)).copy()).cuda()
+        goff = torch.from_numpy(np.ctypeslib.as_array(plan.bin_goff, shape=(plan.n_bins + 1,)).copy()).cuda()
+        ws = _lib.CbmWalkStreamDev(n, plan.n_bins, plan.n_slots, plan.n_elems, gidx.data_ptr(), ginfo.data_ptr(), goff.data_ptr())
+        say("hand-made tree, stream", name, "levels", levels, "slots", plan.n_slots, "bins", plan.n_bins, "entries", plan.n_elems)
+        if name == "binary":
+            assert plan.n_slots >= levels - 2
+        host.cbm_walk_stream_free(C.byref(plan))
+        for d, norm in ((72, True), (130, False), (41, True)):
+            x = rng.standard_normal((n, d)).astype(np.float32)
+            val = sign * m[cols] if norm else sign
+            z = orc.csr_spmm(rowptr, cols, val.astype(np.float32), x)                 # strictly in entry order
+            want = orc.update_fused(mst_row, mst_col, m, z) if norm else orc.update_plain(mst_row, mst_col, z)
+            xd, y = torch.from_numpy(x).cuda(), torch.full((n, d), float("nan"), device="cuda")
+            md = torch.from_numpy(m).cuda() if norm else None
+            assert lib.cbm_spmm_update_subtrees_f32(C.byref(ws), p(md) if norm else None, p(xd), p(y), n, d, d, d, 0, None) == 0
+            assert np.array_equal(y.cpu().numpy(), want), (name, d, norm)
+
+
 def test_stream_multiply_status_codes():
     lib = _lib.hip_lib()
     ei = graphs.add_self_loops(graphs.staircases(8, 20, 6, 2.0, seed=4))
