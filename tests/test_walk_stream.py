@@ -48,8 +48,9 @@ def interpret(plan, x):
 
 def check_stream_shape(mat, plan):
     """What the layout promises: every row exactly once, its entries the row's delta entries in order (one
-    stand-in for an empty row), bins padded to whole stretches of 64, heads = the children of the root, a row's parent is the row before it or sits
-    in the slot named, bins hold whole subtrees, every slot of ``ginfo`` names a valid row."""
+    stand-in for an empty row), bins padded to whole stretches of 64, heads = the children of the root, a row's
+    parent is the row before it or sits in the slot named, bins hold whole subtrees, every slot of ``ginfo`` names
+    a valid row."""
     gidx, ginfo, goff = plan["gidx"].numpy().view(np.uint32), plan["ginfo"].numpy(), plan["bin_goff"].numpy()
     rp, idx, parent = mat.rowptr.numpy(), mat.idx.numpy().view(np.uint32), mat.parent.numpy()
     n = mat.num_rows
