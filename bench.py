@@ -767,9 +767,10 @@ def main():
         short = argparse.Namespace(**{**vars(args), "steps": min(args.steps, 20), "warmup": min(args.warmup, 3)})
         # (workload, alpha, seconds of CPU legs or None): the CPU legs run where the tree exists -- on the
         # headline graph at alpha = 0, on both readings of the duplication graph, on the dense-community graph
-        # and on the deep-and-wide tree -- so that the reference's OpenMP walk is timed where it walks
+        # on the deep-and-wide tree and on the union of cliques -- so that the reference's OpenMP walk is timed
+        # where it walks
         plan = (("c3", 0, 10.0), ("c1", 0, 4.0), ("c2", 0, 8.0), ("c2", 8, None), ("c2b", 0, 6.0),
-                ("c5", 0, 40.0), ("c6", 0, 12.0))
+                ("c5", 0, 40.0), ("c6", 0, 12.0), ("c7", 0, 8.0))
         wk = None
         for name, a, cpu_s in plan:
             if wk is None or wk.name != name:

@@ -1090,6 +1090,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d load column 0 and store nothing
     const bool all_body = j0 + kWave <= dv;     // wave-uniform: no column of the division tail in this wavefront
+    const bool all_live = j0 + kWave <= d;      // wave-uniform: every lane stores
     float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
     const int first = __builtin_amdgcn_readfirstlane(bin_off[bin]);
     const int count = __builtin_amdgcn_readfirstlane(bin_off[bin + 1]) - first;
@@ -1120,6 +1121,26 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     float run = 0.0f, mu = 1.0f, inv_mu = 1.0f;
     auto consume = [&](auto full, const float (&z)[kChainHalf], uint64_t addr_ids, int c_ids, float m_ids, float im_ids, int base,
                        int half) {
+        // A half stretch of plain chain steps (every control word 0: the parent is the row before, nothing to
+        // keep) in a wavefront without tail columns or idle lanes: no test per row.  Past the end of the bin the
+        // control words are those of the bin's head (never 0), so a partial stretch never comes here.
+        const uint64_t not_plain = __builtin_amdgcn_ballot_w64(c_ids != 0);
+        if (((not_plain >> (half * kChainHalf)) & 0xffffffffull) == 0 && all_live && (!NORM || all_body)) {
+#pragma unroll
+            for (int u = 0; u < kChainHalf; u++) {
+                const int k = half * kChainHalf + u;
+                if constexpr (NORM) {
+                    const float mv = bcast_f(m_ids, k);
+                    run = fmaf(run, inv_mu, z[u]) * mv;
+                    mu = mv;
+                    inv_mu = bcast_f(im_ids, k);
+                } else {
+                    run = z[u] + run;
+                }
+                *row_of(addr_ids, k) = run;
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < kChainHalf; u++) {
             const int k = half * kChainHalf + u;

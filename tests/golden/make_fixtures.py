@@ -48,7 +48,7 @@ def main():
             cases[f"case{seed}_{k}"] = v
     np.savez_compressed(os.path.join(HERE, "er_products.npz"), **cases)
     hashes = {}
-    for name in ("c1", "c2", "c2b", "c3", "c6"):
+    for name in ("c1", "c2", "c2b", "c3", "c6", "c7"):
         w = graphs.workload(name)
         hashes[name] = {"n": int(w.n), "edges": int(w.edge_index.shape[1]), "sha256": graphs.edge_hash(w.edge_index)}
     with open(os.path.join(HERE, "graph_hashes.json"), "w") as f:

@@ -166,7 +166,7 @@ def test_graph_generators_are_pinned():
     import json, os
     with open(os.path.join(os.path.dirname(__file__), "golden", "graph_hashes.json")) as f:
         want = json.load(f)
-    for name in ("c1", "c2", "c2b", "c3", "c6"):
+    for name in ("c1", "c2", "c2b", "c3", "c6", "c7"):
         w = graphs.workload(name)
         assert w.edge_index.shape[1] == want[name]["edges"] and w.n == want[name]["n"]
         assert graphs.edge_hash(w.edge_index) == want[name]["sha256"], name

@@ -347,6 +347,45 @@ def test_deep_and_wide_tree_full_size():
     assert float((unbatched - got).abs().max() / got.abs().max()) <= 1e-5
 
 
+def test_union_of_cliques_full_size():
+    """c7: 150,000 rows in 12,000 overlapping cliques (the co-authorship shape), compression ~5.8, 43 tree levels:
+    1,024 rows against fp64 SciPy rows and the whole product against the GPU CSR baseline at d = 128 (SpMM + walk
+    by the automatic choice) and d = 256 (the one-launch multiply by the automatic choice); the two paths against
+    each other, and a depth limit of 8 levels against the same anchors."""
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    w = graphs.workload("c7")
+    print("[gpu-case] c7 full size, building", flush=True); sys.stdout.flush()
+    mat = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=0, normalized=True)
+    assert mat.compression_ratio() > 5 and mat.n_levels > 30
+    rp, col = _csr(w.edge_index, w.n)
+    m = mat.col_multiplier.numpy()
+    val = torch.from_numpy((np.repeat(m, np.diff(rp)) * m[col]).astype(np.float32)).cuda()
+    rp_d, col_d = torch.from_numpy(rp.astype(np.int32)).cuda(), torch.from_numpy(col).cuda()
+    rows = np.sort(np.random.default_rng(7).choice(w.n, size=1024, replace=False))
+    rows_d = torch.from_numpy(rows).cuda()
+    shallow = cbm_matrix(torch.from_numpy(w.edge_index), None, alpha=0, normalized=True, max_levels=8)
+    assert shallow.n_levels == 8 and 2 < shallow.compression_ratio() < mat.compression_ratio()
+    for d, one_launch in ((128, False), (256, True)):
+        print("[gpu-case] c7 full size, d", d, flush=True); sys.stdout.flush()
+        x = w.features(0, d)
+        xd = x.cuda()
+        assert (mat.stream_plan(d) is not None) == one_launch
+        got = _mul(mat, xd)
+        want_rows = _rows_fp64(rp, col, m, x.numpy(), rows)
+        _assert_rows_close(got[rows_d].cpu().numpy().astype(np.float64), want_rows)
+        base = torch.empty_like(xd)
+        csr_spmm(rp_d, col_d, val, xd, base)
+        assert float((got - base).abs().max() / base.abs().max()) <= 1e-3
+        mat.stream_multiply = "off" if one_launch else "on"          # the other path: another summation order
+        other = _mul(mat, xd)
+        mat.stream_multiply = "auto"
+        assert float((other - got).abs().max() / got.abs().max()) <= 1e-5
+        lim = _mul(shallow, xd)
+        _assert_rows_close(lim[rows_d].cpu().numpy().astype(np.float64), want_rows)
+        assert float((lim - base).abs().max() / base.abs().max()) <= 1e-3
+
+
 def test_alpha_sweep_graph_same_format_for_every_alpha():
     """On the dense-community graph alpha <= 32 prunes nothing (every admissible pair clears the
     threshold by far more): the builder must return the arrays of alpha = 0 for the whole sweep."""
