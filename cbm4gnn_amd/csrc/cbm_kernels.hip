@@ -1066,8 +1066,8 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
 // The walk of all subtrees below a level in ONE launch (plan: cbm_walk_plan_build).  A wavefront takes a bin
 // of the plan -- whole subtrees, each a sequence of rows in depth-first pre-order -- and 64 feature columns
 // (one per lane), and carries the value of the row it has just finished in a register: the next row of the
-// sequence is usually that row's first child.  A row with two or more children also leaves its value (and
-// its m) in an LDS slot of the wavefront, where the later children find it; children are ordered lightest
+// sequence is usually that row's first child.  A row with two or more children also leaves its value (with
+// its m and 1 / m) in an LDS slot of the wavefront, where the later children find it; children are ordered lightest
 // subtree first, so few slots are live at once.  Global memory is touched twice per row -- its SpMM result is
 // read, its final value written -- and no load depends on an earlier store, so, as in propagate_chain, the
 // rows of a stretch of 64 entries are requested half a stretch ahead and every load is unconditional (past
@@ -1075,12 +1075,13 @@ __global__ __launch_bounds__(kWave * kNarrowWaves) void propagate_chain(
 // root after the SpMM, or a row of a level walked before this launch): it is loaded, not stored.
 // Arithmetic per row is exactly that of propagate_row, so Y is bit-identical to the level-by-level walk.
 constexpr int kSubWaves = 4;               // wavefronts per workgroup (each owns its LDS slots)
+constexpr int kSlotFloats = 3 * kWave;     // a slot: a row's value, its m and 1 / m, per feature column of the wavefront
 
 template <bool NORM>
 __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     const int2* __restrict__ entries, const int32_t* __restrict__ bin_off, int n_bins, int slices,
     const float* __restrict__ m, float* __restrict__ Y, int d, int dv, int64_t ldy, int n_slots) {
-    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
+    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][3][64]
     const int lane = threadIdx.x & (kWave - 1);
     const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
     const int bin = w / slices;                                                                // known to be
@@ -1091,7 +1092,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
     const int jj = live ? j : 0;                                  // lanes past d load column 0 and store nothing
     const bool all_body = j0 + kWave <= dv;     // wave-uniform: no column of the division tail in this wavefront
     const bool all_live = j0 + kWave <= d;      // wave-uniform: every lane stores
-    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
+    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * kSlotFloats + lane;
     const int first = __builtin_amdgcn_readfirstlane(bin_off[bin]);
     const int count = __builtin_amdgcn_readfirstlane(bin_off[bin + 1]) - first;
     const int2 e0 = entries[first];
@@ -1153,8 +1154,8 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
                 } else {
                     float a = run, ma = mu, inv = inv_mu;
                     if (src) {
-                        a = st[(src - 1) * 2 * kWave];
-                        if constexpr (NORM) { ma = st[(src - 1) * 2 * kWave + kWave]; inv = 1.0f / ma; }
+                        a = st[(src - 1) * kSlotFloats];
+                        if constexpr (NORM) { ma = st[(src - 1) * kSlotFloats + kWave]; inv = st[(src - 1) * kSlotFloats + 2 * kWave]; }
                     }
                     if constexpr (NORM) {
                         if (all_body) run = fmaf(a, inv, z[u]) * mv;
@@ -1167,8 +1168,8 @@ __global__ __launch_bounds__(kWave * kSubWaves) void propagate_subtrees(
                 mu = mv;
                 if constexpr (NORM) inv_mu = bcast_f(im_ids, k);
                 if (dst) {
-                    st[(dst - 1) * 2 * kWave] = run;
-                    if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
+                    st[(dst - 1) * kSlotFloats] = run;
+                    if constexpr (NORM) { st[(dst - 1) * kSlotFloats + kWave] = mv; st[(dst - 1) * kSlotFloats + 2 * kWave] = bcast_f(im_ids, k); }
                 }
             }
         }
@@ -1221,7 +1222,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
     const uint32_t* __restrict__ gidx, const int2* __restrict__ ginfo, const int32_t* __restrict__ bin_goff, int n_bins,
     int slices, const float* __restrict__ m, const float* __restrict__ X, float* __restrict__ Y, int d, int dv, int64_t ldx,
     int64_t ldy, int n_slots, int relu) {
-    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][2][64]
+    extern __shared__ float walk_slots[];                         // [kSubWaves][n_slots][3][64]
     const int lane = threadIdx.x & (kWave - 1);
     const int w = blockIdx.x * kSubWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, and
     const int bin = w / slices;                                                                // known to be
@@ -1231,7 +1232,7 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
     const bool live = j < d;
     const int jj = live ? j : 0;                                  // lanes past d gather column 0 and store nothing
     const bool all_body = j0 + kWave <= dv;     // wave-uniform: no column of the division tail in this wavefront
-    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * 2 * kWave + lane;
+    float* __restrict__ st = walk_slots + (size_t)(threadIdx.x >> 6) * n_slots * kSlotFloats + lane;
     const int first = __builtin_amdgcn_readfirstlane(bin_goff[bin]);
     const int count = __builtin_amdgcn_readfirstlane(bin_goff[bin + 1]) - first;       // a multiple of 64
     auto at = [&](int base) -> int { return first + min(base, count - kWave) + lane; };   // past the end: the last stretch
@@ -1291,8 +1292,8 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
                 } else {
                     float a = run, ma = mu, inv = inv_mu;
                     if (src) {
-                        a = st[(src - 1) * 2 * kWave];
-                        if constexpr (NORM) { ma = st[(src - 1) * 2 * kWave + kWave]; inv = 1.0f / ma; }
+                        a = st[(src - 1) * kSlotFloats];
+                        if constexpr (NORM) { ma = st[(src - 1) * kSlotFloats + kWave]; inv = st[(src - 1) * kSlotFloats + 2 * kWave]; }
                     }
                     if constexpr (NORM) {
                         if (all_body) run = fmaf(a, inv, acc) * mv;
@@ -1312,8 +1313,8 @@ __global__ __launch_bounds__(kWave * kSubWaves) void spmm_update_subtrees(
                 mu = mv;
                 if constexpr (NORM) inv_mu = bcast_f(ir_cur, rs);
                 if (dst) {
-                    st[(dst - 1) * 2 * kWave] = run;
-                    if constexpr (NORM) st[(dst - 1) * 2 * kWave + kWave] = mv;
+                    st[(dst - 1) * kSlotFloats] = run;
+                    if constexpr (NORM) { st[(dst - 1) * kSlotFloats + kWave] = mv; st[(dst - 1) * kSlotFloats + 2 * kWave] = bcast_f(ir_cur, rs); }
                 }
                 acc = 0.0f;
                 rs++;
@@ -2035,7 +2036,7 @@ int launch_subtrees(const cbm_walk_dev* w, const float* m, float* Y, int32_t d, 
     const int64_t waves = (int64_t)w->n_bins * slices;
     const int64_t blocks = (waves + kSubWaves - 1) / kSubWaves;
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
-    const size_t lds = (size_t)kSubWaves * w->n_slots * 2 * kWave * sizeof(float);       // at most 62 KB
+    const size_t lds = (size_t)kSubWaves * w->n_slots * kSlotFloats * sizeof(float);     // at most 93 KB
     hipLaunchKernelGGL((propagate_subtrees<NORM>), dim3((unsigned)blocks), dim3(kWave * kSubWaves), lds, s,
                        reinterpret_cast<const int2*>(w->entries), w->bin_off, w->n_bins, slices, m, Y, d, d - d % 8, ldy,
                        w->n_slots);
@@ -2050,7 +2051,7 @@ int launch_stream(const cbm_walk_stream_dev* w, const float* m, const float* X, 
     const int64_t waves = (int64_t)w->n_bins * slices;
     const int64_t blocks = (waves + kSubWaves - 1) / kSubWaves;
     if (blocks > INT32_MAX) return CBM_ERR_SHAPE;
-    const size_t lds = (size_t)kSubWaves * w->n_slots * 2 * kWave * sizeof(float);       // at most 62 KB
+    const size_t lds = (size_t)kSubWaves * w->n_slots * kSlotFloats * sizeof(float);     // at most 93 KB
     hipLaunchKernelGGL((spmm_update_subtrees<NORM>), dim3((unsigned)blocks), dim3(kWave * kSubWaves), lds, s, w->gidx,
                        reinterpret_cast<const int2*>(w->ginfo), w->bin_goff, w->n_bins, slices, m, X, Y, d, d - d % 8, ldx,
                        ldy, w->n_slots, relu);
